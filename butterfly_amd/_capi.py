@@ -1,0 +1,164 @@
+"""ctypes binding of the C ABI in ``include/butterfly_hip.h`` (``libbutterfly_hip.so``).
+
+Used by the parity tests and the benchmark to call the library below the operator shim,
+with raw device pointers taken from torch tensors.
+"""
+import ctypes
+import os
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libbutterfly_hip.so")
+
+BF_F32, BF_C64 = 0, 1
+
+SYMBOLS = [
+    "bf_version", "bf_hip_version", "bf_last_error",
+    "bf_butterfly_multiply_fw", "bf_butterfly_multiply_bw_workspace_bytes", "bf_butterfly_multiply_bw",
+    "bf_butterfly_multiply_base4_fw", "bf_butterfly_multiply_base4_bw_workspace_bytes",
+    "bf_butterfly_multiply_base4_bw",
+]
+
+
+class Problem(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32),
+        ("increasing_stride", ctypes.c_int32),
+        ("batch", ctypes.c_int64),
+        ("nstacks", ctypes.c_int64),
+        ("log_n", ctypes.c_int64),
+        ("nblocks", ctypes.c_int64),
+        ("input_size", ctypes.c_int64),
+        ("output_size", ctypes.c_int64),
+        ("input_stride", ctypes.c_int64 * 3),
+        ("output_stride", ctypes.c_int64 * 3),
+        ("d_input_stride", ctypes.c_int64 * 3),
+    ]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.isfile(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: run `python -m butterfly_amd.build`")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, sz = ctypes.c_void_p, ctypes.c_size_t
+        pp = ctypes.POINTER(Problem)
+        L.bf_version.restype = ctypes.c_int
+        L.bf_hip_version.restype = ctypes.c_int
+        L.bf_last_error.restype = ctypes.c_char_p
+        L.bf_butterfly_multiply_fw.argtypes = [pp, vp, vp, vp, vp]
+        L.bf_butterfly_multiply_bw_workspace_bytes.argtypes = [pp]
+        L.bf_butterfly_multiply_bw_workspace_bytes.restype = sz
+        L.bf_butterfly_multiply_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_base4_fw.argtypes = [pp, vp, vp, vp, vp, vp]
+        L.bf_butterfly_multiply_base4_bw_workspace_bytes.argtypes = [pp]
+        L.bf_butterfly_multiply_base4_bw_workspace_bytes.restype = sz
+        L.bf_butterfly_multiply_base4_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+        _lib = L
+    return _lib
+
+
+class ButterflyError(RuntimeError):
+    def __init__(self, code):
+        self.code = code
+        super().__init__(f"libbutterfly_hip error {code}: {lib().bf_last_error().decode()}")
+
+
+def _check(rc):
+    if rc != 0:
+        raise ButterflyError(rc)
+
+
+def _dtype_code(t):
+    if t.dtype == torch.float32:
+        return BF_F32
+    if t.dtype == torch.complex64:
+        return BF_C64
+    raise TypeError(f"unsupported dtype {t.dtype}")
+
+
+def _strides(t):
+    return (ctypes.c_int64 * 3)(*[t.stride(i) if t.size(i) > 1 else 0 for i in range(3)])
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else ctypes.c_void_p(0)
+
+
+def make_problem(input, log_n, nblocks, increasing_stride, output_size):
+    p = Problem()
+    p.dtype = _dtype_code(input)
+    p.increasing_stride = int(bool(increasing_stride))
+    p.batch, p.nstacks, p.input_size = input.shape
+    p.log_n, p.nblocks = log_n, nblocks
+    p.output_size = output_size
+    p.input_stride = _strides(input)
+    return p
+
+
+def multiply_fw(twiddle, input, increasing_stride, output_size=None):
+    """Forward through the C ABI; twiddle must be dense.  Returns (B, S, output_size)."""
+    assert twiddle.is_contiguous() and twiddle.is_cuda and input.is_cuda
+    nb, log_n = twiddle.shape[1], twiddle.shape[2]
+    n = 1 << log_n
+    O = n if output_size is None else output_size
+    p = make_problem(input, log_n, nb, increasing_stride, O)
+    out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
+    p.output_stride = _strides(out)
+    _check(lib().bf_butterfly_multiply_fw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(out), _stream()))
+    return out
+
+
+def multiply_bw(twiddle, input, grad, increasing_stride):
+    assert twiddle.is_contiguous() and twiddle.is_cuda and input.is_cuda and grad.is_cuda
+    nb, log_n = twiddle.shape[1], twiddle.shape[2]
+    p = make_problem(input, log_n, nb, increasing_stride, grad.shape[2])
+    p.output_stride = _strides(grad)
+    d_twiddle = torch.empty_like(twiddle)
+    d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
+    p.d_input_stride = _strides(d_input)
+    nbytes = lib().bf_butterfly_multiply_bw_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_bw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
+                                          _ptr(d_twiddle), _ptr(d_input), _ptr(ws), nbytes, _stream()))
+    return d_twiddle, d_input
+
+
+def multiply_base4_fw(twiddle4, twiddle2, input, increasing_stride, output_size=None):
+    assert twiddle4.is_contiguous() and twiddle2.is_contiguous()
+    nb = twiddle4.shape[1]
+    log_n = twiddle4.shape[2] * 2 + twiddle2.shape[2]
+    n = 1 << log_n
+    O = n if output_size is None else output_size
+    p = make_problem(input, log_n, nb, increasing_stride, O)
+    out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
+    p.output_stride = _strides(out)
+    _check(lib().bf_butterfly_multiply_base4_fw(ctypes.byref(p), _ptr(twiddle4), _ptr(twiddle2),
+                                                _ptr(input), _ptr(out), _stream()))
+    return out
+
+
+def multiply_base4_bw(twiddle4, twiddle2, input, grad, increasing_stride):
+    assert twiddle4.is_contiguous() and twiddle2.is_contiguous()
+    nb = twiddle4.shape[1]
+    log_n = twiddle4.shape[2] * 2 + twiddle2.shape[2]
+    p = make_problem(input, log_n, nb, increasing_stride, grad.shape[2])
+    p.output_stride = _strides(grad)
+    d4, d2 = torch.empty_like(twiddle4), torch.empty_like(twiddle2)
+    d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
+    p.d_input_stride = _strides(d_input)
+    nbytes = lib().bf_butterfly_multiply_base4_bw_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_base4_bw(ctypes.byref(p), _ptr(twiddle4), _ptr(twiddle2), _ptr(input),
+                                                _ptr(grad), _ptr(d4), _ptr(d2), _ptr(d_input), _ptr(ws),
+                                                nbytes, _stream()))
+    return d4, d2, d_input

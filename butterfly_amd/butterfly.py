@@ -1,0 +1,182 @@
+"""``Butterfly``: an ``nn.Linear``-compatible layer whose weight is a product of butterfly
+factors, evaluated by the native multiply.
+
+Mirrors the constructor, parameters (``twiddle``, ``bias``), state-dict layout and forward
+flags of the reference module (torch_butterfly/butterfly.py:15-207).
+"""
+import math
+import numbers
+
+import torch
+from torch import nn
+
+from .complex_utils import complex_reshape, real_dtype_to_complex
+from .multiply import butterfly_multiply
+
+_INITS = ("empty", "randn", "ortho", "identity", "fft_no_br", "ifft_no_br")
+
+
+def _ortho_real(core_shape):
+    """Random 2x2 rotations / reflections [[d c, -d s], [s, c]], d = +-1."""
+    theta = torch.rand(core_shape) * (2 * math.pi)
+    c, s = theta.cos(), theta.sin()
+    d = torch.randint(0, 2, core_shape, dtype=c.dtype) * 2 - 1
+    return torch.stack((torch.stack((d * c, -d * s), -1), torch.stack((s, c), -1)), -2)
+
+
+def _ortho_complex(core_shape):
+    """Haar-distributed U(2) factors: [[e^{i(a+p)} c, e^{i(a+x)} s], [-e^{i(a-x)} s, e^{i(a-p)} c]]."""
+    phi = torch.rand(core_shape).sqrt().asin()
+    c, s = phi.cos(), phi.sin()
+    alpha, psi, chi = torch.rand((3,) + tuple(core_shape)) * (2 * math.pi)
+    top = torch.stack((torch.exp(1j * (alpha + psi)) * c, torch.exp(1j * (alpha + chi)) * s), -1)
+    bot = torch.stack((-torch.exp(1j * (alpha - chi)) * s, torch.exp(1j * (alpha - psi)) * c), -1)
+    return torch.stack((top, bot), -2)
+
+
+class Butterfly(nn.Module):
+    """Product of ``nblocks * log_n`` butterfly factors (block-diagonal 2x2 stages).
+
+    Parameters:
+        in_size, out_size: like ``nn.Linear``.  ``n`` is ``in_size`` rounded up to a power of 2
+            and ``nstacks = ceil(out_size / n)`` independent products are stacked.
+        bias: learn an additive bias of size ``out_size``.
+        complex: complex64/128 twiddle instead of real.
+        increasing_stride: the first block multiplies with stride 1, 2, ..., n/2 (else
+            n/2, ..., 1); the direction alternates from block to block.
+        init: a tensor of shape (nstacks, nblocks, log_n, n/2, 2, 2), or one of 'randn',
+            'ortho', 'identity', 'fft_no_br', 'ifft_no_br', 'empty'.
+        nblocks: number of alternating B / B^T blocks.
+    """
+
+    def __init__(self, in_size, out_size, bias=True, complex=False, increasing_stride=True,
+                 init="randn", nblocks=1):
+        super().__init__()
+        if nblocks < 1:
+            raise ValueError("nblocks must be >= 1")
+        self.in_size = in_size
+        self.out_size = out_size
+        self.log_n = int(math.ceil(math.log2(in_size)))
+        self.n = 1 << self.log_n
+        self.nstacks = -(-out_size // self.n)
+        self.complex = complex
+        self.increasing_stride = increasing_stride
+        self.nblocks = nblocks
+        dtype = torch.get_default_dtype()
+        if complex:
+            dtype = real_dtype_to_complex[dtype]
+        shape = (self.nstacks, nblocks, self.log_n, self.n // 2, 2, 2)
+        if isinstance(init, torch.Tensor):
+            if tuple(init.shape) != shape or init.dtype != dtype:
+                raise ValueError(f"init tensor must have shape {shape} and dtype {dtype}")
+            self.init = None
+            self.twiddle = nn.Parameter(init.clone())
+        else:
+            if init not in _INITS:
+                raise ValueError(f"init must be a tensor or one of {_INITS}")
+            self.init = init
+            self.twiddle = nn.Parameter(torch.empty(shape, dtype=dtype))
+        if bias:
+            self.bias = nn.Parameter(torch.empty(out_size, dtype=dtype))
+        else:
+            self.register_parameter("bias", None)
+        self.twiddle._is_structured = True  # lets optimisers exempt it from weight decay
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        if self.bias is not None:
+            bound = 1 / math.sqrt(self.in_size)  # same rule as nn.Linear
+            nn.init.uniform_(self.bias, -bound, bound)
+        tw = self.twiddle
+        if self.init in (None, "empty"):
+            return
+        with torch.no_grad():
+            if self.init == "randn":
+                # variance 1/2 per entry keeps the output variance equal to the input's
+                tw.copy_(torch.randn(tw.shape, dtype=tw.dtype) / math.sqrt(2))
+            elif self.init == "ortho":
+                core = tw.shape[:-2]
+                tw.copy_(_ortho_complex(core) if self.complex else _ortho_real(core))
+            elif self.init == "identity":
+                tw.copy_(torch.eye(2, dtype=tw.dtype).expand(tw.shape))
+            else:
+                if not self.complex:
+                    raise ValueError("fft_no_br / ifft_no_br init needs complex=True")
+                from . import special
+                make = special.fft if self.init == "fft_no_br" else special.ifft
+                b = make(self.n, normalized=True, br_first=self.increasing_stride, with_br_perm=False)
+                tw[:, 0] = b.twiddle
+                if self.nblocks > 1:
+                    tw[:, 1:] = torch.eye(2, dtype=tw.dtype)
+
+    def forward(self, input, transpose=False, conjugate=False, subtwiddle=False):
+        """input (batch, *, in_size) -> (batch, *, out_size).
+
+        transpose / conjugate apply the transposed / conjugated matrix; subtwiddle uses only
+        the leading part of the parameters for a shorter input (output is then
+        nstacks * n' wide, n' the input size rounded up to a power of 2)."""
+        twiddle = self.twiddle
+        x = self.pre_process(input)
+        output_size = self.out_size if self.nstacks == 1 else None
+        if subtwiddle:
+            log_n = int(math.ceil(math.log2(input.size(-1))))
+            half = (1 << log_n) // 2
+            if self.increasing_stride:
+                twiddle = twiddle[:, :, :log_n, :half]
+            else:
+                twiddle = twiddle[:, :, self.log_n - log_n:, :half]
+            output_size = None
+        if conjugate and self.complex:
+            twiddle = twiddle.conj()
+        if transpose:
+            # (prod of stages)^T: transpose every 2x2 and reverse the stage and block order
+            twiddle = twiddle.transpose(-1, -2).flip([1, 2])
+            last_inc = self.increasing_stride != ((self.nblocks - 1) % 2 == 1)
+            x = butterfly_multiply(twiddle, x, not last_inc, output_size)
+        else:
+            x = butterfly_multiply(twiddle, x, self.increasing_stride, output_size)
+        return self.post_process(input, x, out_size=x.size(-1) if subtwiddle else None)
+
+    def pre_process(self, input):
+        size = input.size(-1)
+        x = complex_reshape(input, -1, size)
+        return x.unsqueeze(1).expand(x.shape[0], self.nstacks, size)
+
+    def post_process(self, input, output, out_size=None):
+        out_size = self.out_size if out_size is None else out_size
+        batch = output.shape[0]
+        flat = output.reshape(batch, self.nstacks * output.size(-1))
+        if flat.shape[-1] != out_size:
+            flat = flat[:, :out_size]
+        if self.bias is not None:
+            flat = flat + self.bias[:out_size]
+        return flat.reshape(*input.shape[:-1], out_size)
+
+    def __imul__(self, scale):
+        """Scale the whole matrix by a non-negative number, spread evenly over the stages."""
+        if not isinstance(scale, numbers.Number) or scale < 0:
+            raise ValueError("scale must be a non-negative number")
+        self.twiddle *= scale ** (1.0 / (self.twiddle.shape[1] * self.twiddle.shape[2]))
+        return self
+
+    def diagonal_multiply_(self, diagonal, diag_first):
+        from .combine import diagonal_butterfly
+        return diagonal_butterfly(self, diagonal, diag_first, inplace=True)
+
+    def to_base4(self):
+        from .butterfly_base4 import ButterflyBase4
+        from .multiply_base4 import twiddle_base2_to_base4
+        with torch.no_grad():
+            tw4, tw2 = twiddle_base2_to_base4(self.twiddle, self.increasing_stride)
+        new = ButterflyBase4(self.in_size, self.out_size, self.bias is not None, self.complex,
+                             self.increasing_stride, init=(tw4, tw2),
+                             nblocks=self.nblocks).to(self.twiddle.device)
+        if new.bias is not None:
+            with torch.no_grad():
+                new.bias.copy_(self.bias)
+        return new
+
+    def extra_repr(self):
+        return (f"in_size={self.in_size}, out_size={self.out_size}, bias={self.bias is not None}, "
+                f"complex={self.complex}, increasing_stride={self.increasing_stride}, "
+                f"init={self.init}, nblocks={self.nblocks}")

@@ -1,0 +1,405 @@
+// C ABI of libbutterfly_hip.so: argument checks, launch planning and kernel launches.
+// See include/butterfly_hip.h for the contract of every entry point.
+
+#include "../../include/butterfly_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_version.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <mutex>
+#include <string>
+
+#include "common.hpp"
+#include "generic.hpp"
+
+namespace {
+
+using namespace bf;
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+#define BF_HIP_CHECK(expr)                                                              \
+    do {                                                                                \
+        hipError_t e_ = (expr);                                                         \
+        if (e_ != hipSuccess)                                                           \
+            return fail(BF_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));     \
+    } while (0)
+
+constexpr size_t kLdsBytes = 160 * 1024;        // LDS per compute unit on gfx950
+constexpr size_t kGenericFwLds = 128 * 1024;    // most a generic forward workgroup stages
+constexpr size_t kGenericBwLds = 144 * 1024;    // most a generic backward workgroup stages
+constexpr int kMaxGrid = 1 << 30;
+
+size_t elem_bytes(int dtype) { return dtype == BF_C64 ? 8 : 4; }
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// ---- validation -----------------------------------------------------------------------
+
+int check_problem(const bf_problem *p, bool backward)
+{
+    if (!p) return fail(BF_ERR_INVALID, "problem descriptor is NULL");
+    if (p->dtype != BF_F32 && p->dtype != BF_C64)
+        return fail(BF_ERR_INVALID, "dtype must be BF_F32 or BF_C64 (device kernels cover float and complex64)");
+    if (p->batch < 0 || p->nstacks < 0 || p->nblocks < 0 || p->input_size < 0 || p->output_size < 0)
+        return fail(BF_ERR_INVALID, "sizes must be non-negative");
+    if (p->log_n < 0 || p->log_n > 30) return fail(BF_ERR_INVALID, "log_n must be in [0, 30]");
+    const int64_t n = (int64_t)1 << p->log_n;
+    if (p->output_size > n) return fail(BF_ERR_INVALID, "output_size must be <= n");
+    for (int i = 0; i < 3; ++i) {
+        if (p->input_stride[i] < 0 || p->output_stride[i] < 0 || (backward && p->d_input_stride[i] < 0))
+            return fail(BF_ERR_INVALID, "strides must be non-negative");
+    }
+    if (p->nstacks > 65535) return fail(BF_ERR_UNSUPPORTED, "nstacks above 65535 is not supported");
+    if (p->batch > ((int64_t)1 << 40)) return fail(BF_ERR_UNSUPPORTED, "batch too large");
+    return BF_OK;
+}
+
+Schedule make_schedule(const bf_problem *p, bool base4)
+{
+    Schedule sc;
+    sc.log_n = (int)p->log_n;
+    sc.nblocks = (int)p->nblocks;
+    sc.increasing_stride = p->increasing_stride != 0;
+    sc.base4 = base4;
+    const int64_t n = (int64_t)1 << p->log_n;
+    if (base4) {
+        sc.per = (int)(p->log_n / 2 + p->log_n % 2);
+        sc.tw4_stack_stride = p->nblocks * (p->log_n / 2) * (n / 4) * 16;
+        sc.tw2_stack_stride = p->nblocks * (p->log_n % 2) * (n / 2) * 4;
+    } else {
+        sc.per = (int)p->log_n;
+        sc.tw4_stack_stride = 0;
+        sc.tw2_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
+    }
+    return sc;
+}
+
+View make_view(const int64_t stride[3], int64_t width)
+{
+    View v;
+    v.sb = stride[0];
+    v.ss = stride[1];
+    v.se = stride[2];
+    v.width = width;
+    return v;
+}
+
+View dense_view(int64_t nstacks, int64_t n)
+{
+    View v;
+    v.sb = nstacks * n;
+    v.ss = n;
+    v.se = 1;
+    v.width = n;
+    return v;
+}
+
+// ---- one-time kernel attributes ---------------------------------------------------------
+
+std::once_flag g_attr_once;
+hipError_t g_attr_status = hipSuccess;
+
+void set_attributes()
+{
+    auto set = [](const void *fn, size_t bytes) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess && g_attr_status == hipSuccess) g_attr_status = e;
+    };
+    set(reinterpret_cast<const void *>(&generic_fw_kernel<float>), kGenericFwLds);
+    set(reinterpret_cast<const void *>(&generic_fw_kernel<float2>), kGenericFwLds);
+    set(reinterpret_cast<const void *>(&generic_bw_kernel<float>), kGenericBwLds);
+    set(reinterpret_cast<const void *>(&generic_bw_kernel<float2>), kGenericBwLds);
+}
+
+int ensure_attributes()
+{
+    std::call_once(g_attr_once, set_attributes);
+    if (g_attr_status != hipSuccess)
+        return fail(BF_ERR_HIP, "hipFuncSetAttribute failed: %s", hipGetErrorString(g_attr_status));
+    return BF_OK;
+}
+
+// ---- generic forward ----------------------------------------------------------------------
+
+int launch_generic_fw(const bf_problem *p, const Schedule &sc, int t0, int t1, const void *tw2,
+                      const void *tw4, const void *in, const View &in_view, void *out,
+                      const View &out_view, hipStream_t stream)
+{
+    const int64_t n = (int64_t)1 << p->log_n;
+    const size_t row_bytes = (size_t)n * elem_bytes(p->dtype);
+    if (row_bytes > kGenericFwLds)
+        return fail(BF_ERR_UNSUPPORTED, "n = %lld does not fit in LDS (row of %zu bytes, limit %zu)",
+                    (long long)n, row_bytes, kGenericFwLds);
+    if (p->batch == 0 || p->nstacks == 0) return BF_OK;
+    int64_t rows = std::max<int64_t>(1, (int64_t)(64 * 1024 / row_bytes));
+    rows = std::min<int64_t>(rows, 32);
+    while (rows > 1 && ((p->batch + rows - 1) / rows) * p->nstacks < 2048) rows /= 2;
+    const int64_t gx = (p->batch + rows - 1) / rows;
+    if (gx > kMaxGrid) return fail(BF_ERR_UNSUPPORTED, "batch too large for one launch");
+    GenericFwArgs a;
+    a.sc = sc;
+    a.t0 = t0;
+    a.t1 = t1;
+    a.rows_per_wg = (int)rows;
+    a.batch = p->batch;
+    a.tw2 = tw2;
+    a.tw4 = tw4;
+    a.in = in;
+    a.in_view = in_view;
+    a.out = out;
+    a.out_view = out_view;
+    const dim3 grid((unsigned)gx, (unsigned)p->nstacks);
+    const size_t lds = (size_t)rows * row_bytes;
+    if (p->dtype == BF_F32)
+        hipLaunchKernelGGL(generic_fw_kernel<float>, grid, dim3(kGenericThreads), lds, stream, a);
+    else
+        hipLaunchKernelGGL(generic_fw_kernel<float2>, grid, dim3(kGenericThreads), lds, stream, a);
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
+}
+
+int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, const void *input,
+            void *output, void *stream_)
+{
+    int rc = check_problem(p, false);
+    if (rc) return rc;
+    if ((rc = ensure_attributes())) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const Schedule sc = make_schedule(p, base4);
+    const int64_t n = (int64_t)1 << p->log_n;
+    if (p->batch > 0 && p->nstacks > 0) {
+        if (!input && p->input_size > 0) return fail(BF_ERR_INVALID, "input is NULL");
+        if (!output && p->output_size > 0) return fail(BF_ERR_INVALID, "output is NULL");
+        if (sc.per * sc.nblocks > 0) {
+            if (!base4 && !tw2) return fail(BF_ERR_INVALID, "twiddle is NULL");
+            if (base4 && p->log_n >= 2 && !tw4) return fail(BF_ERR_INVALID, "twiddle4 is NULL");
+            if (base4 && (p->log_n & 1) && !tw2) return fail(BF_ERR_INVALID, "twiddle2 is NULL");
+        }
+    }
+    const View in_view = make_view(p->input_stride, std::min(p->input_size, n));
+    const View out_view = make_view(p->output_stride, p->output_size);
+    return launch_generic_fw(p, sc, 0, sc.per * sc.nblocks, tw2, tw4, input, in_view, output,
+                             out_view, stream);
+}
+
+// ---- generic backward -----------------------------------------------------------------------
+
+struct BwPlan {
+    int nstages;
+    int chunk;          // stages per launch
+    int nchunks;
+    int64_t nparts;     // persistent workgroups per stack
+    int64_t slot;       // scalars per stage in the partial buffer
+    size_t boundary_bytes;  // one (B, S, n) activation plane
+    size_t off_boundaries, off_gbuf, off_partials, total;
+    bool fits;
+};
+
+BwPlan plan_bw(const bf_problem *p, bool base4)
+{
+    BwPlan pl = {};
+    const int64_t n = (int64_t)1 << p->log_n;
+    const size_t e = elem_bytes(p->dtype);
+    const size_t row_bytes = (size_t)n * e;
+    const Schedule sc = make_schedule(p, base4);
+    pl.nstages = sc.per * sc.nblocks;
+    pl.fits = 2 * row_bytes <= kGenericBwLds;
+    if (!pl.fits) return pl;
+    const int cmax = (int)(kGenericBwLds / row_bytes) - 1;
+    pl.nchunks = pl.nstages == 0 ? 0 : (pl.nstages + cmax - 1) / cmax;
+    pl.chunk = pl.nchunks == 0 ? 0 : (pl.nstages + pl.nchunks - 1) / pl.nchunks;
+    pl.nparts = std::min<int64_t>(p->batch, std::max<int64_t>(1, 512 / std::max<int64_t>(1, p->nstacks)));
+    pl.slot = base4 ? 4 * n : 2 * n;
+    pl.boundary_bytes = align256((size_t)p->batch * p->nstacks * row_bytes);
+    size_t off = 0;
+    pl.off_boundaries = off;
+    off += pl.nchunks > 1 ? (size_t)(pl.nchunks - 1) * pl.boundary_bytes : 0;
+    pl.off_gbuf = off;
+    off += pl.nchunks > 1 ? pl.boundary_bytes : 0;
+    pl.off_partials = off;
+    off += align256((size_t)pl.nparts * p->nstacks * pl.chunk * pl.slot * e);
+    pl.total = off;
+    return pl;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void copy_pad_kernel(const T *in, View iv, T *out, View ov, int64_t batch)
+{
+    const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int s = blockIdx.y;
+    if (j >= ov.width) return;
+    for (int64_t b = blockIdx.z; b < batch; b += gridDim.z) {
+        T v = zero_of(T());
+        if (j < iv.width) v = in[b * iv.sb + s * iv.ss + j * iv.se];
+        out[b * ov.sb + s * ov.ss + j * ov.se] = v;
+    }
+}
+
+int launch_copy_pad(const bf_problem *p, const void *in, const View &iv, void *out, const View &ov,
+                    hipStream_t stream)
+{
+    if (p->batch == 0 || p->nstacks == 0 || ov.width == 0) return BF_OK;
+    const dim3 grid((unsigned)((ov.width + 255) / 256), (unsigned)p->nstacks,
+                    (unsigned)std::min<int64_t>(p->batch, 1024));
+    if (p->dtype == BF_F32)
+        hipLaunchKernelGGL(copy_pad_kernel<float>, grid, dim3(256), 0, stream, (const float *)in, iv,
+                           (float *)out, ov, p->batch);
+    else
+        hipLaunchKernelGGL(copy_pad_kernel<float2>, grid, dim3(256), 0, stream, (const float2 *)in, iv,
+                           (float2 *)out, ov, p->batch);
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
+}
+
+int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, const void *input,
+             const void *grad, void *d_tw2, void *d_tw4, void *d_input, void *workspace,
+             size_t workspace_bytes, void *stream_)
+{
+    int rc = check_problem(p, true);
+    if (rc) return rc;
+    if ((rc = ensure_attributes())) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const Schedule sc = make_schedule(p, base4);
+    const int64_t n = (int64_t)1 << p->log_n;
+    const BwPlan pl = plan_bw(p, base4);
+    if (!pl.fits)
+        return fail(BF_ERR_UNSUPPORTED, "n = %lld does not fit in LDS for the backward pass", (long long)n);
+    if (pl.total > 0 && (!workspace || workspace_bytes < pl.total))
+        return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", pl.total, workspace_bytes);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
+        return fail(BF_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+
+    const View x_view = make_view(p->input_stride, std::min(p->input_size, n));
+    const View g_view = make_view(p->output_stride, std::min(p->output_size, n));
+    const View di_view = make_view(p->d_input_stride, p->input_size);
+    const View dense = dense_view(p->nstacks, n);
+    char *ws = static_cast<char *>(workspace);
+
+    if (pl.nstages == 0) return launch_copy_pad(p, grad, g_view, d_input, di_view, stream);
+
+    const bool have_rows = p->batch > 0 && p->nstacks > 0;
+    // forward launches that materialise the input of every chunk after the first
+    for (int c = 1; c < pl.nchunks && have_rows; ++c) {
+        const void *src = c == 1 ? input : ws + pl.off_boundaries + (size_t)(c - 2) * pl.boundary_bytes;
+        void *dst = ws + pl.off_boundaries + (size_t)(c - 1) * pl.boundary_bytes;
+        rc = launch_generic_fw(p, sc, (c - 1) * pl.chunk, c * pl.chunk, tw2, tw4, src,
+                               c == 1 ? x_view : dense, dst, dense, stream);
+        if (rc) return rc;
+    }
+    const size_t e = elem_bytes(p->dtype);
+    for (int c = pl.nchunks - 1; c >= 0; --c) {
+        const int t0 = c * pl.chunk;
+        const int t1 = std::min(pl.nstages, t0 + pl.chunk);
+        if (have_rows) {
+            GenericBwArgs a;
+            a.sc = sc;
+            a.t0 = t0;
+            a.t1 = t1;
+            a.batch = p->batch;
+            a.tw2 = tw2;
+            a.tw4 = tw4;
+            a.x_in = c == 0 ? input : ws + pl.off_boundaries + (size_t)(c - 1) * pl.boundary_bytes;
+            a.x_view = c == 0 ? x_view : dense;
+            a.g_out = c == pl.nchunks - 1 ? grad : ws + pl.off_gbuf;
+            a.g_view = c == pl.nchunks - 1 ? g_view : dense;
+            a.g_in = c == 0 ? d_input : ws + pl.off_gbuf;
+            a.gi_view = c == 0 ? di_view : dense;
+            a.partial = ws + pl.off_partials;
+            a.slot = pl.slot;
+            const dim3 grid((unsigned)pl.nparts, (unsigned)p->nstacks);
+            const size_t lds = (size_t)(t1 - t0 + 1) * n * e;
+            if (p->dtype == BF_F32)
+                hipLaunchKernelGGL(generic_bw_kernel<float>, grid, dim3(kGenericThreads), lds, stream, a);
+            else
+                hipLaunchKernelGGL(generic_bw_kernel<float2>, grid, dim3(kGenericThreads), lds, stream, a);
+            BF_HIP_CHECK(hipGetLastError());
+        }
+        if (p->nstacks > 0) {
+            ReduceArgs r;
+            r.sc = sc;
+            r.t0 = t0;
+            r.t1 = t1;
+            r.nparts = have_rows ? (int)pl.nparts : 0;
+            r.nstacks = p->nstacks;
+            r.partial = ws + pl.off_partials;
+            r.slot = pl.slot;
+            r.d_tw2 = d_tw2;
+            r.d_tw4 = d_tw4;
+            const dim3 grid((unsigned)((pl.slot + 255) / 256), (unsigned)(t1 - t0), (unsigned)p->nstacks);
+            if (p->dtype == BF_F32)
+                hipLaunchKernelGGL(reduce_partials_kernel<float>, grid, dim3(256), 0, stream, r);
+            else
+                hipLaunchKernelGGL(reduce_partials_kernel<float2>, grid, dim3(256), 0, stream, r);
+            BF_HIP_CHECK(hipGetLastError());
+        }
+    }
+    return BF_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int bf_version(void) { return 100; }
+
+int bf_hip_version(void) { return HIP_VERSION; }
+
+const char *bf_last_error(void) { return g_last_error.c_str(); }
+
+int bf_butterfly_multiply_fw(const bf_problem *p, const void *twiddle, const void *input,
+                             void *output, void *stream)
+{
+    return forward(p, false, twiddle, nullptr, input, output, stream);
+}
+
+size_t bf_butterfly_multiply_bw_workspace_bytes(const bf_problem *p)
+{
+    if (check_problem(p, true)) return 0;
+    return plan_bw(p, false).total;
+}
+
+int bf_butterfly_multiply_bw(const bf_problem *p, const void *twiddle, const void *input,
+                             const void *grad, void *d_twiddle, void *d_input, void *workspace,
+                             size_t workspace_bytes, void *stream)
+{
+    return backward(p, false, twiddle, nullptr, input, grad, d_twiddle, nullptr, d_input, workspace,
+                    workspace_bytes, stream);
+}
+
+int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4, const void *twiddle2,
+                                   const void *input, void *output, void *stream)
+{
+    return forward(p, true, twiddle2, twiddle4, input, output, stream);
+}
+
+size_t bf_butterfly_multiply_base4_bw_workspace_bytes(const bf_problem *p)
+{
+    if (check_problem(p, true)) return 0;
+    return plan_bw(p, true).total;
+}
+
+int bf_butterfly_multiply_base4_bw(const bf_problem *p, const void *twiddle4, const void *twiddle2,
+                                   const void *input, const void *grad, void *d_twiddle4,
+                                   void *d_twiddle2, void *d_input, void *workspace,
+                                   size_t workspace_bytes, void *stream)
+{
+    return backward(p, true, twiddle2, twiddle4, input, grad, d_twiddle2, d_twiddle4, d_input,
+                    workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,294 @@
+// torch-library shim: registers the torch_butterfly operators and forwards them to the
+// C ABI of libbutterfly_hip.so.  No kernels live here.
+//
+// Operator names, argument order and checks follow the reference shim
+// (csrc/butterfly.cpp:20-131): twiddle first, then input, the stride flag and the
+// optional output size.  The base-4 operators are new; their argument order follows
+// butterfly_multiply_base4_torch (torch_butterfly/multiply_base4.py:7-8).
+//
+// Device tensors only: there is deliberately no CPU path behind these operators.
+
+#include <ATen/ATen.h>
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/csrc/autograd/custom_function.h>
+#include <torch/library.h>
+
+#include <tuple>
+
+#include "../../include/butterfly_hip.h"
+
+namespace {
+
+using at::Tensor;
+
+#define CHECK_DEVICE(x) \
+    TORCH_CHECK(x.device().type() == at::kCPU || x.device().type() == at::kCUDA, #x " must be on CPU or CUDA")
+#define CHECK_SAME_DEVICE(x, y) TORCH_CHECK(x.device() == y.device(), #x " and " #y " must be on the same device")
+#define CHECK_DIM(x, y) TORCH_CHECK(x.dim() == y, #x " must have dimension " #y)
+#define CHECK_SHAPE(x, ...) \
+    TORCH_CHECK(x.sizes() == at::IntArrayRef({__VA_ARGS__}), #x " must have shape (" #__VA_ARGS__ ")")
+
+int dtype_code(const Tensor &t, const char *who)
+{
+    if (t.scalar_type() == at::kFloat) return BF_F32;
+    if (t.scalar_type() == at::kComplexFloat) return BF_C64;
+    TORCH_CHECK(false, who, ": device kernels support float32 and complex64, got ", t.scalar_type());
+    return -1;
+}
+
+void require_device(const Tensor &t, const char *who)
+{
+    TORCH_CHECK(t.is_cuda(), who, ": tensors must live on a HIP device; this library has no CPU path");
+}
+
+void set_strides(int64_t dst[3], const Tensor &t)
+{
+    for (int i = 0; i < 3; ++i) dst[i] = t.size(i) > 1 ? t.stride(i) : 0;
+    for (int i = 0; i < 3; ++i) TORCH_CHECK(dst[i] >= 0, "negative strides are not supported");
+}
+
+void check_rc(int rc, const char *who) { TORCH_CHECK(rc == BF_OK, who, ": ", bf_last_error()); }
+
+// Dense copy of a (small) twiddle tensor; also materialises lazy conjugation.
+Tensor dense(const Tensor &t) { return t.resolve_conj().contiguous(); }
+
+struct Shapes {
+    int64_t batch, nstacks, nblocks, log_n, n, input_size;
+};
+
+bf_problem make_problem(const Shapes &s, const Tensor &input, bool increasing_stride, int64_t output_size,
+                        const char *who)
+{
+    bf_problem p = {};
+    p.dtype = dtype_code(input, who);
+    p.increasing_stride = increasing_stride;
+    p.batch = s.batch;
+    p.nstacks = s.nstacks;
+    p.log_n = s.log_n;
+    p.nblocks = s.nblocks;
+    p.input_size = s.input_size;
+    p.output_size = output_size;
+    set_strides(p.input_stride, input);
+    return p;
+}
+
+// ---- base-2 -----------------------------------------------------------------------------
+
+Tensor butterfly_multiply_fw(const Tensor twiddle, const Tensor input, bool increasing_stride,
+                             c10::optional<int64_t> output_size)
+{
+    CHECK_DEVICE(twiddle); CHECK_DEVICE(input); CHECK_SAME_DEVICE(twiddle, input);
+    CHECK_DIM(twiddle, 6); CHECK_DIM(input, 3);
+    Shapes s;
+    s.batch = input.size(0);
+    s.nstacks = input.size(1);
+    s.input_size = input.size(2);
+    s.nblocks = twiddle.size(1);
+    s.log_n = twiddle.size(2);
+    TORCH_CHECK(s.log_n <= 30, "butterfly_multiply_fw: n must be a power of 2");
+    s.n = (int64_t)1 << s.log_n;
+    CHECK_SHAPE(twiddle, s.nstacks, s.nblocks, s.log_n, s.n / 2, 2, 2);
+    const int64_t output_size_val = output_size.has_value() ? output_size.value() : s.n;
+    TORCH_CHECK(output_size_val <= s.n, "butterfly_multiply_fw: output_size must be <= n");
+    TORCH_CHECK(output_size_val >= 0, "butterfly_multiply_fw: output_size must be >= 0");
+    require_device(input, "butterfly_multiply_fw");
+    TORCH_CHECK(twiddle.scalar_type() == input.scalar_type(),
+                "butterfly_multiply_fw: twiddle and input must have the same dtype");
+
+    const c10::hip::HIPGuard guard(input.device());
+    const Tensor tw = dense(twiddle);
+    const Tensor x = input.resolve_conj();
+    Tensor output = at::empty({s.batch, s.nstacks, s.n}, x.options());
+    if (output_size_val < s.n) output = output.slice(2, 0, output_size_val);
+    bf_problem p = make_problem(s, x, increasing_stride, output_size_val, "butterfly_multiply_fw");
+    set_strides(p.output_stride, output);
+    check_rc(bf_butterfly_multiply_fw(&p, tw.data_ptr(), x.data_ptr(), output.data_ptr(),
+                                      c10::hip::getCurrentHIPStream().stream()),
+             "butterfly_multiply_fw");
+    return output;
+}
+
+std::tuple<Tensor, Tensor> butterfly_multiply_bw(const Tensor twiddle, const Tensor input,
+                                                 const Tensor grad, bool increasing_stride)
+{
+    CHECK_DEVICE(twiddle); CHECK_DEVICE(input); CHECK_DEVICE(grad);
+    CHECK_SAME_DEVICE(twiddle, input); CHECK_SAME_DEVICE(input, grad);
+    CHECK_DIM(twiddle, 6); CHECK_DIM(input, 3); CHECK_DIM(grad, 3);
+    Shapes s;
+    s.batch = input.size(0);
+    s.nstacks = input.size(1);
+    s.input_size = input.size(2);
+    s.nblocks = twiddle.size(1);
+    s.log_n = twiddle.size(2);
+    TORCH_CHECK(s.log_n <= 30, "butterfly_multiply_bw: n must be a power of 2");
+    s.n = (int64_t)1 << s.log_n;
+    const int64_t output_size = grad.size(2);
+    CHECK_SHAPE(twiddle, s.nstacks, s.nblocks, s.log_n, s.n / 2, 2, 2);
+    CHECK_SHAPE(grad, s.batch, s.nstacks, output_size);
+    TORCH_CHECK(output_size <= s.n, "butterfly_multiply_bw: grad must have at most n columns");
+    require_device(input, "butterfly_multiply_bw");
+    TORCH_CHECK(twiddle.scalar_type() == input.scalar_type() && grad.scalar_type() == input.scalar_type(),
+                "butterfly_multiply_bw: twiddle, input and grad must have the same dtype");
+
+    const c10::hip::HIPGuard guard(input.device());
+    const Tensor tw = dense(twiddle);
+    const Tensor x = input.resolve_conj();
+    const Tensor g = grad.resolve_conj();
+    Tensor d_twiddle = at::empty(tw.sizes(), tw.options());
+    Tensor d_input = at::empty({s.batch, s.nstacks, std::max(s.input_size, s.n)}, x.options());
+    if (s.input_size < s.n) d_input = d_input.slice(2, 0, s.input_size);
+    bf_problem p = make_problem(s, x, increasing_stride, output_size, "butterfly_multiply_bw");
+    set_strides(p.output_stride, g);
+    set_strides(p.d_input_stride, d_input);
+    const size_t ws_bytes = bf_butterfly_multiply_bw_workspace_bytes(&p);
+    Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+    check_rc(bf_butterfly_multiply_bw(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), d_twiddle.data_ptr(),
+                                      d_input.data_ptr(), ws.data_ptr(), ws_bytes,
+                                      c10::hip::getCurrentHIPStream().stream()),
+             "butterfly_multiply_bw");
+    return std::make_tuple(d_twiddle, d_input);
+}
+
+using torch::autograd::AutogradContext;
+using torch::autograd::variable_list;
+
+class ButterflyMultiply : public torch::autograd::Function<ButterflyMultiply> {
+public:
+    static Tensor forward(AutogradContext *ctx, Tensor twiddle, Tensor input, bool increasing_stride,
+                          c10::optional<int64_t> output_size)
+    {
+        ctx->saved_data["increasing_stride"] = increasing_stride;
+        ctx->save_for_backward({twiddle, input});
+        return butterfly_multiply_fw(twiddle, input, increasing_stride, output_size);
+    }
+
+    static variable_list backward(AutogradContext *ctx, variable_list grad_output)
+    {
+        const auto saved = ctx->get_saved_variables();
+        const bool increasing_stride = ctx->saved_data["increasing_stride"].toBool();
+        auto result = butterfly_multiply_bw(saved[0], saved[1], grad_output[0], increasing_stride);
+        return {std::get<0>(result), std::get<1>(result), Tensor(), Tensor()};
+    }
+};
+
+Tensor butterfly_multiply(Tensor twiddle, Tensor input, bool increasing_stride,
+                          c10::optional<int64_t> output_size)
+{
+    return ButterflyMultiply::apply(twiddle, input, increasing_stride, output_size);
+}
+
+// ---- base-4 -----------------------------------------------------------------------------
+
+Shapes base4_shapes(const Tensor &twiddle4, const Tensor &twiddle2, const Tensor &input, const char *who)
+{
+    CHECK_DEVICE(twiddle4); CHECK_DEVICE(twiddle2); CHECK_DEVICE(input);
+    CHECK_SAME_DEVICE(twiddle4, input); CHECK_SAME_DEVICE(twiddle2, input);
+    CHECK_DIM(twiddle4, 6); CHECK_DIM(twiddle2, 6); CHECK_DIM(input, 3);
+    Shapes s;
+    s.batch = input.size(0);
+    s.nstacks = input.size(1);
+    s.input_size = input.size(2);
+    s.nblocks = twiddle4.size(1);
+    s.log_n = twiddle4.size(2) * 2 + twiddle2.size(2);
+    TORCH_CHECK(s.log_n <= 30, who, ": n must be a power of 2");
+    s.n = (int64_t)1 << s.log_n;
+    TORCH_CHECK(twiddle2.size(2) <= 1, "twiddle2 must have shape (nstacks, nblocks, log_n % 2, n / 2, 2, 2)");
+    if (s.log_n / 2 > 0) CHECK_SHAPE(twiddle4, s.nstacks, s.nblocks, s.log_n / 2, s.n / 4, 4, 4);
+    if (s.log_n % 2 == 1) CHECK_SHAPE(twiddle2, s.nstacks, s.nblocks, 1, s.n / 2, 2, 2);
+    require_device(input, who);
+    TORCH_CHECK(twiddle4.scalar_type() == input.scalar_type() && twiddle2.scalar_type() == input.scalar_type(),
+                who, ": twiddle4, twiddle2 and input must have the same dtype");
+    return s;
+}
+
+Tensor butterfly_multiply_base4_fw(const Tensor twiddle4, const Tensor twiddle2, const Tensor input,
+                                   bool increasing_stride, c10::optional<int64_t> output_size)
+{
+    const Shapes s = base4_shapes(twiddle4, twiddle2, input, "butterfly_multiply_base4_fw");
+    const int64_t output_size_val = output_size.has_value() ? output_size.value() : s.n;
+    TORCH_CHECK(output_size_val <= s.n, "butterfly_multiply_base4_fw: output_size must be <= n");
+    TORCH_CHECK(output_size_val >= 0, "butterfly_multiply_base4_fw: output_size must be >= 0");
+    const c10::hip::HIPGuard guard(input.device());
+    const Tensor tw4 = dense(twiddle4), tw2 = dense(twiddle2);
+    const Tensor x = input.resolve_conj();
+    Tensor output = at::empty({s.batch, s.nstacks, s.n}, x.options());
+    if (output_size_val < s.n) output = output.slice(2, 0, output_size_val);
+    bf_problem p = make_problem(s, x, increasing_stride, output_size_val, "butterfly_multiply_base4_fw");
+    set_strides(p.output_stride, output);
+    check_rc(bf_butterfly_multiply_base4_fw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(),
+                                            output.data_ptr(), c10::hip::getCurrentHIPStream().stream()),
+             "butterfly_multiply_base4_fw");
+    return output;
+}
+
+std::tuple<Tensor, Tensor, Tensor> butterfly_multiply_base4_bw(const Tensor twiddle4, const Tensor twiddle2,
+                                                               const Tensor input, const Tensor grad,
+                                                               bool increasing_stride)
+{
+    const Shapes s = base4_shapes(twiddle4, twiddle2, input, "butterfly_multiply_base4_bw");
+    CHECK_DEVICE(grad); CHECK_SAME_DEVICE(input, grad); CHECK_DIM(grad, 3);
+    const int64_t output_size = grad.size(2);
+    CHECK_SHAPE(grad, s.batch, s.nstacks, output_size);
+    TORCH_CHECK(output_size <= s.n, "butterfly_multiply_base4_bw: grad must have at most n columns");
+    TORCH_CHECK(grad.scalar_type() == input.scalar_type(),
+                "butterfly_multiply_base4_bw: grad and input must have the same dtype");
+    const c10::hip::HIPGuard guard(input.device());
+    const Tensor tw4 = dense(twiddle4), tw2 = dense(twiddle2);
+    const Tensor x = input.resolve_conj();
+    const Tensor g = grad.resolve_conj();
+    Tensor d4 = at::empty(tw4.sizes(), tw4.options());
+    Tensor d2 = at::empty(tw2.sizes(), tw2.options());
+    Tensor d_input = at::empty({s.batch, s.nstacks, std::max(s.input_size, s.n)}, x.options());
+    if (s.input_size < s.n) d_input = d_input.slice(2, 0, s.input_size);
+    bf_problem p = make_problem(s, x, increasing_stride, output_size, "butterfly_multiply_base4_bw");
+    set_strides(p.output_stride, g);
+    set_strides(p.d_input_stride, d_input);
+    const size_t ws_bytes = bf_butterfly_multiply_base4_bw_workspace_bytes(&p);
+    Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+    check_rc(bf_butterfly_multiply_base4_bw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(), g.data_ptr(),
+                                            d4.data_ptr(), d2.data_ptr(), d_input.data_ptr(), ws.data_ptr(),
+                                            ws_bytes, c10::hip::getCurrentHIPStream().stream()),
+             "butterfly_multiply_base4_bw");
+    return std::make_tuple(d4, d2, d_input);
+}
+
+class ButterflyMultiplyBase4 : public torch::autograd::Function<ButterflyMultiplyBase4> {
+public:
+    static Tensor forward(AutogradContext *ctx, Tensor twiddle4, Tensor twiddle2, Tensor input,
+                          bool increasing_stride, c10::optional<int64_t> output_size)
+    {
+        ctx->saved_data["increasing_stride"] = increasing_stride;
+        ctx->save_for_backward({twiddle4, twiddle2, input});
+        return butterfly_multiply_base4_fw(twiddle4, twiddle2, input, increasing_stride, output_size);
+    }
+
+    static variable_list backward(AutogradContext *ctx, variable_list grad_output)
+    {
+        const auto saved = ctx->get_saved_variables();
+        const bool increasing_stride = ctx->saved_data["increasing_stride"].toBool();
+        auto r = butterfly_multiply_base4_bw(saved[0], saved[1], saved[2], grad_output[0], increasing_stride);
+        return {std::get<0>(r), std::get<1>(r), std::get<2>(r), Tensor(), Tensor()};
+    }
+};
+
+Tensor butterfly_multiply_base4(Tensor twiddle4, Tensor twiddle2, Tensor input, bool increasing_stride,
+                                c10::optional<int64_t> output_size)
+{
+    return ButterflyMultiplyBase4::apply(twiddle4, twiddle2, input, increasing_stride, output_size);
+}
+
+int64_t hip_version() { return bf_hip_version(); }
+
+}  // namespace
+
+TORCH_LIBRARY(torch_butterfly, m)
+{
+    m.def("butterfly_multiply_fw", butterfly_multiply_fw);
+    m.def("butterfly_multiply_bw", butterfly_multiply_bw);
+    m.def("butterfly_multiply", butterfly_multiply);
+    m.def("butterfly_multiply_base4_fw", butterfly_multiply_base4_fw);
+    m.def("butterfly_multiply_base4_bw", butterfly_multiply_base4_bw);
+    m.def("butterfly_multiply_base4", butterfly_multiply_base4);
+    m.def("hip_version", hip_version);
+}

@@ -1,0 +1,69 @@
+"""Functional entry points of the base-2 butterfly multiply.
+
+``butterfly_multiply{,_fw,_bw}`` call the registered operators (HIP kernels); they are the
+counterparts of the scripted wrappers in the reference's torch_butterfly/multiply.py:8-25.
+``butterfly_multiply_torch`` is a plain-PyTorch restatement of the same product, kept as a
+differentiable cross-check like the reference's (multiply.py:28-51); nothing dispatches to
+it automatically.
+"""
+from typing import Optional, Tuple
+
+import torch
+
+
+def butterfly_multiply_fw(twiddle: torch.Tensor, input: torch.Tensor, increasing_stride: bool,
+                          output_size: Optional[int] = None) -> torch.Tensor:
+    return torch.ops.torch_butterfly.butterfly_multiply_fw(twiddle, input, increasing_stride,
+                                                           output_size)
+
+
+def butterfly_multiply_bw(twiddle: torch.Tensor, input: torch.Tensor, grad: torch.Tensor,
+                          increasing_stride: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    return torch.ops.torch_butterfly.butterfly_multiply_bw(twiddle, input, grad, increasing_stride)
+
+
+def butterfly_multiply(twiddle: torch.Tensor, input: torch.Tensor, increasing_stride: bool,
+                       output_size: Optional[int] = None) -> torch.Tensor:
+    """twiddle (nstacks, nblocks, log_n, n/2, 2, 2); input (batch, nstacks, input_size), zero
+    padded or trimmed to n; returns (batch, nstacks, output_size or n).  Differentiable."""
+    return torch.ops.torch_butterfly.butterfly_multiply(twiddle, input, increasing_stride,
+                                                        output_size)
+
+
+def fit_last_dim(x: torch.Tensor, n: int) -> torch.Tensor:
+    """Zero-pad or trim the last dimension to exactly ``n``."""
+    size = x.shape[-1]
+    if size == n:
+        return x
+    if size > n:
+        return x[..., :n]
+    return torch.nn.functional.pad(x, (0, n - size))
+
+
+def stage_strides(log_n: int, nblocks: int, increasing_stride: bool):
+    """log2(stride) of every stage, block by block (direction alternates per block)."""
+    out = []
+    for block in range(nblocks):
+        inc = increasing_stride != (block % 2 == 1)
+        out.append([idx if inc else log_n - 1 - idx for idx in range(log_n)])
+    return out
+
+
+def butterfly_multiply_torch(twiddle, input, increasing_stride=True, output_size=None):
+    batch, nstacks, _ = input.shape
+    nblocks, log_n = twiddle.shape[1], twiddle.shape[2]
+    n = 1 << log_n
+    if tuple(twiddle.shape) != (nstacks, nblocks, log_n, n // 2, 2, 2):
+        raise ValueError("twiddle must have shape (nstacks, nblocks, log_n, n / 2, 2, 2)")
+    output_size = n if output_size is None else output_size
+    if output_size > n:
+        raise ValueError("output_size must be <= n")
+    x = fit_last_dim(input, n)
+    for block, strides in enumerate(stage_strides(log_n, nblocks, increasing_stride)):
+        for idx, log_stride in enumerate(strides):
+            st = 1 << log_stride
+            # pair i = h * st + l couples elements (2 h st + l) and (2 h st + st + l)
+            t = twiddle[:, block, idx].reshape(nstacks, n // (2 * st), st, 2, 2)
+            xv = x.reshape(batch, nstacks, n // (2 * st), 2, st)
+            x = torch.einsum("shlrc,bshcl->bshrl", t, xv).reshape(batch, nstacks, n)
+    return x[:, :, :output_size]

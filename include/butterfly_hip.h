@@ -1,0 +1,103 @@
+/*
+ * C ABI of libbutterfly_hip.so -- butterfly matrix multiply on AMD gfx950 (MI355X).
+ *
+ * Every pointer argument named twiddle*, input, grad, output, d_* and workspace is a
+ * DEVICE pointer.  Nothing here allocates or synchronises: the caller supplies the
+ * workspace (size from the *_workspace_bytes query) and the HIP stream (hipStream_t
+ * passed as void*, NULL = the null stream); kernels are enqueued and the call returns.
+ *
+ * Element types: BF_F32 = float; BF_C64 = interleaved (re, im) float pairs, the memory
+ * layout of torch.complex64.  All strides are in ELEMENTS of that type, may be zero
+ * (broadcast stacks) and must be non-negative.  Twiddles are dense row-major.
+ *
+ * Return value: 0 on success, a negative BF_ERR_* code otherwise; bf_last_error()
+ * returns the message for the calling thread.
+ */
+#ifndef BUTTERFLY_HIP_H
+#define BUTTERFLY_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BF_F32 0
+#define BF_C64 1
+
+#define BF_OK 0
+#define BF_ERR_INVALID (-1)     /* bad shape / stride / argument                      */
+#define BF_ERR_UNSUPPORTED (-2) /* valid request the library cannot run (e.g. n too large) */
+#define BF_ERR_HIP (-3)         /* a HIP call or kernel launch failed                 */
+#define BF_ERR_WORKSPACE (-4)   /* workspace missing or too small                     */
+
+/* Problem description shared by all entry points.  Plain data, no ownership. */
+typedef struct bf_problem {
+    int32_t dtype;             /* BF_F32 or BF_C64                                              */
+    int32_t increasing_stride; /* first block multiplies with stride 1,2,..,n/2 (else n/2,..,1) */
+    int64_t batch;             /* B                                                             */
+    int64_t nstacks;           /* S                                                             */
+    int64_t log_n;             /* n = 1 << log_n                                                */
+    int64_t nblocks;           /* nb                                                            */
+    int64_t input_size;        /* I: input is zero-padded / trimmed to n                        */
+    int64_t output_size;       /* O <= n: columns of output (fw) or of grad (bw)                */
+    int64_t input_stride[3];   /* of input  (B, S, I)                                           */
+    int64_t output_stride[3];  /* fw: of output (B, S, O); bw: of grad (B, S, O)                */
+    int64_t d_input_stride[3]; /* bw only: of d_input (B, S, I)                                 */
+} bf_problem;
+
+/* Library version (major * 10000 + minor * 100 + patch). */
+int bf_version(void);
+
+/* HIP runtime version the library was built against (HIP_VERSION).  Stands where the
+ * reference's torch_butterfly::cuda_version reports CUDA_VERSION (csrc/version.cpp:14-23). */
+int bf_hip_version(void);
+
+/* Message describing the last error on this thread ("" if none). */
+const char *bf_last_error(void);
+
+/* Forward multiply: output = (prod of nb * log_n block-diagonal 2x2 stages) pad(input).
+ * Replaces butterfly_multiply_fw_cuda / butterfly_multiply_fw_cpu behind
+ * torch_butterfly::butterfly_multiply_fw (csrc/butterfly.cpp:20-53,
+ * csrc/cpu/butterfly_cpu.cpp:17-66, csrc/cuda/butterfly_cuda.cu:349-416).
+ *   twiddle (S, nb, log_n, n/2, 2, 2) dense.                                          */
+int bf_butterfly_multiply_fw(const bf_problem *p, const void *twiddle, const void *input,
+                             void *output, void *stream);
+
+/* Workspace the backward call needs for this problem, in bytes. */
+size_t bf_butterfly_multiply_bw_workspace_bytes(const bf_problem *p);
+
+/* Backward multiply: d_twiddle (dense, twiddle shape, fully overwritten) and d_input
+ * (B, S, I) with columns >= n zero-filled.  The batch reduction of d_twiddle uses no
+ * atomics: per-workgroup partial sums then a fixed-order second pass, so results are
+ * bitwise reproducible run to run.
+ * Replaces butterfly_multiply_bw_cuda / butterfly_multiply_bw_cpu behind
+ * torch_butterfly::butterfly_multiply_bw (csrc/butterfly.cpp:56-93,
+ * csrc/cpu/butterfly_cpu.cpp:68-177, csrc/cuda/butterfly_cuda.cu:534-646).            */
+int bf_butterfly_multiply_bw(const bf_problem *p, const void *twiddle, const void *input,
+                             const void *grad, void *d_twiddle, void *d_input,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
+/* Base-4 forward: per block log_n/2 radix-4 stages from twiddle4
+ * (S, nb, log_n/2, n/4, 4, 4), then one 2x2 stage from twiddle2 (S, nb, 1, n/2, 2, 2)
+ * when log_n is odd (twiddle2 may be NULL when log_n is even).
+ * Native counterpart of butterfly_multiply_base4_torch
+ * (torch_butterfly/multiply_base4.py:7-41), which the reference runs as PyTorch ops. */
+int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4,
+                                   const void *twiddle2, const void *input, void *output,
+                                   void *stream);
+
+size_t bf_butterfly_multiply_base4_bw_workspace_bytes(const bf_problem *p);
+
+/* Base-4 backward: what autograd derives for multiply_base4.py:7-41.
+ * d_twiddle2 may be NULL when log_n is even.                                          */
+int bf_butterfly_multiply_base4_bw(const bf_problem *p, const void *twiddle4,
+                                   const void *twiddle2, const void *input, const void *grad,
+                                   void *d_twiddle4, void *d_twiddle2, void *d_input,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BUTTERFLY_HIP_H */

@@ -1,0 +1,143 @@
+"""The module layer on the device: Butterfly / ButterflyBase4 as nn.Linear drop-ins and the
+closed-form transforms against library routines (the reference's tests/test_butterfly.py
+and tests/test_special.py are the model)."""
+import math
+import sys
+
+import numpy as np
+import pytest
+import scipy.linalg
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def close(a, b, rtol=1e-3, atol=1e-5):
+    return torch.allclose(a, b, rtol=rtol, atol=atol)
+
+
+def test_butterfly_shapes_and_matrix_flags():
+    import butterfly_amd as bfa
+    for in_size, out_size in [(7, 15), (15, 7)]:
+        for complex_ in (False, True):
+            for nblocks in (1, 2, 3):
+                for inc in (True, False):
+                    say("module", in_size, out_size, complex_, nblocks, inc)
+                    b = bfa.Butterfly(in_size, out_size, True, complex_, inc, "ortho", nblocks).cuda()
+                    dtype = torch.complex64 if complex_ else torch.float32
+                    x = torch.randn(5, 3, in_size, dtype=dtype, device="cuda")
+                    y = b(x)
+                    assert y.shape == (5, 3, out_size)
+                    # dense matrix through the identity (bias removed)
+                    eye = torch.eye(in_size, dtype=dtype, device="cuda")
+                    M = (b(eye) - b.bias).t()                       # (out, in)
+                    assert close(y, x @ M.t() + b.bias, atol=1e-4)
+    # transpose / conjugate flags on a square complex layer
+    n = 16
+    b = bfa.Butterfly(n, n, False, True, True, "randn", 2).cuda()
+    eye = torch.eye(n, dtype=torch.complex64, device="cuda")
+    M = b(eye).t()
+    assert close(b(eye, transpose=True).t(), M.t(), atol=1e-4)
+    assert close(b(eye, conjugate=True).t(), M.conj(), atol=1e-4)
+    assert close(b(eye, transpose=True, conjugate=True).t(), M.t().conj(), atol=1e-4)
+
+
+def test_autograd_through_module_reduces_loss():
+    import butterfly_amd as bfa
+    torch.manual_seed(0)
+    b = bfa.Butterfly(64, 64, True, False, True, "randn", 2).cuda()
+    x = torch.randn(256, 64, device="cuda")
+    target = torch.randn(256, 64, device="cuda")
+    opt = torch.optim.SGD(b.parameters(), lr=1e-2)
+    losses = []
+    for _ in range(20):
+        opt.zero_grad()
+        loss = ((b(x) - target) ** 2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < losses[0]
+
+
+def test_fft_ifft_hadamard_circulant():
+    from butterfly_amd import special
+    torch.manual_seed(1)
+    for n in (2, 8, 256, 4096):
+        say("fft", n)
+        x = torch.randn(3, n, dtype=torch.complex64, device="cuda")
+        for br_first in (True, False):
+            for normalized in (False, True):
+                f = special.fft(n, normalized=normalized, br_first=br_first).cuda()
+                want = torch.fft.fft(x, norm="ortho" if normalized else None)
+                assert close(f(x), want, rtol=1e-3, atol=1e-3 * math.sqrt(n)), (n, br_first, normalized)
+                fi = special.ifft(n, normalized=normalized, br_first=br_first).cuda()
+                want = torch.fft.ifft(x, norm="ortho" if normalized else None)
+                assert close(fi(x), want, rtol=1e-3, atol=1e-4), (n, br_first, normalized)
+    for n in (2, 16, 512):
+        for inc in (True, False):
+            h = special.hadamard(n, increasing_stride=inc).cuda()
+            x = torch.randn(4, n, device="cuda")
+            H = torch.tensor(scipy.linalg.hadamard(n), dtype=torch.float32, device="cuda")
+            assert close(h(x), x @ H.t(), atol=1e-3)
+    for n in (13, 16):
+        for sep in (True, False):
+            for transposed in (False, True):
+                say("circulant", n, sep, transposed)
+                col = torch.randn(n, device="cuda")
+                C = torch.tensor(scipy.linalg.circulant(col.cpu().numpy()), device="cuda")
+                if transposed:
+                    C = C.t()
+                m = special.circulant(col, transposed=transposed, separate_diagonal=sep)
+                x = torch.randn(3, n, device="cuda")
+                assert close(m(x), x @ C.t(), atol=1e-4), (n, sep, transposed)
+    col, row = torch.randn(9, device="cuda"), torch.randn(6, device="cuda")
+    T = torch.tensor(scipy.linalg.toeplitz(col.cpu().numpy(), row.cpu().numpy()), device="cuda")
+    m = special.toeplitz(col, row)
+    x = torch.randn(2, 6, device="cuda")
+    assert close(m(x), x @ T.t(), atol=1e-4)
+
+
+def test_fft_headline_complex_against_torch_fft():
+    """complex64, n = 4096, normalised DFT twiddles, bit reversal outside the operator."""
+    from butterfly_amd import special
+    torch.manual_seed(2)
+    n, B = 4096, 512
+    f = special.fft(n, normalized=True).cuda()
+    x = torch.randn(B, n, dtype=torch.complex64, device="cuda", requires_grad=True)
+    y = f(x)
+    want = torch.fft.fft(x.detach(), norm="ortho")
+    err = (y.detach() - want).abs().max().item() / want.abs().max().item()
+    say("fft 4096 fwd err", err)
+    assert err < 1e-5
+    g = torch.randn_like(want)
+    (dx,) = torch.autograd.grad(y, x, g)
+    # adjoint of the unitary DFT is the inverse DFT
+    want_dx = torch.fft.ifft(g, norm="ortho")
+    err = (dx - want_dx).abs().max().item() / want_dx.abs().max().item()
+    say("fft 4096 bwd err", err)
+    assert err < 1e-4
+
+
+def test_base4_module_equals_base2_module():
+    import butterfly_amd as bfa
+    torch.manual_seed(3)
+    for in_size, out_size, nblocks, complex_ in [(256, 256, 1, False), (100, 300, 2, False), (32, 32, 3, True),
+                                                 (128, 128, 2, True)]:
+        for inc in (True, False):
+            say("base4 module", in_size, out_size, nblocks, complex_, inc)
+            b2 = bfa.Butterfly(in_size, out_size, True, complex_, inc, "randn", nblocks).cuda()
+            b4 = b2.to_base4()
+            assert isinstance(b4, bfa.ButterflyBase4) and not hasattr(b4, "twiddle")
+            dtype = torch.complex64 if complex_ else torch.float32
+            x = torch.randn(9, in_size, dtype=dtype, device="cuda", requires_grad=True)
+            y2, y4 = b2(x), b4(x)
+            assert close(y4, y2, atol=1e-4)
+            g = torch.randn_like(y2)
+            (dx2,) = torch.autograd.grad(y2, x, g)
+            (dx4,) = torch.autograd.grad(y4, x, g)
+            assert close(dx4, dx2, atol=1e-4)

@@ -1,0 +1,219 @@
+"""Parity of the HIP library (through its C ABI and through the registered operators)
+against the CPU oracle.  Tolerances are max|err| / max|ref|: 1e-5 forward, 1e-4 gradients."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import randn, rel_err
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+FW_TOL = 1e-5
+BW_TOL = 1e-4
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def make_case(rng, dtype, B, S, L, nb, I=None, O=None):
+    n = 1 << L
+    I = n if I is None else I
+    tw = (randn(rng, (S, nb, L, n // 2, 2, 2), dtype) / np.sqrt(2)).astype(dtype)
+    x = randn(rng, (B, S, I), dtype)
+    g = randn(rng, (B, S, n if O is None else O), dtype)
+    return tw, x, g
+
+
+CASES = [
+    # dtype, B, S, L, nb, I, O, inc
+    (np.float32, 7, 1, 1, 1, None, None, True),
+    (np.float32, 5, 2, 2, 3, None, None, False),
+    (np.float32, 33, 2, 5, 3, 15, None, True),
+    (np.float32, 10, 2, 5, 3, 28, 14, False),
+    (np.float32, 10, 2, 5, 2, 71, 27, True),
+    (np.float32, 64, 1, 10, 1, None, None, True),
+    (np.float32, 50, 1, 10, 2, None, None, False),
+    (np.float32, 10, 2, 12, 3, None, None, True),
+    (np.float32, 10, 2, 12, 3, 4092, 2046, False),
+    (np.float32, 3, 1, 14, 1, None, None, False),
+    (np.complex64, 9, 2, 3, 2, None, None, True),
+    (np.complex64, 10, 2, 5, 3, 2 * 32 + 7, 32 - 5, False),
+    (np.complex64, 40, 1, 9, 2, None, None, False),
+    (np.complex64, 10, 2, 12, 3, None, None, True),
+    (np.complex64, 6, 1, 12, 1, 2047, None, False),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: f"{np.dtype(c[0]).name}-B{c[1]}-S{c[2]}-L{c[3]}-nb{c[4]}-I{c[5]}-O{c[6]}-inc{int(c[7])}")
+def test_c_abi_matches_oracle(case):
+    from butterfly_amd import _capi
+    dtype, B, S, L, nb, I, O, inc = case
+    say("case", case)
+    rng = np.random.default_rng(hash((L, nb, B, S)) % (1 << 31))
+    tw, x, g = make_case(rng, dtype, B, S, L, nb, I, O)
+    y_ref = oracle.butterfly_fw(tw, x, inc, O)
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+    y = _capi.multiply_fw(dev(tw), dev(x), inc, O)
+    dtw, dx = _capi.multiply_bw(dev(tw), dev(x), dev(g), inc)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
+def test_c_abi_strided_operands():
+    """Stride-0 stack broadcast (what Butterfly.pre_process hands over), a transposed input
+    and a non-contiguous gradient."""
+    from butterfly_amd import _capi
+    rng = np.random.default_rng(11)
+    B, S, L, nb = 12, 3, 6, 2
+    n = 1 << L
+    tw = (randn(rng, (S, nb, L, n // 2, 2, 2), np.float32) / np.sqrt(2)).astype(np.float32)
+    x1 = randn(rng, (B, n), np.float32)
+    x_np = np.broadcast_to(x1[:, None, :], (B, S, n))
+    g_big = randn(rng, (B, S, 2 * n), np.float32)
+    x_dev = dev(x1).unsqueeze(1).expand(B, S, n)
+    g_dev = dev(g_big)[:, :, ::2]
+    say("strided: expand + strided grad")
+    y = _capi.multiply_fw(dev(tw), x_dev, True)
+    dtw, dx = _capi.multiply_bw(dev(tw), x_dev, g_dev, True)
+    y_ref = oracle.butterfly_fw(tw, x_np, True)
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x_np, g_big[:, :, ::2], True)
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+    say("strided: transposed input")
+    xt = dev(np.ascontiguousarray(x_np.transpose(2, 0, 1))).permute(1, 2, 0)
+    assert not xt.is_contiguous()
+    y2 = _capi.multiply_fw(dev(tw), xt, True)
+    assert torch.equal(y2, y)
+
+
+BASE4_CASES = [
+    (np.float32, 9, 2, 2, 1, None, None, True),
+    (np.float32, 9, 2, 3, 2, None, None, False),
+    (np.float32, 20, 4, 8, 1, None, None, True),
+    (np.float32, 11, 2, 7, 3, 100, 90, False),
+    (np.float32, 6, 1, 11, 2, None, None, True),
+    (np.complex64, 7, 2, 5, 2, 40, 17, True),
+    (np.complex64, 5, 1, 10, 2, None, None, False),
+    (np.float32, 5, 2, 1, 2, None, None, True),
+]
+
+
+@pytest.mark.parametrize("case", BASE4_CASES, ids=lambda c: f"{np.dtype(c[0]).name}-B{c[1]}-S{c[2]}-L{c[3]}-nb{c[4]}-I{c[5]}-O{c[6]}-inc{int(c[7])}")
+def test_c_abi_base4_matches_oracle(case):
+    from butterfly_amd import _capi
+    dtype, B, S, L, nb, I, O, inc = case
+    say("base4 case", case)
+    rng = np.random.default_rng(100 + L * 7 + nb)
+    n = 1 << L
+    I_ = n if I is None else I
+    tw4 = (randn(rng, (S, nb, L // 2, n // 4, 4, 4), dtype) / 2).astype(dtype)
+    tw2 = (randn(rng, (S, nb, L % 2, n // 2, 2, 2), dtype) / np.sqrt(2)).astype(dtype)
+    x = randn(rng, (B, S, I_), dtype)
+    g = randn(rng, (B, S, n if O is None else O), dtype)
+    y_ref = oracle.butterfly_base4_fw(tw4, tw2, x, inc, O)
+    d4_ref, d2_ref, dx_ref = oracle.butterfly_base4_bw(tw4, tw2, x, g, inc)
+    y = _capi.multiply_base4_fw(dev(tw4), dev(tw2), dev(x), inc, O)
+    d4, d2, dx = _capi.multiply_base4_bw(dev(tw4), dev(tw2), dev(x), dev(g), inc)
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(d4.cpu().numpy(), d4_ref) < BW_TOL
+    assert rel_err(d2.cpu().numpy(), d2_ref) < BW_TOL
+
+
+def test_operators_match_oracle_and_autograd():
+    """torch.ops.torch_butterfly.* end to end: views returned, autograd wired, lazy conj
+    and transposed twiddle views accepted."""
+    import butterfly_amd  # noqa: F401  (registers the operators)
+    rng = np.random.default_rng(21)
+    for dtype in (np.float32, np.complex64):
+        B, S, L, nb, I, O = 6, 2, 5, 3, 29, 20
+        n = 1 << L
+        tw, x, g = make_case(rng, dtype, B, S, L, nb, I, O)
+        say("ops", np.dtype(dtype).name)
+        twd = dev(tw).requires_grad_()
+        xd = dev(x).requires_grad_()
+        y = torch.ops.torch_butterfly.butterfly_multiply(twd, xd, False, O)
+        assert y.shape == (B, S, O) and y.stride() == (S * n, n, 1)   # a view of an n-wide buffer
+        dtw, dx = torch.autograd.grad(y, (twd, xd), dev(g))
+        y_ref = oracle.butterfly_fw(tw, x, False, O)
+        dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, False)
+        assert rel_err(y.detach().cpu().numpy(), y_ref) < FW_TOL
+        assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+        assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+        # transposed + flipped (+ conjugated) twiddle view, as Butterfly.forward(transpose=True) builds
+        tv = dev(tw).transpose(-1, -2).flip([1, 2])
+        tv_np = np.ascontiguousarray(np.flip(np.swapaxes(tw, -1, -2), (1, 2)))
+        if np.dtype(dtype).kind == "c":
+            tv, tv_np = tv.conj(), tv_np.conj()
+        y2 = torch.ops.torch_butterfly.butterfly_multiply_fw(tv, dev(x), True, None)
+        assert rel_err(y2.cpu().numpy(), oracle.butterfly_fw(tv_np, x, True)) < FW_TOL
+
+
+def test_operator_errors():
+    import butterfly_amd  # noqa: F401
+    ops = torch.ops.torch_butterfly
+    tw = torch.randn(1, 1, 3, 4, 2, 2, device="cuda")
+    x = torch.randn(2, 1, 8, device="cuda")
+    with pytest.raises(RuntimeError, match="must have shape"):
+        ops.butterfly_multiply_fw(tw[:, :, :, :3], x, True, None)
+    with pytest.raises(RuntimeError, match="output_size must be <= n"):
+        ops.butterfly_multiply_fw(tw, x, True, 9)
+    with pytest.raises(RuntimeError, match="same device"):
+        ops.butterfly_multiply_fw(tw.cpu(), x, True, None)
+    with pytest.raises(RuntimeError, match="float32 and complex64"):
+        ops.butterfly_multiply_fw(tw.double(), x.double(), True, None)
+    with pytest.raises(RuntimeError, match="must have dimension"):
+        ops.butterfly_multiply_bw(tw, x, torch.randn(2, 8, device="cuda"), True)
+
+
+def test_backward_is_bitwise_reproducible():
+    """No atomics in the d_twiddle reduction: two runs give identical bits."""
+    from butterfly_amd import _capi
+    rng = np.random.default_rng(31)
+    tw, x, g = make_case(rng, np.float32, 4096, 1, 10, 2)
+    twd, xd, gd = dev(tw), dev(x), dev(g)
+    say("determinism")
+    a = _capi.multiply_bw(twd, xd, gd, False)
+    b = _capi.multiply_bw(twd, xd, gd, False)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_headline_size_properties():
+    """Batch 16384, n = 1024, nblocks = 2, decreasing stride first.  Too big for the scalar
+    oracle in seconds, so: (i) a 512-row slice against the oracle, (ii) linearity in the
+    batch (rows are independent), (iii) the adjoint identity <y, g> = <x, d_input>,
+    (iv) d_twiddle equals the sum of d_twiddle over batch chunks."""
+    from butterfly_amd import _capi
+    rng = np.random.default_rng(41)
+    B, L, nb = 16384, 10, 2
+    tw, x, g = make_case(rng, np.float32, B, 1, L, nb)
+    twd, xd, gd = dev(tw), dev(x), dev(g)
+    say("headline fw")
+    y = _capi.multiply_fw(twd, xd, False)
+    say("headline bw")
+    dtw, dx = _capi.multiply_bw(twd, xd, gd, False)
+    torch.cuda.synchronize()
+    sl = slice(7000, 7512)
+    assert rel_err(y[sl].cpu().numpy(), oracle.butterfly_fw(tw, x[sl], False)) < FW_TOL
+    _, dx_ref = oracle.butterfly_bw(tw, x[sl], g[sl], False)
+    assert rel_err(dx[sl].cpu().numpy(), dx_ref) < BW_TOL
+    lhs = torch.sum(y.double() * gd.double()).item()
+    rhs = torch.sum(xd.double() * dx.double()).item()
+    assert abs(lhs - rhs) < 1e-5 * abs(lhs) + 1e-2
+    parts = [_capi.multiply_bw(twd, xd[i:i + 4096], gd[i:i + 4096], False)[0].double() for i in range(0, B, 4096)]
+    assert rel_err(dtw.cpu().numpy(), sum(parts).cpu().numpy()) < BW_TOL
+    dtw_ref, _ = oracle.butterfly_bw(tw, x[:1024], g[:1024], False)
+    dtw_small, _ = _capi.multiply_bw(twd, xd[:1024], gd[:1024], False)
+    assert rel_err(dtw_small.cpu().numpy(), dtw_ref) < BW_TOL

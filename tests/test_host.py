@@ -1,0 +1,200 @@
+"""CPU-only checks: the C ABI library loads and exports what the header declares, argument
+validation, host-side twiddle algebra and module bookkeeping.  No kernel is launched."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, randn, rel_err
+from oracle import oracle
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "butterfly_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from butterfly_amd import _capi
+    names = header_functions()
+    assert len(names) >= 9
+    assert sorted(_capi.SYMBOLS) == names
+    L = _capi.lib()
+    for name in names:
+        assert hasattr(L, name), name
+    assert L.bf_version() >= 100
+    assert L.bf_hip_version() > 0
+
+
+def test_c_abi_rejects_bad_problems_on_the_host():
+    from butterfly_amd import _capi
+    L = _capi.lib()
+    p = _capi.Problem()
+    p.dtype, p.batch, p.nstacks, p.log_n, p.nblocks = 7, 1, 1, 3, 1
+    p.input_size = p.output_size = 8
+    null = ctypes.c_void_p(0)
+    assert L.bf_butterfly_multiply_fw(ctypes.byref(p), null, null, null, null) == -1
+    assert b"dtype" in L.bf_last_error()
+    p.dtype, p.output_size = 0, 9
+    assert L.bf_butterfly_multiply_fw(ctypes.byref(p), null, null, null, null) == -1
+    assert b"output_size" in L.bf_last_error()
+    p.output_size, p.log_n = 8, 31
+    assert L.bf_butterfly_multiply_fw(ctypes.byref(p), null, null, null, null) == -1
+    p.log_n = 3
+    p.input_stride[2] = -1
+    assert L.bf_butterfly_multiply_bw(ctypes.byref(p), null, null, null, null, null, null, 0, null) == -1
+    assert L.bf_butterfly_multiply_fw(None, null, null, null, null) == -1
+    # workspace query is pure host arithmetic
+    p.input_stride[2] = 1
+    p.batch, p.log_n, p.nblocks = 16384, 10, 2
+    assert L.bf_butterfly_multiply_bw_workspace_bytes(ctypes.byref(p)) > 0
+
+
+def test_operator_schemas_and_host_side_checks():
+    import butterfly_amd  # noqa: F401
+    ops = torch.ops.torch_butterfly
+    assert str(ops.butterfly_multiply_fw.default._schema) == \
+        "torch_butterfly::butterfly_multiply_fw(Tensor _0, Tensor _1, bool _2, int? _3) -> Tensor _0"
+    assert str(ops.butterfly_multiply_bw.default._schema) == \
+        "torch_butterfly::butterfly_multiply_bw(Tensor _0, Tensor _1, Tensor _2, bool _3) -> (Tensor _0, Tensor _1)"
+    assert str(ops.butterfly_multiply.default._schema) == \
+        "torch_butterfly::butterfly_multiply(Tensor _0, Tensor _1, bool _2, int? _3) -> Tensor _0"
+    assert ops.cuda_version() == -1 and ops.hip_version() > 0
+    tw, x = torch.randn(1, 1, 3, 4, 2, 2), torch.randn(2, 1, 8)
+    with pytest.raises(RuntimeError, match="must have shape"):
+        ops.butterfly_multiply_fw(tw[:, :, :2], x, True, None)
+    with pytest.raises(RuntimeError, match="output_size must be <= n"):
+        ops.butterfly_multiply_fw(tw, x, True, 9)
+    with pytest.raises(RuntimeError, match="must have dimension"):
+        ops.butterfly_multiply_fw(tw, x[0], True, None)
+    # there is no CPU path: CPU tensors are refused, loudly
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.butterfly_multiply_fw(tw, x, True, None)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.butterfly_multiply_bw(tw, x, x.clone(), True)
+    # the wrappers are TorchScript-callable like the reference's scripted functions
+    @torch.jit.script
+    def scripted(t: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+        return torch.ops.torch_butterfly.butterfly_multiply(t, v, True, None)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        scripted(tw, x)
+
+
+@pytest.mark.parametrize("inc", [True, False])
+def test_twiddle_base2_to_base4_host(inc):
+    from butterfly_amd.multiply_base4 import butterfly_multiply_base4_torch, twiddle_base2_to_base4
+    from butterfly_amd.multiply import butterfly_multiply_torch
+    rng = np.random.default_rng(0)
+    for L in (1, 2, 3, 4, 5, 6):
+        for nb in (1, 2, 3):
+            n = 1 << L
+            dtype = np.complex128 if L % 2 else np.float64
+            tw = randn(rng, (2, nb, L, n // 2, 2, 2), dtype)
+            t4, t2 = twiddle_base2_to_base4(torch.from_numpy(tw), inc)
+            o4, o2 = oracle.twiddle_base2_to_base4(tw, inc)
+            assert t2.shape == o2.shape and rel_err(t4.numpy(), o4) < 1e-12
+            if L % 2:
+                assert np.array_equal(t2.numpy(), o2)
+            x = randn(rng, (3, 2, n - 1 if n > 2 else n), dtype)
+            y2 = butterfly_multiply_torch(torch.from_numpy(tw), torch.from_numpy(x), inc)
+            y4 = butterfly_multiply_base4_torch(t4, t2, torch.from_numpy(x), inc)
+            assert rel_err(y4.numpy(), y2.numpy()) < 1e-12
+            assert rel_err(y2.numpy(), oracle.butterfly_fw(tw, x, inc)) < 1e-12
+            assert rel_err(y4.numpy(), oracle.butterfly_base4_fw(o4, o2, x, inc)) < 1e-12
+
+
+def test_torch_restatement_gradients_match_oracle():
+    from butterfly_amd.multiply import butterfly_multiply_torch
+    from butterfly_amd.multiply_base4 import butterfly_multiply_base4_torch
+    rng = np.random.default_rng(1)
+    for dtype in (np.float64, np.complex128):
+        L, nb, B, S = 5, 2, 4, 2
+        n = 1 << L
+        tw = randn(rng, (S, nb, L, n // 2, 2, 2), dtype)
+        x = randn(rng, (B, S, n - 3), dtype)
+        g = randn(rng, (B, S, n - 5), dtype)
+        t, xx = torch.from_numpy(tw).requires_grad_(), torch.from_numpy(x).requires_grad_()
+        y = butterfly_multiply_torch(t, xx, False, n - 5)
+        dt, dx = torch.autograd.grad(y, (t, xx), torch.from_numpy(g))
+        dt_ref, dx_ref = oracle.butterfly_bw(tw, x, g, False)
+        assert rel_err(dt.numpy(), dt_ref) < 1e-12 and rel_err(dx.numpy(), dx_ref) < 1e-12
+        tw4 = randn(rng, (S, nb, L // 2, n // 4, 4, 4), dtype)
+        tw2 = randn(rng, (S, nb, L % 2, n // 2, 2, 2), dtype)
+        t4, t2 = torch.from_numpy(tw4).requires_grad_(), torch.from_numpy(tw2).requires_grad_()
+        y = butterfly_multiply_base4_torch(t4, t2, xx, True, n - 5)
+        d4, d2, dx = torch.autograd.grad(y, (t4, t2, xx), torch.from_numpy(g))
+        d4_ref, d2_ref, dx_ref = oracle.butterfly_base4_bw(tw4, tw2, x, g, True)
+        assert rel_err(d4.numpy(), d4_ref) < 1e-12 and rel_err(d2.numpy(), d2_ref) < 1e-12
+        assert rel_err(dx.numpy(), dx_ref) < 1e-12
+
+
+def apply_cpu(b, x):
+    """Evaluate a Butterfly module's matrix on the CPU through the oracle (host-logic check
+    of the twiddle a constructor produced; the module's own forward needs the device)."""
+    xs = np.broadcast_to(x[:, None, :], (x.shape[0], b.nstacks, x.shape[1]))
+    tw = b.twiddle.detach().numpy()
+    y = oracle.butterfly_fw(tw, xs.astype(tw.dtype), b.increasing_stride, b.out_size if b.nstacks == 1 else None)
+    return y.reshape(x.shape[0], -1)[:, :b.out_size]
+
+
+def test_special_twiddles_on_the_host():
+    import scipy.linalg
+    from butterfly_amd import special
+    from butterfly_amd.permutation import bitreversal_permutation
+    rng = np.random.default_rng(2)
+    for n in (2, 16, 128):
+        br = bitreversal_permutation(n)
+        assert sorted(br) == list(range(n)) and np.array_equal(br[br], np.arange(n))
+        x = randn(rng, (3, n), np.complex64)
+        for normalized in (False, True):
+            f = special.fft(n, normalized=normalized, br_first=True, with_br_perm=False)
+            want = np.fft.fft(x, norm="ortho" if normalized else None)
+            assert rel_err(apply_cpu(f, x[:, br]), want) < 1e-5
+            f = special.fft(n, normalized=normalized, br_first=False, with_br_perm=False)
+            assert not f.increasing_stride
+            assert rel_err(apply_cpu(f, x)[:, br], want) < 1e-5
+            fi = special.ifft(n, normalized=normalized, br_first=True, with_br_perm=False)
+            want = np.fft.ifft(x, norm="ortho" if normalized else None)
+            assert rel_err(apply_cpu(fi, x[:, br]), want) < 1e-5
+        h = special.hadamard(n, normalized=False, increasing_stride=False)
+        xr = randn(rng, (3, n), np.float32)
+        assert rel_err(apply_cpu(h, xr), xr @ scipy.linalg.hadamard(n).T.astype(np.float32)) < 1e-5
+    # circulant with the diagonal folded in: one Butterfly with two blocks
+    col = torch.from_numpy(randn(rng, (16,), np.complex64))
+    b = special.circulant(col, separate_diagonal=False)
+    assert b.nblocks == 2 and b.twiddle.shape == (1, 2, 4, 8, 2, 2)
+    x = randn(rng, (3, 16), np.complex64)
+    assert rel_err(apply_cpu(b, x), x @ scipy.linalg.circulant(col.numpy()).T) < 1e-5
+
+
+def test_module_bookkeeping():
+    import butterfly_amd as bfa
+    torch.manual_seed(0)
+    b = bfa.Butterfly(7, 15, nblocks=2)
+    assert (b.log_n, b.n, b.nstacks) == (3, 8, 2)
+    assert list(b.state_dict().keys()) == ["twiddle", "bias"]
+    assert b.twiddle.shape == (2, 2, 3, 4, 2, 2) and b.bias.shape == (15,)
+    assert b.twiddle._is_structured
+    assert b.bias.abs().max() <= 1 / np.sqrt(7)
+    for complex_ in (False, True):
+        o = bfa.Butterfly(64, 64, complex=complex_, init="ortho", nblocks=3)
+        sv = torch.linalg.svdvals(o.twiddle.detach().reshape(-1, 2, 2))
+        assert torch.allclose(sv, torch.ones_like(sv), atol=1e-5)
+    e = bfa.Butterfly(16, 16, init="identity", bias=False)
+    x = np.random.default_rng(0).standard_normal((2, 16)).astype(np.float32)
+    assert np.array_equal(apply_cpu(e, x), x)
+    f = bfa.Butterfly(16, 16, complex=True, init="fft_no_br", nblocks=2, bias=False)
+    assert torch.equal(f.twiddle[:, 1], torch.eye(2, dtype=torch.complex64).expand(1, 4, 8, 2, 2))
+    b4 = bfa.ButterflyBase4(32, 32, nblocks=2)
+    assert sorted(b4.state_dict().keys()) == ["bias", "twiddle2", "twiddle4"]
+    assert b4.twiddle4.shape == (1, 2, 2, 8, 4, 4) and b4.twiddle2.shape == (1, 2, 1, 16, 2, 2)
+    before = b.twiddle.detach().clone()
+    with torch.no_grad():
+        b *= 2.0
+    assert torch.allclose(b.twiddle, before * 2.0 ** (1 / 6))
+    with pytest.raises(ValueError):
+        bfa.Butterfly(8, 8, init=torch.zeros(3))
