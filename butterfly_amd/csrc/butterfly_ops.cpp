@@ -9,8 +9,8 @@
 // Device tensors only: there is deliberately no CPU path behind these operators.
 
 #include <ATen/ATen.h>
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/csrc/autograd/custom_function.h>
 #include <torch/library.h>
 
@@ -47,6 +47,10 @@ void set_strides(int64_t dst[3], const Tensor &t)
     for (int i = 0; i < 3; ++i) dst[i] = t.size(i) > 1 ? t.stride(i) : 0;
     for (int i = 0; i < 3; ++i) TORCH_CHECK(dst[i] >= 0, "negative strides are not supported");
 }
+
+// PyTorch on ROCm presents HIP devices under the "cuda" device type; these are the stream
+// and guard types that go with that.
+void *current_stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
 
 void check_rc(int rc, const char *who) { TORCH_CHECK(rc == BF_OK, who, ": ", bf_last_error()); }
 
@@ -96,7 +100,7 @@ Tensor butterfly_multiply_fw(const Tensor twiddle, const Tensor input, bool incr
     TORCH_CHECK(twiddle.scalar_type() == input.scalar_type(),
                 "butterfly_multiply_fw: twiddle and input must have the same dtype");
 
-    const c10::hip::HIPGuard guard(input.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const Tensor tw = dense(twiddle);
     const Tensor x = input.resolve_conj();
     Tensor output = at::empty({s.batch, s.nstacks, s.n}, x.options());
@@ -104,7 +108,7 @@ Tensor butterfly_multiply_fw(const Tensor twiddle, const Tensor input, bool incr
     bf_problem p = make_problem(s, x, increasing_stride, output_size_val, "butterfly_multiply_fw");
     set_strides(p.output_stride, output);
     check_rc(bf_butterfly_multiply_fw(&p, tw.data_ptr(), x.data_ptr(), output.data_ptr(),
-                                      c10::hip::getCurrentHIPStream().stream()),
+                                      current_stream()),
              "butterfly_multiply_fw");
     return output;
 }
@@ -131,7 +135,7 @@ std::tuple<Tensor, Tensor> butterfly_multiply_bw(const Tensor twiddle, const Ten
     TORCH_CHECK(twiddle.scalar_type() == input.scalar_type() && grad.scalar_type() == input.scalar_type(),
                 "butterfly_multiply_bw: twiddle, input and grad must have the same dtype");
 
-    const c10::hip::HIPGuard guard(input.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const Tensor tw = dense(twiddle);
     const Tensor x = input.resolve_conj();
     const Tensor g = grad.resolve_conj();
@@ -145,7 +149,7 @@ std::tuple<Tensor, Tensor> butterfly_multiply_bw(const Tensor twiddle, const Ten
     Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
     check_rc(bf_butterfly_multiply_bw(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), d_twiddle.data_ptr(),
                                       d_input.data_ptr(), ws.data_ptr(), ws_bytes,
-                                      c10::hip::getCurrentHIPStream().stream()),
+                                      current_stream()),
              "butterfly_multiply_bw");
     return std::make_tuple(d_twiddle, d_input);
 }
@@ -209,7 +213,7 @@ Tensor butterfly_multiply_base4_fw(const Tensor twiddle4, const Tensor twiddle2,
     const int64_t output_size_val = output_size.has_value() ? output_size.value() : s.n;
     TORCH_CHECK(output_size_val <= s.n, "butterfly_multiply_base4_fw: output_size must be <= n");
     TORCH_CHECK(output_size_val >= 0, "butterfly_multiply_base4_fw: output_size must be >= 0");
-    const c10::hip::HIPGuard guard(input.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const Tensor tw4 = dense(twiddle4), tw2 = dense(twiddle2);
     const Tensor x = input.resolve_conj();
     Tensor output = at::empty({s.batch, s.nstacks, s.n}, x.options());
@@ -217,7 +221,7 @@ Tensor butterfly_multiply_base4_fw(const Tensor twiddle4, const Tensor twiddle2,
     bf_problem p = make_problem(s, x, increasing_stride, output_size_val, "butterfly_multiply_base4_fw");
     set_strides(p.output_stride, output);
     check_rc(bf_butterfly_multiply_base4_fw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(),
-                                            output.data_ptr(), c10::hip::getCurrentHIPStream().stream()),
+                                            output.data_ptr(), current_stream()),
              "butterfly_multiply_base4_fw");
     return output;
 }
@@ -233,7 +237,7 @@ std::tuple<Tensor, Tensor, Tensor> butterfly_multiply_base4_bw(const Tensor twid
     TORCH_CHECK(output_size <= s.n, "butterfly_multiply_base4_bw: grad must have at most n columns");
     TORCH_CHECK(grad.scalar_type() == input.scalar_type(),
                 "butterfly_multiply_base4_bw: grad and input must have the same dtype");
-    const c10::hip::HIPGuard guard(input.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const Tensor tw4 = dense(twiddle4), tw2 = dense(twiddle2);
     const Tensor x = input.resolve_conj();
     const Tensor g = grad.resolve_conj();
@@ -248,7 +252,7 @@ std::tuple<Tensor, Tensor, Tensor> butterfly_multiply_base4_bw(const Tensor twid
     Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
     check_rc(bf_butterfly_multiply_base4_bw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(), g.data_ptr(),
                                             d4.data_ptr(), d2.data_ptr(), d_input.data_ptr(), ws.data_ptr(),
-                                            ws_bytes, c10::hip::getCurrentHIPStream().stream()),
+                                            ws_bytes, current_stream()),
              "butterfly_multiply_base4_bw");
     return std::make_tuple(d4, d2, d_input);
 }
