@@ -14,6 +14,7 @@
 
 #include "common.hpp"
 #include "generic.hpp"
+#include "fast.hpp"
 
 namespace {
 
@@ -134,6 +135,84 @@ int ensure_attributes()
     return BF_OK;
 }
 
+// ---- twiddle-stationary fast path (float, base-2, n <= 1024, nblocks <= 2) ------------------
+
+constexpr int kNumCU = 256;     // MI355X
+constexpr int kFastFwRows = 4;  // row groups in flight per forward workgroup
+
+bool fast_applicable(const bf_problem *p, bool base4)
+{
+    return !base4 && p->dtype == BF_F32 && p->log_n >= 1 && p->log_n <= 10 && p->nblocks >= 1 &&
+           p->nblocks <= 2 && p->batch > 0 && p->nstacks > 0;
+}
+
+struct FastGrid {
+    int64_t slots, ngroups, nwg, groups_per_wg;
+};
+
+FastGrid fast_grid(const bf_problem *p, int rows_in_flight, int wg_per_cu)
+{
+    FastGrid g;
+    g.slots = 1024 >> p->log_n;
+    g.ngroups = (p->batch + g.slots - 1) / g.slots;
+    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * wg_per_cu / p->nstacks);
+    const int64_t iters = (g.ngroups + rows_in_flight - 1) / rows_in_flight;
+    g.nwg = std::min(want, iters);
+    g.groups_per_wg = ((iters + g.nwg - 1) / g.nwg) * rows_in_flight;
+    g.nwg = (g.ngroups + g.groups_per_wg - 1) / g.groups_per_wg;
+    return g;
+}
+
+template <int L, int NB, bool INC>
+void launch_fast_fw_t(const FastFwArgs &a, dim3 grid, hipStream_t stream)
+{
+    hipLaunchKernelGGL((fast_fw_kernel<L, NB, INC, kFastFwRows>), grid, dim3(kFastThreads), 0, stream, a);
+}
+
+template <int L, int NB, bool INC>
+void launch_fast_bw_t(const FastBwArgs &a, dim3 grid, hipStream_t stream)
+{
+    hipLaunchKernelGGL((fast_bw_kernel<L, NB, INC>), grid, dim3(kFastThreads), 0, stream, a);
+}
+
+#define BF_FAST_DISPATCH(FN, ...)                                                        \
+    do {                                                                                 \
+        const int key_ = (int)p->log_n * 4 + ((int)p->nblocks - 1) * 2 + (p->increasing_stride ? 1 : 0); \
+        switch (key_) {                                                                  \
+            BF_FAST_CASES(FN, 1, __VA_ARGS__) BF_FAST_CASES(FN, 2, __VA_ARGS__)          \
+            BF_FAST_CASES(FN, 3, __VA_ARGS__) BF_FAST_CASES(FN, 4, __VA_ARGS__)          \
+            BF_FAST_CASES(FN, 5, __VA_ARGS__) BF_FAST_CASES(FN, 6, __VA_ARGS__)          \
+            BF_FAST_CASES(FN, 7, __VA_ARGS__) BF_FAST_CASES(FN, 8, __VA_ARGS__)          \
+            BF_FAST_CASES(FN, 9, __VA_ARGS__) BF_FAST_CASES(FN, 10, __VA_ARGS__)         \
+            default: return fail(BF_ERR_UNSUPPORTED, "no fast kernel for this shape");   \
+        }                                                                                \
+    } while (0)
+#define BF_FAST_CASES(FN, LL, ...)                              \
+    case LL * 4 + 0: FN<LL, 1, false>(__VA_ARGS__); break;      \
+    case LL * 4 + 1: FN<LL, 1, true>(__VA_ARGS__); break;       \
+    case LL * 4 + 2: FN<LL, 2, false>(__VA_ARGS__); break;      \
+    case LL * 4 + 3: FN<LL, 2, true>(__VA_ARGS__); break;
+
+int fast_forward(const bf_problem *p, const void *tw, const void *input, void *output, hipStream_t stream)
+{
+    const int64_t n = (int64_t)1 << p->log_n;
+    const FastGrid g = fast_grid(p, kFastFwRows, 1);
+    FastFwArgs a;
+    a.tw = static_cast<const float *>(tw);
+    a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
+    a.in = static_cast<const float *>(input);
+    a.in_view = make_view(p->input_stride, std::min(p->input_size, n));
+    a.out = static_cast<float *>(output);
+    a.out_view = make_view(p->output_stride, p->output_size);
+    a.batch = p->batch;
+    a.ngroups = g.ngroups;
+    a.groups_per_wg = g.groups_per_wg;
+    const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks);
+    BF_FAST_DISPATCH(launch_fast_fw_t, a, grid, stream);
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
+}
+
 // ---- generic forward ----------------------------------------------------------------------
 
 int launch_generic_fw(const bf_problem *p, const Schedule &sc, int t0, int t1, const void *tw2,
@@ -191,6 +270,7 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
             if (base4 && (p->log_n & 1) && !tw2) return fail(BF_ERR_INVALID, "twiddle2 is NULL");
         }
     }
+    if (fast_applicable(p, base4)) return fast_forward(p, tw2, input, output, stream);
     const View in_view = make_view(p->input_stride, std::min(p->input_size, n));
     const View out_view = make_view(p->output_stride, p->output_size);
     return launch_generic_fw(p, sc, 0, sc.per * sc.nblocks, tw2, tw4, input, in_view, output,
@@ -208,6 +288,7 @@ struct BwPlan {
     size_t boundary_bytes;  // one (B, S, n) activation plane
     size_t off_boundaries, off_gbuf, off_partials, total;
     bool fits;
+    bool fast;          // single launch of the twiddle-stationary kernel
 };
 
 BwPlan plan_bw(const bf_problem *p, bool base4)
@@ -218,6 +299,19 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
     const size_t row_bytes = (size_t)n * e;
     const Schedule sc = make_schedule(p, base4);
     pl.nstages = sc.per * sc.nblocks;
+    if (fast_applicable(p, base4)) {
+        // one launch; partial sums from every (workgroup, row slot)
+        const FastGrid g = fast_grid(p, 1, 1);
+        pl.fits = true;
+        pl.fast = true;
+        pl.nchunks = 1;
+        pl.chunk = pl.nstages;
+        pl.nparts = g.nwg * g.slots;
+        pl.slot = 2 * n;
+        pl.off_partials = 0;
+        pl.total = align256((size_t)pl.nparts * p->nstacks * pl.nstages * pl.slot * e);
+        return pl;
+    }
     pl.fits = 2 * row_bytes <= kGenericBwLds;
     if (!pl.fits) return pl;
     const int cmax = (int)(kGenericBwLds / row_bytes) - 1;
@@ -291,6 +385,40 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     char *ws = static_cast<char *>(workspace);
 
     if (pl.nstages == 0) return launch_copy_pad(p, grad, g_view, d_input, di_view, stream);
+
+    if (pl.fast) {
+        const FastGrid g = fast_grid(p, 1, 1);
+        FastBwArgs a;
+        a.tw = static_cast<const float *>(tw2);
+        a.tw_stack_stride = sc.tw2_stack_stride;
+        a.x_in = static_cast<const float *>(input);
+        a.x_view = x_view;
+        a.g_out = static_cast<const float *>(grad);
+        a.g_view = g_view;
+        a.g_in = static_cast<float *>(d_input);
+        a.gi_view = di_view;
+        a.partial = reinterpret_cast<float *>(ws + pl.off_partials);
+        a.batch = p->batch;
+        a.ngroups = g.ngroups;
+        a.groups_per_wg = g.groups_per_wg;
+        const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks);
+        BF_FAST_DISPATCH(launch_fast_bw_t, a, grid, stream);
+        BF_HIP_CHECK(hipGetLastError());
+        ReduceArgs r;
+        r.sc = sc;
+        r.t0 = 0;
+        r.t1 = pl.nstages;
+        r.nparts = (int)pl.nparts;
+        r.nstacks = p->nstacks;
+        r.partial = ws + pl.off_partials;
+        r.slot = pl.slot;
+        r.d_tw2 = d_tw2;
+        r.d_tw4 = d_tw4;
+        const dim3 rgrid((unsigned)((pl.slot + 255) / 256), (unsigned)pl.nstages, (unsigned)p->nstacks);
+        hipLaunchKernelGGL(reduce_partials_kernel<float>, rgrid, dim3(256), 0, stream, r);
+        BF_HIP_CHECK(hipGetLastError());
+        return BF_OK;
+    }
 
     const bool have_rows = p->batch > 0 && p->nstacks > 0;
     // forward launches that materialise the input of every chunk after the first

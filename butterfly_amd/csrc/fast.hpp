@@ -1,0 +1,426 @@
+// Twiddle-stationary kernels for base-2 float rows of n <= 1024.
+//
+// One workgroup of 1024 threads (16 wavefronts) owns a group of 1024 / n rows at a time and
+// keeps every 2x2 factor it needs in registers for the whole launch: thread t holds one
+// element per row and, per stage, the two factor entries of its own output row.  Rows
+// stream through; HBM sees each row once in and once out.
+//
+// A stage pairs element e with e ^ (1 << bit).  Where the partner lives decides the
+// exchange:
+//   * lanes of one 16-lane row:   DPP (quad_perm / row_half_mirror / row_mirror), fused
+//     into the multiply.  The 16 lanes of a row hold element low bits phi4(lane), a
+//     GF(2)-linear relabelling chosen so that XOR by element bit 0, 1, 2, 3 is exactly one
+//     of those four DPP patterns.
+//   * lane bits 4 and 5:          ds_swizzle (xor 16) and ds_bpermute (xor 32); these use the
+//     LDS crossbar, not the vector ALU.
+//   * across wavefronts (element bits >= 6): the workgroup transposes through LDS into a
+//     second layout ("B") in which those bits sit on the DPP lanes and the low bits sit on
+//     the wavefront index; it transposes back ("A") when low bits are needed again.  A
+//     10-stage block costs two transposes, not four exchanges.
+//
+// The backward kernel replays the forward stages keeping every stage input in registers,
+// then walks back accumulating d_twiddle in registers across all rows of the workgroup;
+// partial sums are written once at the end and reduced by reduce_partials_kernel in a
+// fixed order (no atomics).
+#pragma once
+
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace bf {
+
+constexpr int kFastThreads = 1024;
+constexpr int kFastRowWords = 1024 + 16;  // one LDS row: 1024 words + 1 pad word per 64
+
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+__host__ __device__ constexpr int phi4(int l)
+{
+    return ((l & 1) ? 1 : 0) ^ ((l & 2) ? 2 : 0) ^ ((l & 4) ? 7 : 0) ^ ((l & 8) ? 12 : 0);
+}
+
+template <int L, int NB, bool INC>
+struct FastPlan {
+    static constexpr int NS = L * NB;
+    static constexpr int NSWAP = L > 6 ? L - 6 : 0;  // element bits exchanged between layouts
+    static constexpr int SLOTS = 1024 >> L;          // rows a workgroup holds at once
+
+    // element bit paired by stage s
+    static constexpr int bit(int s)
+    {
+        const int k = s / L, idx = s % L;
+        const bool inc = INC != ((k & 1) != 0);
+        return inc ? idx : L - 1 - idx;
+    }
+    // layout (0 = A, 1 = B) in which stage s runs: bits >= 6 need B, bits < NSWAP need A,
+    // anything else stays where the previous stage left the data.
+    static constexpr int layout(int s)
+    {
+        int cur = 0;
+        for (int j = 0; j <= s; ++j) {
+            const int b = bit(j);
+            if (b >= 6) cur = 1;
+            else if (b < NSWAP) cur = 0;
+        }
+        return cur;
+    }
+    static constexpr int layout_before(int s) { return s == 0 ? 0 : layout(s - 1); }
+    // exchange kind: 0..3 DPP pattern for phi bit, 4 swizzle xor 16, 5 bpermute xor 32
+    static constexpr int kind(int s)
+    {
+        const int b = bit(s);
+        return b >= 6 ? b - 6 : b;
+    }
+    // LDS transposes performed before stage s of a forward walk (for buffer parity)
+    static constexpr int fw_transposes_before(int s)
+    {
+        int c = 0, cur = 0;
+        for (int j = 0; j < s; ++j) {
+            if (layout(j) != cur) { ++c; cur = layout(j); }
+        }
+        return c;
+    }
+    static constexpr int fw_transposes_total()
+    {
+        int c = fw_transposes_before(NS);
+        return c + (layout(NS - 1) != 0 ? 1 : 0);
+    }
+    // The reverse walk starts in layout A and visits stages NS-1 .. 0; layout the running
+    // gradient is in when stage s is reached, and transposes performed before that point.
+    static constexpr int layout_after(int s) { return s == NS - 1 ? 0 : layout(s + 1); }
+    static constexpr int bw_transposes_before(int s)
+    {
+        int c = 0;
+        for (int j = NS - 1; j > s; --j) {
+            if (layout(j) != layout_after(j)) ++c;
+        }
+        return c;
+    }
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL,
+                                                                  0xf, 0xf, true));
+}
+
+// Value of `v` held by the partner thread of an exchange of kind K.
+template <int K>
+__device__ __forceinline__ float partner(float v, int bperm_addr)
+{
+    if constexpr (K == 0) return dpp_move<0xB1>(v);        // quad_perm [1,0,3,2]
+    else if constexpr (K == 1) return dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+    else if constexpr (K == 2) return dpp_move<0x141>(v);  // row_half_mirror
+    else if constexpr (K == 3) return dpp_move<0x140>(v);  // row_mirror
+    else if constexpr (K == 4)
+        return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+    else
+        return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(bperm_addr, __builtin_bit_cast(int, v)));
+}
+
+// acc += g * x, pinned where it is written: the accumulators live across the whole row loop
+// and the compiler otherwise sinks these to the end of the iteration, which keeps every
+// stage's operands alive and overflows the register file.
+__device__ __forceinline__ void fmac_pinned(float &acc, float g, float x)
+{
+    asm volatile("v_fmac_f32_e32 %0, %1, %2" : "+v"(acc) : "v"(g), "v"(x));
+}
+
+// acc += g * (x held by the partner thread), for the DPP exchange kinds: one v_fmac with a
+// DPP source.  The s_nop covers the two wait states a DPP read needs after a VALU write of
+// its source register.
+template <int K>
+__device__ __forceinline__ void fmac_partner_dpp(float &acc, float g, float x)
+{
+    static_assert(K >= 0 && K < 4, "DPP kinds only");
+    if constexpr (K == 0)
+        asm volatile("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1"
+                     : "+v"(acc) : "v"(x), "v"(g));
+    else if constexpr (K == 1)
+        asm volatile("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1"
+                     : "+v"(acc) : "v"(x), "v"(g));
+    else if constexpr (K == 2)
+        asm volatile("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1"
+                     : "+v"(acc) : "v"(x), "v"(g));
+    else
+        asm volatile("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1"
+                     : "+v"(acc) : "v"(x), "v"(g));
+}
+
+// Per-thread coordinates in both layouts.
+struct FastCoords {
+    int eA, eB;    // element index in layout A / B
+    int fA, fB;    // padded LDS word offsets of those elements (slot included)
+    int slot;      // which of the workgroup's rows this thread works on
+    int bperm_addr;
+};
+
+template <int L>
+__device__ __forceinline__ FastCoords fast_coords(int t)
+{
+    constexpr int NSWAP = L > 6 ? L - 6 : 0;
+    constexpr int m = (1 << NSWAP) - 1;
+    const int v4 = phi4(t & 15), h = (t >> 4) & 3, w = t >> 6;
+    const int VA = v4 | (h << 4) | (w << 6);
+    const int VB = ((v4 & ~m) | (w & m)) | (h << 4) | (((w & ~m) | (v4 & m)) << 6);
+    FastCoords c;
+    c.eA = VA & ((1 << L) - 1);
+    c.eB = VB & ((1 << L) - 1);
+    c.fA = VA + (VA >> 6);
+    c.fB = VB + (VB >> 6);
+    c.slot = VA >> L;
+    c.bperm_addr = ((t & 63) ^ 32) << 2;
+    return c;
+}
+
+struct FastFwArgs {
+    const float *tw;           // factors of the first block of this launch, stack 0
+    int64_t tw_stack_stride;
+    const float *in;
+    View in_view;
+    float *out;
+    View out_view;
+    int64_t batch;
+    int64_t ngroups;           // ceil(batch / SLOTS)
+    int64_t groups_per_wg;
+};
+
+template <int L, int NB, bool INC, int R>
+__global__ __launch_bounds__(kFastThreads) void fast_fw_kernel(FastFwArgs a)
+{
+    using P = FastPlan<L, NB, INC>;
+    constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
+    __shared__ float lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
+    const int t = threadIdx.x;
+    const int stack = blockIdx.y;
+    const FastCoords c = fast_coords<L>(t);
+
+    float ta[NS], tb[NS];
+    {
+        const float *twp = a.tw + stack * a.tw_stack_stride;
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            constexpr int bit = P::bit(s);
+            constexpr int lay = P::layout(s);
+            const int e = lay ? c.eB : c.eA;
+            const int r = (e >> bit) & 1;
+            const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
+            const float *T = twp + ((int64_t)s * (n / 2) + i) * 4;
+            ta[s] = T[3 * r];   // T[r][r]
+            tb[s] = T[r + 1];   // T[r][1 - r]
+        });
+    }
+
+    const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
+    const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
+    const bool col_in = c.eA < a.in_view.width;
+    const bool col_out = c.eA < a.out_view.width;
+    const int64_t in_off = stack * a.in_view.ss + c.eA * a.in_view.se;
+    const int64_t out_off = stack * a.out_view.ss + c.eA * a.out_view.se;
+
+    auto load_rows = [&](int64_t g, float (&v)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t row = (g + r) * SLOTS + c.slot;
+            v[r] = (g + r < g1 && row < a.batch && col_in) ? a.in[row * a.in_view.sb + in_off] : 0.0f;
+        }
+    };
+
+    float nxt[R];
+    if (g0 < g1) load_rows(g0, nxt);
+    for (int64_t g = g0; g < g1; g += R) {
+        float v[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) v[r] = nxt[r];
+        if (g + R < g1) load_rows(g + R, nxt);
+
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            constexpr int K = P::kind(s);
+            if constexpr (P::layout(s) != P::layout_before(s)) {
+                constexpr int par = P::fw_transposes_before(s) & 1;
+                constexpr int to_b = P::layout(s);
+                float *buf = lds + par * R * kFastRowWords;
+                const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
+#pragma unroll
+                for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float p = tb[s] * partner<K>(v[r], c.bperm_addr);
+                v[r] = fmaf(ta[s], v[r], p);
+            }
+        });
+        if constexpr (P::layout(NS - 1) != 0) {
+            constexpr int par = P::fw_transposes_before(NS) & 1;
+            float *buf = lds + par * R * kFastRowWords;
+#pragma unroll
+            for (int r = 0; r < R; ++r) buf[r * kFastRowWords + c.fB] = v[r];
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + c.fA];
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t row = (g + r) * SLOTS + c.slot;
+            if (g + r < g1 && row < a.batch && col_out) a.out[row * a.out_view.sb + out_off] = v[r];
+        }
+    }
+}
+
+struct FastBwArgs {
+    const float *tw;
+    int64_t tw_stack_stride;
+    const float *x_in;
+    View x_view;
+    const float *g_out;
+    View g_view;
+    float *g_in;
+    View gi_view;              // columns in [n, width) are zero-filled
+    float *partial;            // (gridDim.x * SLOTS, S, NS, 2 n)
+    int64_t batch;
+    int64_t ngroups;
+    int64_t groups_per_wg;
+};
+
+template <int L, int NB, bool INC>
+__global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
+{
+    using P = FastPlan<L, NB, INC>;
+    constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
+    constexpr int FWT = P::fw_transposes_before(NS);  // transposes of the forward replay
+    __shared__ float lds[P::NSWAP > 0 ? 2 * kFastRowWords : 1];
+    const int t = threadIdx.x;
+    const int stack = blockIdx.y;
+    const FastCoords c = fast_coords<L>(t);
+
+    float ta[NS], tb[NS], acc_self[NS], acc_cross[NS];
+    {
+        const float *twp = a.tw + stack * a.tw_stack_stride;
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            constexpr int bit = P::bit(s);
+            constexpr int lay = P::layout(s);
+            const int e = lay ? c.eB : c.eA;
+            const int r = (e >> bit) & 1;
+            const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
+            const float *T = twp + ((int64_t)s * (n / 2) + i) * 4;
+            ta[s] = T[3 * r];
+            tb[s] = T[r + 1];
+            acc_self[s] = 0.0f;
+            acc_cross[s] = 0.0f;
+        });
+    }
+
+    const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
+    const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
+    const bool col_x = c.eA < a.x_view.width;
+    const bool col_g = c.eA < a.g_view.width;
+    const int64_t x_off = stack * a.x_view.ss + c.eA * a.x_view.se;
+    const int64_t g_off = stack * a.g_view.ss + c.eA * a.g_view.se;
+    const int64_t gi_off = stack * a.gi_view.ss;
+
+    auto transpose = [&](float v, int parity, int to_layout) -> float {
+        float *buf = lds + (parity & 1) * kFastRowWords;
+        buf[to_layout ? c.fA : c.fB] = v;
+        __syncthreads();
+        return buf[to_layout ? c.fB : c.fA];
+    };
+
+    float nx = 0.0f, ng = 0.0f;
+    {
+        const int64_t row = g0 * SLOTS + c.slot;
+        const bool ok = g0 < g1 && row < a.batch;
+        if (ok && col_x) nx = a.x_in[row * a.x_view.sb + x_off];
+        if (ok && col_g) ng = a.g_out[row * a.g_view.sb + g_off];
+    }
+    for (int64_t g = g0; g < g1; ++g) {
+        float v = nx, gv = ng;
+        nx = 0.0f;
+        ng = 0.0f;
+        {
+            const int64_t row = (g + 1) * SLOTS + c.slot;
+            const bool ok = g + 1 < g1 && row < a.batch;
+            if (ok && col_x) nx = a.x_in[row * a.x_view.sb + x_off];
+            if (ok && col_g) ng = a.g_out[row * a.g_view.sb + g_off];
+        }
+        float act[NS];
+        // forward replay: act[s] = input of stage s, in the layout stage s runs in
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            constexpr int K = P::kind(s);
+            if constexpr (P::layout(s) != P::layout_before(s)) {
+                constexpr int par = P::fw_transposes_before(s) & 1;
+                constexpr int to_b = P::layout(s);
+                v = transpose(v, par, to_b);
+            }
+            act[s] = v;
+            if constexpr (s + 1 < NS) {
+                const float p = tb[s] * partner<K>(v, c.bperm_addr);
+                v = fmaf(ta[s], v, p);
+            }
+        });
+        // reverse sweep; the gradient arrives in layout A
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = NS - 1 - S;
+            constexpr int K = P::kind(s);
+            if constexpr (P::layout(s) != P::layout_after(s)) {
+                constexpr int par = (FWT + P::bw_transposes_before(s)) & 1;
+                constexpr int to_b = P::layout(s);
+                gv = transpose(gv, par, to_b);
+            }
+            const float xs = act[s];
+            fmac_pinned(acc_self[s], gv, xs);
+            if constexpr (K < 4) fmac_partner_dpp<K>(acc_cross[s], gv, xs);
+            else fmac_pinned(acc_cross[s], gv, partner<K>(xs, c.bperm_addr));
+            // d_x[r] = T[r][r] g[r] + T[1-r][r] g[1-r]; the second product is formed by the
+            // partner from its own factor entry and fetched.
+            const float m = tb[s] * gv;
+            if constexpr (K < 4) gv = ta[s] * gv + partner<K>(m, c.bperm_addr);
+            else gv = fmaf(ta[s], gv, partner<K>(m, c.bperm_addr));
+        });
+        if constexpr (P::layout(0) != 0) {
+            constexpr int par = (FWT + P::bw_transposes_before(-1)) & 1;
+            gv = transpose(gv, par, 0);
+        }
+
+        const int64_t row = g * SLOTS + c.slot;
+        if (row < a.batch) {
+            float *dst = a.g_in + row * a.gi_view.sb + gi_off;
+            if (c.eA < a.gi_view.width) dst[c.eA * a.gi_view.se] = gv;
+            for (int64_t j = n + c.eA; j < a.gi_view.width; j += n) dst[j * a.gi_view.se] = 0.0f;
+        }
+    }
+
+    // Recompute the coordinates from a laundered thread id: sharing them with the prologue
+    // would keep one address per stage alive across the whole row loop.
+    int t2 = t;
+    asm volatile("" : "+v"(t2));
+    const FastCoords c2 = fast_coords<L>(t2);
+    float *part = a.partial + (((int64_t)blockIdx.x * SLOTS + c2.slot) * gridDim.y + stack) * NS * (2 * n);
+    static_for<0, NS>([&](auto S) {
+        constexpr int s = S;
+        constexpr int bit = P::bit(s);
+        constexpr int lay = P::layout(s);
+        const int e = lay ? c2.eB : c2.eA;
+        const int r = (e >> bit) & 1;
+        const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
+        float *d = part + (int64_t)s * (2 * n) + i * 4;
+        d[3 * r] = acc_self[s];    // dT[r][r]
+        d[r + 1] = acc_cross[s];   // dT[r][1 - r]
+    });
+}
+
+}  // namespace bf

@@ -70,6 +70,30 @@ def test_c_abi_matches_oracle(case):
     assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
 
 
+@pytest.mark.parametrize("L", list(range(1, 11)))
+def test_register_resident_kernels_all_sizes(L):
+    """n = 2 .. 1024 with one or two blocks run on the twiddle-stationary kernels: every
+    size, both stride orders, ragged batch (partial row groups), padded input, sliced
+    output, two stacks."""
+    from butterfly_amd import _capi
+    n = 1 << L
+    rng = np.random.default_rng(500 + L)
+    for nb in (1, 2):
+        for inc in (True, False):
+            for B, S, I, O in [(1, 1, n, n), (37, 2, n, n), (300, 1, max(1, n - 1), max(1, n - 1)),
+                               (19, 2, n + 5, max(1, n // 2))]:
+                say("fast case", L, nb, inc, B, S, I, O)
+                tw, x, g = make_case(rng, np.float32, B, S, L, nb, I, O)
+                y_ref = oracle.butterfly_fw(tw, x, inc, O)
+                dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+                y = _capi.multiply_fw(dev(tw), dev(x), inc, O)
+                dtw, dx = _capi.multiply_bw(dev(tw), dev(x), dev(g), inc)
+                torch.cuda.synchronize()
+                assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL, (L, nb, inc, B, S, I, O)
+                assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL, (L, nb, inc, B, S, I, O)
+                assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL, (L, nb, inc, B, S, I, O)
+
+
 def test_c_abi_strided_operands():
     """Stride-0 stack broadcast (what Butterfly.pre_process hands over), a transposed input
     and a non-contiguous gradient."""
