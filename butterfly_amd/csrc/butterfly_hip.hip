@@ -135,15 +135,18 @@ int ensure_attributes()
     return BF_OK;
 }
 
-// ---- twiddle-stationary fast path (float, base-2, n <= 1024, nblocks <= 2) ------------------
-
 constexpr int kNumCU = 256;     // MI355X
 constexpr int kFastFwRows = 4;  // row groups in flight per forward workgroup
 
-bool fast_applicable(const bf_problem *p, bool base4)
+// ---- twiddle-stationary fast path (float, base-2, n <= 1024, nblocks <= 2) ------------------
+
+
+// Largest byte offset one workgroup forms into an operand with these strides; the fast
+// kernels address through 32-bit offsets and need it below 2 GiB.
+bool span_ok(const int64_t stride[3], int64_t rows, int64_t width)
 {
-    return !base4 && p->dtype == BF_F32 && p->log_n >= 1 && p->log_n <= 10 && p->nblocks >= 1 &&
-           p->nblocks <= 2 && p->batch > 0 && p->nstacks > 0;
+    const double bytes = 4.0 * ((double)rows * (double)stride[0] + (double)width * (double)stride[2]);
+    return bytes < 2147483000.0;
 }
 
 struct FastGrid {
@@ -161,6 +164,19 @@ FastGrid fast_grid(const bf_problem *p, int rows_in_flight, int wg_per_cu)
     g.groups_per_wg = ((iters + g.nwg - 1) / g.nwg) * rows_in_flight;
     g.nwg = (g.ngroups + g.groups_per_wg - 1) / g.groups_per_wg;
     return g;
+}
+
+bool fast_applicable(const bf_problem *p, bool base4, bool backward)
+{
+    if (base4 || p->dtype != BF_F32 || p->log_n < 1 || p->log_n > 10 || p->nblocks < 1 || p->nblocks > 2 ||
+        p->batch <= 0 || p->nstacks <= 0 || p->input_size <= 0 || p->output_size <= 0)
+        return false;
+    const int64_t n = (int64_t)1 << p->log_n;
+    const FastGrid g = fast_grid(p, backward ? 1 : kFastFwRows, 1);
+    const int64_t rows = (g.groups_per_wg + kFastFwRows) * g.slots;
+    if (!span_ok(p->input_stride, rows, n) || !span_ok(p->output_stride, rows, n)) return false;
+    if (backward && !span_ok(p->d_input_stride, rows, std::max(n, p->input_size))) return false;
+    return true;
 }
 
 template <int L, int NB, bool INC>
@@ -270,7 +286,7 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
             if (base4 && (p->log_n & 1) && !tw2) return fail(BF_ERR_INVALID, "twiddle2 is NULL");
         }
     }
-    if (fast_applicable(p, base4)) return fast_forward(p, tw2, input, output, stream);
+    if (fast_applicable(p, base4, false)) return fast_forward(p, tw2, input, output, stream);
     const View in_view = make_view(p->input_stride, std::min(p->input_size, n));
     const View out_view = make_view(p->output_stride, p->output_size);
     return launch_generic_fw(p, sc, 0, sc.per * sc.nblocks, tw2, tw4, input, in_view, output,
@@ -299,7 +315,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
     const size_t row_bytes = (size_t)n * e;
     const Schedule sc = make_schedule(p, base4);
     pl.nstages = sc.per * sc.nblocks;
-    if (fast_applicable(p, base4)) {
+    if (fast_applicable(p, base4, true)) {
         // one launch; partial sums from every (workgroup, row slot)
         const FastGrid g = fast_grid(p, 1, 1);
         pl.fits = true;
@@ -360,6 +376,29 @@ int launch_copy_pad(const bf_problem *p, const void *in, const View &iv, void *o
     return BF_OK;
 }
 
+int launch_reduce(const bf_problem *p, const Schedule &sc, int t0, int t1, int64_t nparts, const void *partial,
+                  int64_t slot, void *d_tw2, void *d_tw4, hipStream_t stream)
+{
+    if (p->nstacks == 0 || t1 <= t0) return BF_OK;
+    if (((reinterpret_cast<uintptr_t>(d_tw2) | reinterpret_cast<uintptr_t>(d_tw4)) & 15) != 0)
+        return fail(BF_ERR_INVALID, "d_twiddle pointers must be 16-byte aligned");
+    ReduceArgs r;
+    r.sc = sc;
+    r.t0 = t0;
+    r.t1 = t1;
+    r.nparts = (int)nparts;
+    r.elem_floats = p->dtype == BF_C64 ? 2 : 1;
+    r.nstacks = p->nstacks;
+    r.partial = static_cast<const float *>(partial);
+    r.slot = slot;
+    r.d_tw2 = static_cast<float *>(d_tw2);
+    r.d_tw4 = static_cast<float *>(d_tw4);
+    const dim3 grid((unsigned)((slot * r.elem_floats + 63) / 64), (unsigned)(t1 - t0), (unsigned)p->nstacks);
+    hipLaunchKernelGGL(reduce_partials_kernel, grid, dim3(256), 0, stream, r);
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
+}
+
 int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, const void *input,
              const void *grad, void *d_tw2, void *d_tw4, void *d_input, void *workspace,
              size_t workspace_bytes, void *stream_)
@@ -404,19 +443,8 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
         const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks);
         BF_FAST_DISPATCH(launch_fast_bw_t, a, grid, stream);
         BF_HIP_CHECK(hipGetLastError());
-        ReduceArgs r;
-        r.sc = sc;
-        r.t0 = 0;
-        r.t1 = pl.nstages;
-        r.nparts = (int)pl.nparts;
-        r.nstacks = p->nstacks;
-        r.partial = ws + pl.off_partials;
-        r.slot = pl.slot;
-        r.d_tw2 = d_tw2;
-        r.d_tw4 = d_tw4;
-        const dim3 rgrid((unsigned)((pl.slot + 255) / 256), (unsigned)pl.nstages, (unsigned)p->nstacks);
-        hipLaunchKernelGGL(reduce_partials_kernel<float>, rgrid, dim3(256), 0, stream, r);
-        BF_HIP_CHECK(hipGetLastError());
+        rc = launch_reduce(p, sc, 0, pl.nstages, pl.nparts, ws + pl.off_partials, pl.slot, d_tw2, d_tw4, stream);
+        if (rc) return rc;
         return BF_OK;
     }
 
@@ -457,24 +485,9 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                 hipLaunchKernelGGL(generic_bw_kernel<float2>, grid, dim3(kGenericThreads), lds, stream, a);
             BF_HIP_CHECK(hipGetLastError());
         }
-        if (p->nstacks > 0) {
-            ReduceArgs r;
-            r.sc = sc;
-            r.t0 = t0;
-            r.t1 = t1;
-            r.nparts = have_rows ? (int)pl.nparts : 0;
-            r.nstacks = p->nstacks;
-            r.partial = ws + pl.off_partials;
-            r.slot = pl.slot;
-            r.d_tw2 = d_tw2;
-            r.d_tw4 = d_tw4;
-            const dim3 grid((unsigned)((pl.slot + 255) / 256), (unsigned)(t1 - t0), (unsigned)p->nstacks);
-            if (p->dtype == BF_F32)
-                hipLaunchKernelGGL(reduce_partials_kernel<float>, grid, dim3(256), 0, stream, r);
-            else
-                hipLaunchKernelGGL(reduce_partials_kernel<float2>, grid, dim3(256), 0, stream, r);
-            BF_HIP_CHECK(hipGetLastError());
-        }
+        rc = launch_reduce(p, sc, t0, t1, have_rows ? pl.nparts : 0, ws + pl.off_partials, pl.slot, d_tw2, d_tw4,
+                           stream);
+        if (rc) return rc;
     }
     return BF_OK;
 }

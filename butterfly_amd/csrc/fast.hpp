@@ -182,6 +182,31 @@ __device__ __forceinline__ FastCoords fast_coords(int t)
     return c;
 }
 
+// ---- global memory through buffer resources ---------------------------------------------------
+// Every operand is addressed as base + 32-bit byte offset through a raw buffer resource whose
+// base is the first row this workgroup touches (stack offset folded in).  An access that must
+// not happen (row past the batch, column past the operand width) uses the offset kOob, which
+// lies outside the resource's range: the hardware returns zero for such a load and drops
+// such a store.  No branches, so the row loop is straight-line code and the prefetch of the
+// next rows really overlaps the stages of the current ones.  The host guarantees that all
+// valid offsets of one workgroup stay below 2 GiB.
+constexpr int kOob = (int)0x80000000u;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)0x80000000u, 0x00020000);
+}
+
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int byte_off)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+}
+
+__device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, int byte_off, float v)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, byte_off, 0, 0);
+}
+
 struct FastFwArgs {
     const float *tw;           // factors of the first block of this launch, stack 0
     int64_t tw_stack_stride;
@@ -222,26 +247,30 @@ __global__ __launch_bounds__(kFastThreads) void fast_fw_kernel(FastFwArgs a)
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
-    const bool col_in = c.eA < a.in_view.width;
-    const bool col_out = c.eA < a.out_view.width;
-    const int64_t in_off = stack * a.in_view.ss + c.eA * a.in_view.se;
-    const int64_t out_off = stack * a.out_view.ss + c.eA * a.out_view.se;
+    const int ng = (int)(g1 - g0);
+    const int64_t row_end = g1 * SLOTS < a.batch ? g1 * SLOTS : a.batch;
+    const int rows_valid = (int)(row_end - g0 * SLOTS);
+    const __amdgpu_buffer_rsrc_t in_rs = make_rsrc(a.in + g0 * SLOTS * a.in_view.sb + stack * a.in_view.ss);
+    const __amdgpu_buffer_rsrc_t out_rs = make_rsrc(a.out + g0 * SLOTS * a.out_view.sb + stack * a.out_view.ss);
+    const int in_row = (int)(a.in_view.sb * 4), out_row = (int)(a.out_view.sb * 4);
+    const int in_col = c.eA < a.in_view.width ? (int)(c.eA * a.in_view.se * 4) : kOob;
+    const int out_col = c.eA < a.out_view.width ? (int)(c.eA * a.out_view.se * 4) : kOob;
 
-    auto load_rows = [&](int64_t g, float (&v)[R]) {
+    auto load_rows = [&](int grel, float (&v)[R]) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int64_t row = (g + r) * SLOTS + c.slot;
-            v[r] = (g + r < g1 && row < a.batch && col_in) ? a.in[row * a.in_view.sb + in_off] : 0.0f;
+            const int rr = (grel + r) * SLOTS + c.slot;
+            v[r] = buf_load(in_rs, rr < rows_valid ? rr * in_row + in_col : kOob);
         }
     };
 
     float nxt[R];
-    if (g0 < g1) load_rows(g0, nxt);
-    for (int64_t g = g0; g < g1; g += R) {
+    load_rows(0, nxt);
+    for (int grel = 0; grel < ng; grel += R) {
         float v[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) v[r] = nxt[r];
-        if (g + R < g1) load_rows(g + R, nxt);
+        load_rows(grel + R, nxt);
 
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
@@ -274,8 +303,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_fw_kernel(FastFwArgs a)
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int64_t row = (g + r) * SLOTS + c.slot;
-            if (g + r < g1 && row < a.batch && col_out) a.out[row * a.out_view.sb + out_off] = v[r];
+            const int rr = (grel + r) * SLOTS + c.slot;
+            buf_store(out_rs, rr < rows_valid ? rr * out_row + out_col : kOob, v[r]);
         }
     }
 }
@@ -326,11 +355,16 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
-    const bool col_x = c.eA < a.x_view.width;
-    const bool col_g = c.eA < a.g_view.width;
-    const int64_t x_off = stack * a.x_view.ss + c.eA * a.x_view.se;
-    const int64_t g_off = stack * a.g_view.ss + c.eA * a.g_view.se;
-    const int64_t gi_off = stack * a.gi_view.ss;
+    const int ng = (int)(g1 - g0);
+    const int64_t row_end = g1 * SLOTS < a.batch ? g1 * SLOTS : a.batch;
+    const int rows_valid = (int)(row_end - g0 * SLOTS);
+    const __amdgpu_buffer_rsrc_t x_rs = make_rsrc(a.x_in + g0 * SLOTS * a.x_view.sb + stack * a.x_view.ss);
+    const __amdgpu_buffer_rsrc_t g_rs = make_rsrc(a.g_out + g0 * SLOTS * a.g_view.sb + stack * a.g_view.ss);
+    const __amdgpu_buffer_rsrc_t gi_rs = make_rsrc(a.g_in + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
+    const int x_row = (int)(a.x_view.sb * 4), g_row = (int)(a.g_view.sb * 4), gi_row = (int)(a.gi_view.sb * 4);
+    const int x_col = c.eA < a.x_view.width ? (int)(c.eA * a.x_view.se * 4) : kOob;
+    const int g_col = c.eA < a.g_view.width ? (int)(c.eA * a.g_view.se * 4) : kOob;
+    const int gi_col = c.eA < a.gi_view.width ? (int)(c.eA * a.gi_view.se * 4) : kOob;
 
     auto transpose = [&](float v, int parity, int to_layout) -> float {
         float *buf = lds + (parity & 1) * kFastRowWords;
@@ -339,22 +373,14 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         return buf[to_layout ? c.fB : c.fA];
     };
 
-    float nx = 0.0f, ng = 0.0f;
-    {
-        const int64_t row = g0 * SLOTS + c.slot;
-        const bool ok = g0 < g1 && row < a.batch;
-        if (ok && col_x) nx = a.x_in[row * a.x_view.sb + x_off];
-        if (ok && col_g) ng = a.g_out[row * a.g_view.sb + g_off];
-    }
-    for (int64_t g = g0; g < g1; ++g) {
-        float v = nx, gv = ng;
-        nx = 0.0f;
-        ng = 0.0f;
+    float nx = buf_load(x_rs, c.slot < rows_valid ? c.slot * x_row + x_col : kOob);
+    float ng_ = buf_load(g_rs, c.slot < rows_valid ? c.slot * g_row + g_col : kOob);
+    for (int grel = 0; grel < ng; ++grel) {
+        float v = nx, gv = ng_;
         {
-            const int64_t row = (g + 1) * SLOTS + c.slot;
-            const bool ok = g + 1 < g1 && row < a.batch;
-            if (ok && col_x) nx = a.x_in[row * a.x_view.sb + x_off];
-            if (ok && col_g) ng = a.g_out[row * a.g_view.sb + g_off];
+            const int rn = (grel + 1) * SLOTS + c.slot;
+            nx = buf_load(x_rs, rn < rows_valid ? rn * x_row + x_col : kOob);
+            ng_ = buf_load(g_rs, rn < rows_valid ? rn * g_row + g_col : kOob);
         }
         float act[NS];
         // forward replay: act[s] = input of stage s, in the layout stage s runs in
@@ -396,12 +422,12 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             gv = transpose(gv, par, 0);
         }
 
-        const int64_t row = g * SLOTS + c.slot;
-        if (row < a.batch) {
-            float *dst = a.g_in + row * a.gi_view.sb + gi_off;
-            if (c.eA < a.gi_view.width) dst[c.eA * a.gi_view.se] = gv;
-            for (int64_t j = n + c.eA; j < a.gi_view.width; j += n) dst[j * a.gi_view.se] = 0.0f;
-        }
+        const int rr = grel * SLOTS + c.slot;
+        const bool row_ok = rr < rows_valid;
+        buf_store(gi_rs, row_ok ? rr * gi_row + gi_col : kOob, gv);
+        // input wider than n: those columns get a zero gradient
+        for (int64_t j = n + c.eA; j < a.gi_view.width; j += n)
+            buf_store(gi_rs, row_ok ? rr * gi_row + (int)(j * a.gi_view.se * 4) : kOob, 0.0f);
     }
 
     // Recompute the coordinates from a laundered thread id: sharing them with the prologue

@@ -254,34 +254,59 @@ struct ReduceArgs {
     Schedule sc;
     int t0, t1;
     int nparts;        // number of per-workgroup partial slices
+    int elem_floats;   // 1 for float, 2 for complex64
     int64_t nstacks;
-    const void *partial;
-    int64_t slot;
-    void *d_tw2;
-    void *d_tw4;
+    const float *partial;
+    int64_t slot;      // scalars reserved per stage in `partial`
+    float *d_tw2;
+    float *d_tw4;
 };
 
-// d_twiddle[s][stage][j] = sum over workgroups, in ascending workgroup order.
-// grid: (ceil(slot / 256), t1 - t0, S)
-template <typename T>
+// d_twiddle[s][stage][j] = sum over partial slices.  Works on raw floats (a complex sum is
+// two float sums).  A workgroup covers 64 consecutive floats: thread (q, j4) adds the slices
+// of group q (a contiguous sixteenth of them, ascending) for the float4 at j4; the sixteen
+// group sums are then added in ascending q.  The order is fixed by nparts alone, so results
+// are reproducible run to run.
+// grid: (ceil(slot * elem_floats / 64), t1 - t0, S), block 256.
 __global__ __launch_bounds__(256) void reduce_partials_kernel(ReduceArgs a)
 {
-    const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    __shared__ float4 sm[16][16];
+    const int j4 = threadIdx.x & 15, q = threadIdx.x >> 4;
     const int k = blockIdx.y;
     const int s = blockIdx.z;
     const int nst = a.t1 - a.t0;
     const StageInfo si = stage_info(a.sc, a.t0 + k);
     const int64_t n = (int64_t)1 << a.sc.log_n;
-    const int64_t count = si.radix4 ? 4 * n : 2 * n;
-    if (j >= count) return;
-    const T *part = reinterpret_cast<const T *>(a.partial) + ((int64_t)s * nst + k) * a.slot + j;
-    const int64_t wg_stride = a.nstacks * nst * a.slot;
-    T acc = zero_of(T());
-    for (int w = 0; w < a.nparts; ++w) acc = add(acc, part[(int64_t)w * wg_stride]);
-    if (si.radix4)
-        reinterpret_cast<T *>(a.d_tw4)[s * a.sc.tw4_stack_stride + si.tw_off + j] = acc;
-    else
-        reinterpret_cast<T *>(a.d_tw2)[s * a.sc.tw2_stack_stride + si.tw_off + j] = acc;
+    const int64_t ef = a.elem_floats;
+    const int64_t count = (si.radix4 ? 4 * n : 2 * n) * ef;   // floats in this stage
+    const int64_t f = (int64_t)blockIdx.x * 64 + j4 * 4;
+    const int64_t slot_f = a.slot * ef;
+    const int64_t wg_stride = a.nstacks * nst * slot_f;
+    const int chunk = (a.nparts + 15) / 16;
+    const int w0 = q * chunk;
+    const int w1 = w0 + chunk < a.nparts ? w0 + chunk : a.nparts;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (f < count) {
+        const float *src = a.partial + ((int64_t)s * nst + k) * slot_f + f;
+#pragma unroll 8
+        for (int w = w0; w < w1; ++w) {
+            const float4 v = *reinterpret_cast<const float4 *>(src + (int64_t)w * wg_stride);
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+    }
+    sm[q][j4] = acc;
+    __syncthreads();
+    if (q == 0 && f < count) {
+        float4 t = sm[0][j4];
+#pragma unroll
+        for (int qq = 1; qq < 16; ++qq) {
+            const float4 v = sm[qq][j4];
+            t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+        }
+        float *dst = si.radix4 ? a.d_tw4 + (s * a.sc.tw4_stack_stride + si.tw_off) * ef
+                               : a.d_tw2 + (s * a.sc.tw2_stack_stride + si.tw_off) * ef;
+        *reinterpret_cast<float4 *>(dst + f) = t;
+    }
 }
 
 }  // namespace bf
