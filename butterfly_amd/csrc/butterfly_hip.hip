@@ -136,7 +136,14 @@ int ensure_attributes()
 }
 
 constexpr int kNumCU = 256;     // MI355X
-constexpr int kFastFwRows = 4;  // row groups in flight per forward workgroup
+#ifndef BF_FAST_FW_ROWS
+#define BF_FAST_FW_ROWS 4
+#endif
+#ifndef BF_FAST_FW_WGS
+#define BF_FAST_FW_WGS 1
+#endif
+constexpr int kFastFwRows = BF_FAST_FW_ROWS;  // row groups in flight per forward workgroup
+constexpr int kFastFwWgPerCu = BF_FAST_FW_WGS;  // forward workgroups resident per compute unit
 
 // ---- twiddle-stationary fast path (float, base-2, n <= 1024, nblocks <= 2) ------------------
 
@@ -172,7 +179,7 @@ bool fast_applicable(const bf_problem *p, bool base4, bool backward)
         p->batch <= 0 || p->nstacks <= 0 || p->input_size <= 0 || p->output_size <= 0)
         return false;
     const int64_t n = (int64_t)1 << p->log_n;
-    const FastGrid g = fast_grid(p, backward ? 1 : kFastFwRows, 1);
+    const FastGrid g = fast_grid(p, backward ? 1 : kFastFwRows, backward ? 1 : kFastFwWgPerCu);
     const int64_t rows = (g.groups_per_wg + kFastFwRows) * g.slots;
     if (!span_ok(p->input_stride, rows, n) || !span_ok(p->output_stride, rows, n)) return false;
     if (backward && !span_ok(p->d_input_stride, rows, std::max(n, p->input_size))) return false;
@@ -212,7 +219,7 @@ void launch_fast_bw_t(const FastBwArgs &a, dim3 grid, hipStream_t stream)
 int fast_forward(const bf_problem *p, const void *tw, const void *input, void *output, hipStream_t stream)
 {
     const int64_t n = (int64_t)1 << p->log_n;
-    const FastGrid g = fast_grid(p, kFastFwRows, 1);
+    const FastGrid g = fast_grid(p, kFastFwRows, kFastFwWgPerCu);
     FastFwArgs a;
     a.tw = static_cast<const float *>(tw);
     a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;

@@ -197,14 +197,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base)
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)0x80000000u, 0x00020000);
 }
 
-__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int byte_off)
+// voff: per-thread byte offset (range-checked); soff: wave-uniform byte offset added on top.
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int voff, int soff)
 {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
 }
 
-__device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, int byte_off, float v)
+__device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, int voff, int soff, float v)
 {
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, byte_off, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
 }
 
 struct FastFwArgs {
@@ -220,7 +221,10 @@ struct FastFwArgs {
 };
 
 template <int L, int NB, bool INC, int R>
-__global__ __launch_bounds__(kFastThreads) void fast_fw_kernel(FastFwArgs a)
+#ifndef BF_FAST_FW_WAVES
+#define BF_FAST_FW_WAVES 4
+#endif
+__global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel(FastFwArgs a)
 {
     using P = FastPlan<L, NB, INC>;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
@@ -253,19 +257,26 @@ __global__ __launch_bounds__(kFastThreads) void fast_fw_kernel(FastFwArgs a)
     const __amdgpu_buffer_rsrc_t in_rs = make_rsrc(a.in + g0 * SLOTS * a.in_view.sb + stack * a.in_view.ss);
     const __amdgpu_buffer_rsrc_t out_rs = make_rsrc(a.out + g0 * SLOTS * a.out_view.sb + stack * a.out_view.ss);
     const int in_row = (int)(a.in_view.sb * 4), out_row = (int)(a.out_view.sb * 4);
-    const int in_col = c.eA < a.in_view.width ? (int)(c.eA * a.in_view.se * 4) : kOob;
-    const int out_col = c.eA < a.out_view.width ? (int)(c.eA * a.out_view.se * 4) : kOob;
+    // thread-constant part of the offsets; the row group adds a wave-uniform part
+    const int in_thr = c.eA < a.in_view.width ? c.slot * in_row + (int)(c.eA * a.in_view.se * 4) : kOob;
+    const int out_thr = c.eA < a.out_view.width ? c.slot * out_row + (int)(c.eA * a.out_view.se * 4) : kOob;
 
     auto load_rows = [&](int grel, float (&v)[R]) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int rr = (grel + r) * SLOTS + c.slot;
-            v[r] = buf_load(in_rs, rr < rows_valid ? rr * in_row + in_col : kOob);
+            const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
+            v[r] = buf_load(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
         }
     };
 
     float nxt[R];
     load_rows(0, nxt);
+    // R stores that the range check discards.  They put the same "loads, then stores" history
+    // in front of the first iteration as every later iteration has, so the wait for the
+    // prefetched rows at the top of the loop is emitted as "all but the newest R operations"
+    // and does not also wait for the previous iteration's stores to be acknowledged.
+#pragma unroll
+    for (int r = 0; r < R; ++r) buf_store(out_rs, kOob, 4 * r, 0.0f);
     for (int grel = 0; grel < ng; grel += R) {
         float v[R];
 #pragma unroll
@@ -303,8 +314,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_fw_kernel(FastFwArgs a)
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int rr = (grel + r) * SLOTS + c.slot;
-            buf_store(out_rs, rr < rows_valid ? rr * out_row + out_col : kOob, v[r]);
+            const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
+            buf_store(out_rs, ok ? out_thr : kOob, (grel + r) * SLOTS * out_row, v[r]);
         }
     }
 }
@@ -362,9 +373,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const __amdgpu_buffer_rsrc_t g_rs = make_rsrc(a.g_out + g0 * SLOTS * a.g_view.sb + stack * a.g_view.ss);
     const __amdgpu_buffer_rsrc_t gi_rs = make_rsrc(a.g_in + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
     const int x_row = (int)(a.x_view.sb * 4), g_row = (int)(a.g_view.sb * 4), gi_row = (int)(a.gi_view.sb * 4);
-    const int x_col = c.eA < a.x_view.width ? (int)(c.eA * a.x_view.se * 4) : kOob;
-    const int g_col = c.eA < a.g_view.width ? (int)(c.eA * a.g_view.se * 4) : kOob;
-    const int gi_col = c.eA < a.gi_view.width ? (int)(c.eA * a.gi_view.se * 4) : kOob;
+    const int x_thr = c.eA < a.x_view.width ? c.slot * x_row + (int)(c.eA * a.x_view.se * 4) : kOob;
+    const int g_thr = c.eA < a.g_view.width ? c.slot * g_row + (int)(c.eA * a.g_view.se * 4) : kOob;
+    const int gi_thr = c.eA < a.gi_view.width ? c.slot * gi_row + (int)(c.eA * a.gi_view.se * 4) : kOob;
 
     auto transpose = [&](float v, int parity, int to_layout) -> float {
         float *buf = lds + (parity & 1) * kFastRowWords;
@@ -373,14 +384,14 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         return buf[to_layout ? c.fB : c.fA];
     };
 
-    float nx = buf_load(x_rs, c.slot < rows_valid ? c.slot * x_row + x_col : kOob);
-    float ng_ = buf_load(g_rs, c.slot < rows_valid ? c.slot * g_row + g_col : kOob);
+    float nx = buf_load(x_rs, c.slot < rows_valid ? x_thr : kOob, 0);
+    float ng_ = buf_load(g_rs, c.slot < rows_valid ? g_thr : kOob, 0);
     for (int grel = 0; grel < ng; ++grel) {
         float v = nx, gv = ng_;
         {
-            const int rn = (grel + 1) * SLOTS + c.slot;
-            nx = buf_load(x_rs, rn < rows_valid ? rn * x_row + x_col : kOob);
-            ng_ = buf_load(g_rs, rn < rows_valid ? rn * g_row + g_col : kOob);
+            const bool ok = (grel + 1) * SLOTS + c.slot < rows_valid;
+            nx = buf_load(x_rs, ok ? x_thr : kOob, (grel + 1) * SLOTS * x_row);
+            ng_ = buf_load(g_rs, ok ? g_thr : kOob, (grel + 1) * SLOTS * g_row);
         }
         float act[NS];
         // forward replay: act[s] = input of stage s, in the layout stage s runs in
@@ -422,12 +433,11 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             gv = transpose(gv, par, 0);
         }
 
-        const int rr = grel * SLOTS + c.slot;
-        const bool row_ok = rr < rows_valid;
-        buf_store(gi_rs, row_ok ? rr * gi_row + gi_col : kOob, gv);
+        const bool row_ok = grel * SLOTS + c.slot < rows_valid;
+        buf_store(gi_rs, row_ok ? gi_thr : kOob, grel * SLOTS * gi_row, gv);
         // input wider than n: those columns get a zero gradient
         for (int64_t j = n + c.eA; j < a.gi_view.width; j += n)
-            buf_store(gi_rs, row_ok ? rr * gi_row + (int)(j * a.gi_view.se * 4) : kOob, 0.0f);
+            buf_store(gi_rs, row_ok ? c.slot * gi_row + (int)(j * a.gi_view.se * 4) : kOob, grel * SLOTS * gi_row, 0.0f);
     }
 
     // Recompute the coordinates from a laundered thread id: sharing them with the prologue
