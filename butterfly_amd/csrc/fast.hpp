@@ -335,13 +335,58 @@ struct FastBwArgs {
     int64_t groups_per_wg;
 };
 
+// Backward kernel, software-pipelined over rows: iteration i runs the forward replay of
+// row i + 1 (producing its stage inputs) together with the reverse sweep of row i (consuming
+// the stage inputs produced one iteration earlier).  The two walks change layout at mirrored
+// points, so they share every barrier, and their transposes travel through LDS as one
+// 64-bit (x, g) pair.  Two independent dependency chains per thread also hide the DPP and
+// LDS latencies that a single chain exposes.
+template <int L, int NB, bool INC>
+struct BwPipe {
+    using P = FastPlan<L, NB, INC>;
+    static constexpr int NS = P::NS;
+    static constexpr int nF = P::fw_transposes_before(NS);
+    static constexpr int nB = P::bw_transposes_before(-1) + (P::layout(0) != 0 ? 1 : 0);
+    static constexpr int K = nF > nB ? nF : nB;  // phases 0..K; phase k >= 1 opens with transposes #k
+    // phase in which forward stage s / reverse stage s runs
+    static constexpr int fphase(int s) { return P::fw_transposes_before(s + 1); }
+    static constexpr int bphase(int s)
+    {
+        return P::bw_transposes_before(s) + (P::layout(s) != P::layout_after(s) ? 1 : 0);
+    }
+    static constexpr int f_count(int k)
+    {
+        int c = 0;
+        for (int s = 0; s < NS; ++s) c += fphase(s) == k ? 1 : 0;
+        return c;
+    }
+    static constexpr int f_first(int k)
+    {
+        for (int s = 0; s < NS; ++s)
+            if (fphase(s) == k) return s;
+        return NS;
+    }
+    static constexpr int b_count(int k)
+    {
+        int c = 0;
+        for (int s = 0; s < NS; ++s) c += bphase(s) == k ? 1 : 0;
+        return c;
+    }
+    static constexpr int b_first(int k)  // highest stage of the phase: the reverse walk descends
+    {
+        for (int s = NS - 1; s >= 0; --s)
+            if (bphase(s) == k) return s;
+        return -1;
+    }
+};
+
 template <int L, int NB, bool INC>
 __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 {
     using P = FastPlan<L, NB, INC>;
+    using Q = BwPipe<L, NB, INC>;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
-    constexpr int FWT = P::fw_transposes_before(NS);  // transposes of the forward replay
-    __shared__ float lds[P::NSWAP > 0 ? 2 * kFastRowWords : 1];
+    __shared__ float2 lds[P::NSWAP > 0 ? 2 * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const FastCoords c = fast_coords<L>(t);
@@ -377,67 +422,84 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const int g_thr = c.eA < a.g_view.width ? c.slot * g_row + (int)(c.eA * a.g_view.se * 4) : kOob;
     const int gi_thr = c.eA < a.gi_view.width ? c.slot * gi_row + (int)(c.eA * a.gi_view.se * 4) : kOob;
 
-    auto transpose = [&](float v, int parity, int to_layout) -> float {
-        float *buf = lds + (parity & 1) * kFastRowWords;
-        buf[to_layout ? c.fA : c.fB] = v;
-        __syncthreads();
-        return buf[to_layout ? c.fB : c.fA];
-    };
+    auto group_ok = [&](int grp) { return grp >= 0 && grp * SLOTS + c.slot < rows_valid; };
+    auto load_x = [&](int grp) { return buf_load(x_rs, group_ok(grp) ? x_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row); };
+    auto load_g = [&](int grp) { return buf_load(g_rs, group_ok(grp) ? g_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * g_row); };
 
-    float nx = buf_load(x_rs, c.slot < rows_valid ? x_thr : kOob, 0);
-    float ng_ = buf_load(g_rs, c.slot < rows_valid ? g_thr : kOob, 0);
-    for (int grel = 0; grel < ng; ++grel) {
-        float v = nx, gv = ng_;
-        {
-            const bool ok = (grel + 1) * SLOTS + c.slot < rows_valid;
-            nx = buf_load(x_rs, ok ? x_thr : kOob, (grel + 1) * SLOTS * x_row);
-            ng_ = buf_load(g_rs, ok ? g_thr : kOob, (grel + 1) * SLOTS * g_row);
-        }
-        float act[NS];
-        // forward replay: act[s] = input of stage s, in the layout stage s runs in
-        static_for<0, NS>([&](auto S) {
-            constexpr int s = S;
-            constexpr int K = P::kind(s);
-            if constexpr (P::layout(s) != P::layout_before(s)) {
-                constexpr int par = P::fw_transposes_before(s) & 1;
-                constexpr int to_b = P::layout(s);
-                v = transpose(v, par, to_b);
+    // One pipelined iteration: forward replay of group it + 1 into `nxt`, reverse sweep of
+    // group it out of `cur`.  vF / gv enter holding the freshly loaded x and g.
+    auto iteration = [&](int it, float vF, float gv, float (&cur)[NS], float (&nxt)[NS]) {
+        static_for<0, Q::K + 1>([&](auto KK) {
+            constexpr int k = KK;
+            if constexpr (k >= 1) {
+                constexpr bool hasF = k <= Q::nF, hasB = k <= Q::nB;
+                constexpr int to_b = k & 1;  // both walks start in layout A and alternate
+                float2 *buf = lds + (k & 1) * kFastRowWords;
+                const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
+                if constexpr (hasF && hasB) buf[wr] = make_float2(vF, gv);
+                else if constexpr (hasF) buf[wr].x = vF;
+                else buf[wr].y = gv;
+                __syncthreads();
+                if constexpr (hasF && hasB) {
+                    const float2 v2 = buf[rd];
+                    vF = v2.x;
+                    gv = v2.y;
+                } else if constexpr (hasF) {
+                    vF = buf[rd].x;
+                } else {
+                    gv = buf[rd].y;
+                }
             }
-            act[s] = v;
-            if constexpr (s + 1 < NS) {
-                const float p = tb[s] * partner<K>(v, c.bperm_addr);
-                v = fmaf(ta[s], v, p);
-            }
+            constexpr int cf = Q::f_count(k), cb = Q::b_count(k);
+            constexpr int f0 = Q::f_first(k), b0 = Q::b_first(k);
+            static_for<0, (cf > cb ? cf : cb)>([&](auto J) {
+                constexpr int j = J;
+                if constexpr (j < cb) {
+                    // reverse stage s: uses the gradient before it passes through the stage
+                    constexpr int s = b0 - j;
+                    constexpr int Kd = P::kind(s);
+                    const float xs = cur[s];
+                    fmac_pinned(acc_self[s], gv, xs);
+                    if constexpr (Kd < 4) fmac_partner_dpp<Kd>(acc_cross[s], gv, xs);
+                    else fmac_pinned(acc_cross[s], gv, partner<Kd>(xs, c.bperm_addr));
+                    // d_x[r] = T[r][r] g[r] + T[1-r][r] g[1-r]; the partner forms the second
+                    // product from its own factor entry and it is fetched.
+                    const float m = tb[s] * gv;
+                    if constexpr (Kd < 4) gv = ta[s] * gv + partner<Kd>(m, c.bperm_addr);
+                    else gv = fmaf(ta[s], gv, partner<Kd>(m, c.bperm_addr));
+                }
+                if constexpr (j < cf) {
+                    constexpr int s = f0 + j;
+                    constexpr int Kd = P::kind(s);
+                    nxt[s] = vF;
+                    if constexpr (s + 1 < NS) {
+                        const float p = tb[s] * partner<Kd>(vF, c.bperm_addr);
+                        vF = fmaf(ta[s], vF, p);
+                    }
+                }
+            });
         });
-        // reverse sweep; the gradient arrives in layout A
-        static_for<0, NS>([&](auto S) {
-            constexpr int s = NS - 1 - S;
-            constexpr int K = P::kind(s);
-            if constexpr (P::layout(s) != P::layout_after(s)) {
-                constexpr int par = (FWT + P::bw_transposes_before(s)) & 1;
-                constexpr int to_b = P::layout(s);
-                gv = transpose(gv, par, to_b);
-            }
-            const float xs = act[s];
-            fmac_pinned(acc_self[s], gv, xs);
-            if constexpr (K < 4) fmac_partner_dpp<K>(acc_cross[s], gv, xs);
-            else fmac_pinned(acc_cross[s], gv, partner<K>(xs, c.bperm_addr));
-            // d_x[r] = T[r][r] g[r] + T[1-r][r] g[1-r]; the second product is formed by the
-            // partner from its own factor entry and fetched.
-            const float m = tb[s] * gv;
-            if constexpr (K < 4) gv = ta[s] * gv + partner<K>(m, c.bperm_addr);
-            else gv = fmaf(ta[s], gv, partner<K>(m, c.bperm_addr));
-        });
-        if constexpr (P::layout(0) != 0) {
-            constexpr int par = (FWT + P::bw_transposes_before(-1)) & 1;
-            gv = transpose(gv, par, 0);
-        }
-
-        const bool row_ok = grel * SLOTS + c.slot < rows_valid;
-        buf_store(gi_rs, row_ok ? gi_thr : kOob, grel * SLOTS * gi_row, gv);
+        const bool ok = group_ok(it);
+        const int soff = (it < 0 ? 0 : it) * SLOTS * gi_row;
+        buf_store(gi_rs, ok ? gi_thr : kOob, soff, gv);
         // input wider than n: those columns get a zero gradient
         for (int64_t j = n + c.eA; j < a.gi_view.width; j += n)
-            buf_store(gi_rs, row_ok ? c.slot * gi_row + (int)(j * a.gi_view.se * 4) : kOob, grel * SLOTS * gi_row, 0.0f);
+            buf_store(gi_rs, ok ? c.slot * gi_row + (int)(j * a.gi_view.se * 4) : kOob, soff, 0.0f);
+    };
+
+    float actP[NS], actQ[NS];
+    static_for<0, NS>([&](auto S) { actP[S] = 0.0f; });
+    // iteration it pairs group it + 1 (forward) with group it (reverse); it = -1 .. ng - 1
+    float x0 = load_x(0), gm = load_g(-1);
+    float x1 = load_x(1), gp = load_g(0);
+    for (int it = -1; it < ng; it += 2) {
+        const float xa = x0, ga = gm, xb = x1, gb = gp;
+        x0 = load_x(it + 3);
+        gm = load_g(it + 2);
+        x1 = load_x(it + 4);
+        gp = load_g(it + 3);
+        iteration(it, xa, ga, actP, actQ);
+        iteration(it + 1, xb, gb, actQ, actP);
     }
 
     // Recompute the coordinates from a laundered thread id: sharing them with the prologue
