@@ -347,7 +347,11 @@ struct BwPipe {
     static constexpr int NS = P::NS;
     static constexpr int nF = P::fw_transposes_before(NS);
     static constexpr int nB = P::bw_transposes_before(-1) + (P::layout(0) != 0 ? 1 : 0);
-    static constexpr int K = nF > nB ? nF : nB;  // phases 0..K; phase k >= 1 opens with transposes #k
+    // When the reverse walk ends in layout B and the forward walk has no transpose left to
+    // pair with, the closing transpose of the reverse walk is carried into the next
+    // iteration and rides on that iteration's first barrier.
+    static constexpr bool DEFER = P::layout(0) != 0 && nF < nB && nB >= 2;
+    static constexpr int K = DEFER ? nB - 1 : (nF > nB ? nF : nB);  // phases 0..K; phase k >= 1 opens with transposes #k
     // phase in which forward stage s / reverse stage s runs
     static constexpr int fphase(int s) { return P::fw_transposes_before(s + 1); }
     static constexpr int bphase(int s)
@@ -387,6 +391,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     using Q = BwPipe<L, NB, INC>;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
     __shared__ float2 lds[P::NSWAP > 0 ? 2 * kFastRowWords : 1];
+    __shared__ float lds_carry[Q::DEFER ? kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const FastCoords c = fast_coords<L>(t);
@@ -428,18 +433,33 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 
     // One pipelined iteration: forward replay of group it + 1 into `nxt`, reverse sweep of
     // group it out of `cur`.  vF / gv enter holding the freshly loaded x and g.
-    auto iteration = [&](int it, float vF, float gv, float (&cur)[NS], float (&nxt)[NS]) {
+    auto store_grad = [&](int grp, float gval) {
+        const bool ok = group_ok(grp);
+        const int soff = (grp < 0 ? 0 : grp) * SLOTS * gi_row;
+        buf_store(gi_rs, ok ? gi_thr : kOob, soff, gval);
+        // input wider than n: those columns get a zero gradient
+        for (int64_t j = n + c.eA; j < a.gi_view.width; j += n)
+            buf_store(gi_rs, ok ? c.slot * gi_row + (int)(j * a.gi_view.se * 4) : kOob, soff, 0.0f);
+    };
+
+    // `carry` holds the previous group's input gradient still in layout B (DEFER only)
+    // FLIP alternates between the two unrolled calls so that LDS buffers keep alternating
+    // across iterations when the number of phases is odd.
+    auto iteration = [&](auto FLIP, int it, float vF, float gv, float &carry, float (&cur)[NS], float (&nxt)[NS]) {
+        constexpr int flip = decltype(FLIP)::value;
         static_for<0, Q::K + 1>([&](auto KK) {
             constexpr int k = KK;
             if constexpr (k >= 1) {
                 constexpr bool hasF = k <= Q::nF, hasB = k <= Q::nB;
                 constexpr int to_b = k & 1;  // both walks start in layout A and alternate
-                float2 *buf = lds + (k & 1) * kFastRowWords;
+                float2 *buf = lds + ((k + flip * Q::K) & 1) * kFastRowWords;
                 const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
                 if constexpr (hasF && hasB) buf[wr] = make_float2(vF, gv);
                 else if constexpr (hasF) buf[wr].x = vF;
                 else buf[wr].y = gv;
+                if constexpr (Q::DEFER && k == 1) lds_carry[c.fB] = carry;
                 __syncthreads();
+                if constexpr (Q::DEFER && k == 1) store_grad(it - 1, lds_carry[c.fA]);
                 if constexpr (hasF && hasB) {
                     const float2 v2 = buf[rd];
                     vF = v2.x;
@@ -479,12 +499,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 }
             });
         });
-        const bool ok = group_ok(it);
-        const int soff = (it < 0 ? 0 : it) * SLOTS * gi_row;
-        buf_store(gi_rs, ok ? gi_thr : kOob, soff, gv);
-        // input wider than n: those columns get a zero gradient
-        for (int64_t j = n + c.eA; j < a.gi_view.width; j += n)
-            buf_store(gi_rs, ok ? c.slot * gi_row + (int)(j * a.gi_view.se * 4) : kOob, soff, 0.0f);
+        if constexpr (Q::DEFER) carry = gv;
+        else store_grad(it, gv);
     };
 
     float actP[NS], actQ[NS];
@@ -492,14 +508,17 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // iteration it pairs group it + 1 (forward) with group it (reverse); it = -1 .. ng - 1
     float x0 = load_x(0), gm = load_g(-1);
     float x1 = load_x(1), gp = load_g(0);
-    for (int it = -1; it < ng; it += 2) {
+    float carry = 0.0f;
+    // with a deferred closing transpose one more (empty) iteration flushes the last group
+    const int it_end = Q::DEFER ? ng + 1 : ng;
+    for (int it = -1; it < it_end; it += 2) {
         const float xa = x0, ga = gm, xb = x1, gb = gp;
         x0 = load_x(it + 3);
         gm = load_g(it + 2);
         x1 = load_x(it + 4);
         gp = load_g(it + 3);
-        iteration(it, xa, ga, actP, actQ);
-        iteration(it + 1, xb, gb, actQ, actP);
+        iteration(std::integral_constant<int, 0>{}, it, xa, ga, carry, actP, actQ);
+        iteration(std::integral_constant<int, 1>{}, it + 1, xb, gb, carry, actQ, actP);
     }
 
     // Recompute the coordinates from a laundered thread id: sharing them with the prologue
