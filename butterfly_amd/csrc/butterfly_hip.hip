@@ -329,7 +329,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
         pl.fast = true;
         pl.nchunks = 1;
         pl.chunk = pl.nstages;
-        pl.nparts = g.nwg * g.slots;
+        pl.nparts = g.nwg;
         pl.slot = 2 * n;
         pl.off_partials = 0;
         pl.total = align256((size_t)pl.nparts * p->nstacks * pl.nstages * pl.slot * e);

@@ -329,7 +329,7 @@ struct FastBwArgs {
     View g_view;
     float *g_in;
     View gi_view;              // columns in [n, width) are zero-filled
-    float *partial;            // (gridDim.x * SLOTS, S, NS, 2 n)
+    float *partial;            // (gridDim.x, S, NS, 2 n)
     int64_t batch;
     int64_t ngroups;
     int64_t groups_per_wg;
@@ -526,18 +526,44 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     int t2 = t;
     asm volatile("" : "+v"(t2));
     const FastCoords c2 = fast_coords<L>(t2);
-    float *part = a.partial + (((int64_t)blockIdx.x * SLOTS + c2.slot) * gridDim.y + stack) * NS * (2 * n);
-    static_for<0, NS>([&](auto S) {
-        constexpr int s = S;
-        constexpr int bit = P::bit(s);
-        constexpr int lay = P::layout(s);
-        const int e = lay ? c2.eB : c2.eA;
-        const int r = (e >> bit) & 1;
-        const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
-        float *d = part + (int64_t)s * (2 * n) + i * 4;
-        d[3 * r] = acc_self[s];    // dT[r][r]
-        d[r + 1] = acc_cross[s];   // dT[r][1 - r]
-    });
+    // One partial slice per workgroup.  When the workgroup holds several rows at once
+    // (n < 1024) the per-row-slot sums are first added through LDS in ascending slot order.
+    float *part = a.partial + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * (2 * n);
+    if constexpr (SLOTS == 1) {
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            constexpr int bit = P::bit(s);
+            constexpr int lay = P::layout(s);
+            const int e = lay ? c2.eB : c2.eA;
+            const int r = (e >> bit) & 1;
+            const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
+            float *d = part + (int64_t)s * (2 * n) + i * 4;
+            d[3 * r] = acc_self[s];    // dT[r][r]
+            d[r + 1] = acc_cross[s];   // dT[r][1 - r]
+        });
+    } else {
+        __shared__ float red[2 * 1024];
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            constexpr int bit = P::bit(s);
+            constexpr int lay = P::layout(s);
+            const int e = lay ? c2.eB : c2.eA;
+            __syncthreads();
+            red[(c2.slot * n + e) * 2 + 0] = acc_self[s];
+            red[(c2.slot * n + e) * 2 + 1] = acc_cross[s];
+            __syncthreads();
+            if (t2 < 2 * n) {
+                const int eo = t2 >> 1, j = t2 & 1;
+                float sum = red[t2];
+#pragma unroll 4
+                for (int sl = 1; sl < SLOTS; ++sl) sum += red[sl * 2 * n + t2];
+                const int r = (eo >> bit) & 1;
+                const int i = ((eo >> (bit + 1)) << bit) | (eo & ((1 << bit) - 1));
+                // j = 0: dT[r][r], j = 1: dT[r][1 - r]
+                part[(int64_t)s * (2 * n) + i * 4 + (j ? r + 1 : 3 * r)] = sum;
+            }
+        });
+    }
 }
 
 }  // namespace bf
