@@ -22,6 +22,7 @@ if ROOT not in sys.path:
 
 METRIC = "butterfly_multiply fwd+bwd GB/s & % HBM peak, batch 16384 n=1024 fp32"
 HBM_PEAK_GBS = 8000.0
+BW_TRAFFIC_BYTES = 289.4e6
 
 BATCH, NSTACKS, LOG_N, NBLOCKS, INCREASING = 16384, 1, 10, 2, False
 
@@ -72,6 +73,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run plain 64 MiB device copies (a kernel of known traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU; --gpus must be 1 (rows shard trivially, see DESIGN.md)")
@@ -95,6 +99,11 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    if args.calibrate_copy:
+        dst = torch.empty_like(x)
+        for _ in range(5):
+            dst.copy_(x)
+        torch.cuda.synchronize()
     fw_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     bw_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     torch.cuda.synchronize()
@@ -126,7 +135,9 @@ def main():
         "fw_GBps": fw_b / (fw_ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "kernel": "butterfly_multiply_bw (main kernel + partial-sum reduce)",
                      "achieved": bw_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bw_gbs / HBM_PEAK_GBS,
-                     "traffic": None},
+                     # HBM bytes per backward call (main kernel + reduce) from rocprofv3 FETCH_SIZE /
+                     # WRITE_SIZE scaled by a 64 MiB copy; see profiles/butterfly_fw_bw_cfg2_hbm_traffic.md
+                     "traffic": BW_TRAFFIC_BYTES},
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
