@@ -15,6 +15,7 @@
 #include "common.hpp"
 #include "generic.hpp"
 #include "fast.hpp"
+#include "high.hpp"
 
 namespace {
 
@@ -145,8 +146,16 @@ constexpr int kNumCU = 256;     // MI355X
 constexpr int kFastFwRows = BF_FAST_FW_ROWS;  // row groups in flight per forward workgroup
 constexpr int kFastFwWgPerCu = BF_FAST_FW_WGS;  // forward workgroups resident per compute unit
 
-// ---- twiddle-stationary fast path (float, base-2, n <= 1024, nblocks <= 2) ------------------
-
+// ---- register-resident multi-pass path (float, base-2, n <= 4096) ---------------------------
+//
+// The flat stage list is cut into passes, one kernel launch each:
+//   * a LOW pass runs up to 20 consecutive stages that pair element bits below 10 with the
+//     twiddle-stationary kernels of fast.hpp (rows longer than 1024 are treated as
+//     independent 1024-element chunks);
+//   * a HIGH pass runs the stages that pair bits 10 and 11 with the streaming kernels of
+//     high.hpp.
+// n <= 1024 with one or two blocks is a single LOW pass: each row is read once and written
+// once.  Longer schedules pass the activation through the workspace between launches.
 
 // Largest byte offset one workgroup forms into an operand with these strides; the fast
 // kernels address through 32-bit offsets and need it below 2 GiB.
@@ -156,16 +165,92 @@ bool span_ok(const int64_t stride[3], int64_t rows, int64_t width)
     return bytes < 2147483000.0;
 }
 
+struct Pass {
+    int t0, t1;     // stage range [t0, t1)
+    bool high;
+    int L, NB;      // LOW: FastPlan<L, NB, inc> on chunks of 2^L elements
+    bool inc;
+    int H, NST, PAT;  // HIGH: H high bits, NST stages, bit hb of PAT = high bit paired by stage s
+};
+
+struct PassPlan {
+    bool ok = false;
+    int npass = 0;
+    Pass pass[40];
+    int64_t chunks = 1;  // 1024-element chunks per row (LOW passes)
+    int max_nst = 0;
+};
+
+int stage_bit(const bf_problem *p, int t)
+{
+    const int L = (int)p->log_n;
+    const int block = t / L, idx = t % L;
+    const bool inc = (p->increasing_stride != 0) != ((block & 1) != 0);
+    return inc ? idx : L - 1 - idx;
+}
+
+PassPlan build_passes(const bf_problem *p, bool base4)
+{
+    PassPlan pl;
+    const int L = (int)p->log_n;
+    if (base4 || p->dtype != BF_F32 || L < 1 || L > 12 || p->nblocks < 1 || p->batch <= 0 || p->nstacks <= 0 ||
+        p->input_size <= 0 || p->output_size <= 0)
+        return pl;
+    const int NS = L * (int)p->nblocks;
+    if (L <= 10) {
+        for (int k = 0; k < p->nblocks; k += 2) {
+            if (pl.npass == 40) return pl;
+            Pass &q = pl.pass[pl.npass++];
+            q = Pass{};
+            q.NB = std::min<int>(2, (int)p->nblocks - k);
+            q.t0 = k * L;
+            q.t1 = (k + q.NB) * L;
+            q.L = L;
+            q.inc = (p->increasing_stride != 0) != ((k & 1) != 0);
+        }
+    } else {
+        pl.chunks = (int64_t)1 << (L - 10);
+        int t = 0;
+        while (t < NS) {
+            if (pl.npass == 40) return pl;
+            Pass &q = pl.pass[pl.npass++];
+            q = Pass{};
+            q.t0 = t;
+            const bool high = stage_bit(p, t) >= 10;
+            int u = t;
+            while (u < NS && (stage_bit(p, u) >= 10) == high) ++u;
+            q.t1 = u;
+            q.high = high;
+            if (high) {
+                q.H = L - 10;
+                q.NST = u - t;
+                if (q.NST > 2 * q.H) return pl;
+                for (int s = 0; s < q.NST; ++s) q.PAT |= (stage_bit(p, t + s) - 10) << s;
+            } else {
+                q.L = 10;
+                if ((u - t) != 10 && (u - t) != 20) return pl;
+                q.NB = (u - t) / 10;
+                q.inc = stage_bit(p, t) == 0;
+            }
+            t = u;
+        }
+    }
+    for (int k = 0; k < pl.npass; ++k) pl.max_nst = std::max(pl.max_nst, pl.pass[k].t1 - pl.pass[k].t0);
+    pl.ok = true;
+    return pl;
+}
+
 struct FastGrid {
     int64_t slots, ngroups, nwg, groups_per_wg;
 };
 
-FastGrid fast_grid(const bf_problem *p, int rows_in_flight, int wg_per_cu)
+// Row-group partition of a LOW pass: `lanes` independent (stack, chunk) columns share the CUs.
+FastGrid fast_grid(int64_t batch, int Lk, int64_t lanes, int rows_in_flight, int wg_per_cu)
 {
     FastGrid g;
-    g.slots = 1024 >> p->log_n;
-    g.ngroups = (p->batch + g.slots - 1) / g.slots;
-    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * wg_per_cu / p->nstacks);
+    g.slots = 1024 >> Lk;
+    g.ngroups = (batch + g.slots - 1) / g.slots;
+    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * wg_per_cu / lanes);
     const int64_t iters = (g.ngroups + rows_in_flight - 1) / rows_in_flight;
     g.nwg = std::min(want, iters);
     g.groups_per_wg = ((iters + g.nwg - 1) / g.nwg) * rows_in_flight;
@@ -173,16 +258,37 @@ FastGrid fast_grid(const bf_problem *p, int rows_in_flight, int wg_per_cu)
     return g;
 }
 
-bool fast_applicable(const bf_problem *p, bool base4, bool backward)
+// Row partition of a HIGH pass (4 workgroups of 256 low positions per row partition and stack).
+struct HighGrid {
+    int64_t nparts, rows_per_wg;
+};
+
+HighGrid high_grid(int64_t batch, int64_t nstacks)
 {
-    if (base4 || p->dtype != BF_F32 || p->log_n < 1 || p->log_n > 10 || p->nblocks < 1 || p->nblocks > 2 ||
-        p->batch <= 0 || p->nstacks <= 0 || p->input_size <= 0 || p->output_size <= 0)
-        return false;
+    HighGrid g;
+    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * 2 / nstacks);
+    g.nparts = std::min(want, batch);
+    g.rows_per_wg = (batch + g.nparts - 1) / g.nparts;
+    g.nparts = (batch + g.rows_per_wg - 1) / g.rows_per_wg;
+    return g;
+}
+
+// True when every pass can address its operands with 32-bit offsets.
+bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
+{
     const int64_t n = (int64_t)1 << p->log_n;
-    const FastGrid g = fast_grid(p, backward ? 1 : kFastFwRows, backward ? 1 : kFastFwWgPerCu);
-    const int64_t rows = (g.groups_per_wg + kFastFwRows) * g.slots;
-    if (!span_ok(p->input_stride, rows, n) || !span_ok(p->output_stride, rows, n)) return false;
-    if (backward && !span_ok(p->d_input_stride, rows, std::max(n, p->input_size))) return false;
+    int64_t rows = 0;
+    for (int k = 0; k < pl.npass; ++k) {
+        const Pass &q = pl.pass[k];
+        if (q.high) continue;
+        const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, backward ? 1 : kFastFwRows,
+                                     backward ? 1 : kFastFwWgPerCu);
+        rows = std::max(rows, (g.groups_per_wg + kFastFwRows + 2) * g.slots);
+    }
+    const int64_t dense[3] = {p->nstacks * n, n, 1};
+    if (!span_ok(p->input_stride, rows, n) || !span_ok(p->output_stride, rows, n) || !span_ok(dense, rows, n))
+        return false;
+    if (backward && !span_ok(p->d_input_stride, rows, n)) return false;
     return true;
 }
 
@@ -198,9 +304,9 @@ void launch_fast_bw_t(const FastBwArgs &a, dim3 grid, hipStream_t stream)
     hipLaunchKernelGGL((fast_bw_kernel<L, NB, INC>), grid, dim3(kFastThreads), 0, stream, a);
 }
 
-#define BF_FAST_DISPATCH(FN, ...)                                                        \
+#define BF_FAST_DISPATCH(FN, Q, ...)                                                     \
     do {                                                                                 \
-        const int key_ = (int)p->log_n * 4 + ((int)p->nblocks - 1) * 2 + (p->increasing_stride ? 1 : 0); \
+        const int key_ = (Q).L * 4 + ((Q).NB - 1) * 2 + ((Q).inc ? 1 : 0);               \
         switch (key_) {                                                                  \
             BF_FAST_CASES(FN, 1, __VA_ARGS__) BF_FAST_CASES(FN, 2, __VA_ARGS__)          \
             BF_FAST_CASES(FN, 3, __VA_ARGS__) BF_FAST_CASES(FN, 4, __VA_ARGS__)          \
@@ -216,23 +322,85 @@ void launch_fast_bw_t(const FastBwArgs &a, dim3 grid, hipStream_t stream)
     case LL * 4 + 2: FN<LL, 2, false>(__VA_ARGS__); break;      \
     case LL * 4 + 3: FN<LL, 2, true>(__VA_ARGS__); break;
 
-int fast_forward(const bf_problem *p, const void *tw, const void *input, void *output, hipStream_t stream)
+template <typename T, int H, int NST, int PAT>
+void launch_high_t(bool backward, const HighArgs &a, dim3 grid, hipStream_t stream)
+{
+    if (backward)
+        hipLaunchKernelGGL((high_bw_kernel<T, H, NST, PAT>), grid, dim3(kHighThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((high_fw_kernel<T, H, NST, PAT>), grid, dim3(kHighThreads), 0, stream, a);
+}
+
+template <typename T>
+int launch_high(const Pass &q, bool backward, const HighArgs &a, dim3 grid, hipStream_t stream)
+{
+    const int key = q.H * 1000 + q.NST * 100 + q.PAT;
+    switch (key) {
+        case 1 * 1000 + 1 * 100 + 0: launch_high_t<T, 1, 1, 0>(backward, a, grid, stream); break;
+        case 1 * 1000 + 2 * 100 + 0: launch_high_t<T, 1, 2, 0>(backward, a, grid, stream); break;
+        case 2 * 1000 + 2 * 100 + 2: launch_high_t<T, 2, 2, 2>(backward, a, grid, stream); break;  // bits 10, 11
+        case 2 * 1000 + 2 * 100 + 1: launch_high_t<T, 2, 2, 1>(backward, a, grid, stream); break;  // bits 11, 10
+        case 2 * 1000 + 4 * 100 + 6: launch_high_t<T, 2, 4, 6>(backward, a, grid, stream); break;  // 10, 11, 11, 10
+        default: return fail(BF_ERR_UNSUPPORTED, "no kernel for this high-bit stage pattern");
+    }
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
+}
+
+void fill_stage_table(int *dst, int cap, const Pass &q)
+{
+    for (int s = 0; s < cap; ++s) dst[s] = q.t0 + std::min(s, q.t1 - q.t0 - 1);
+}
+
+// Forward through the pass plan.  `scratch` holds one dense (B, S, n) activation when there
+// is more than one pass (passes run in place on it).
+int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, const void *input, void *output,
+                      void *scratch, const View &in_view, const View &out_view, int first, int last,
+                      hipStream_t stream)
 {
     const int64_t n = (int64_t)1 << p->log_n;
-    const FastGrid g = fast_grid(p, kFastFwRows, kFastFwWgPerCu);
-    FastFwArgs a;
-    a.tw = static_cast<const float *>(tw);
-    a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
-    a.in = static_cast<const float *>(input);
-    a.in_view = make_view(p->input_stride, std::min(p->input_size, n));
-    a.out = static_cast<float *>(output);
-    a.out_view = make_view(p->output_stride, p->output_size);
-    a.batch = p->batch;
-    a.ngroups = g.ngroups;
-    a.groups_per_wg = g.groups_per_wg;
-    const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks);
-    BF_FAST_DISPATCH(launch_fast_fw_t, a, grid, stream);
-    BF_HIP_CHECK(hipGetLastError());
+    const View dense = dense_view(p->nstacks, n);
+    for (int k = first; k < last; ++k) {
+        const Pass &q = pl.pass[k];
+        const void *src = k == first ? input : scratch;
+        void *dst = k == last - 1 ? output : scratch;
+        const View sv = k == first ? in_view : dense;
+        const View dv = k == last - 1 ? out_view : dense;
+        if (q.high) {
+            const HighGrid g = high_grid(p->batch, p->nstacks);
+            HighArgs a = {};
+            a.tw = tw;
+            a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
+            a.tw_stage_stride = (n / 2) * 4;
+            fill_stage_table(a.tw_stage, 4, q);
+            a.x_in = src;
+            a.x_view = sv;
+            a.x_out = dst;
+            a.xo_view = dv;
+            a.batch = p->batch;
+            a.rows_per_wg = g.rows_per_wg;
+            const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, 1024 / kHighThreads);
+            const int rc = launch_high<float>(q, false, a, grid, stream);
+            if (rc) return rc;
+        } else {
+            const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, kFastFwRows, kFastFwWgPerCu);
+            FastFwArgs a = {};
+            a.tw = static_cast<const float *>(tw);
+            a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
+            a.tw_stage_stride = (n / 2) * 4;
+            fill_stage_table(a.tw_stage, kFastMaxStages, q);
+            a.in = static_cast<const float *>(src);
+            a.in_view = sv;
+            a.out = static_cast<float *>(dst);
+            a.out_view = dv;
+            a.batch = p->batch;
+            a.ngroups = g.ngroups;
+            a.groups_per_wg = g.groups_per_wg;
+            const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)pl.chunks);
+            BF_FAST_DISPATCH(launch_fast_fw_t, q, a, grid, stream);
+            BF_HIP_CHECK(hipGetLastError());
+        }
+    }
     return BF_OK;
 }
 
@@ -275,8 +443,17 @@ int launch_generic_fw(const bf_problem *p, const Schedule &sc, int t0, int t1, c
     return BF_OK;
 }
 
+// Workspace of the forward call: one dense activation when the pass plan has several passes.
+size_t forward_workspace(const bf_problem *p, bool base4)
+{
+    const PassPlan mp = build_passes(p, base4);
+    if (!mp.ok || mp.npass <= 1 || !passes_addressable(p, mp, false)) return 0;
+    const int64_t n = (int64_t)1 << p->log_n;
+    return align256((size_t)p->batch * p->nstacks * n * elem_bytes(p->dtype));
+}
+
 int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, const void *input,
-            void *output, void *stream_)
+            void *output, void *workspace, size_t workspace_bytes, void *stream_)
 {
     int rc = check_problem(p, false);
     if (rc) return rc;
@@ -293,9 +470,17 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
             if (base4 && (p->log_n & 1) && !tw2) return fail(BF_ERR_INVALID, "twiddle2 is NULL");
         }
     }
-    if (fast_applicable(p, base4, false)) return fast_forward(p, tw2, input, output, stream);
     const View in_view = make_view(p->input_stride, std::min(p->input_size, n));
     const View out_view = make_view(p->output_stride, p->output_size);
+    const PassPlan mp = build_passes(p, base4);
+    if (mp.ok && passes_addressable(p, mp, false)) {
+        const size_t need = forward_workspace(p, base4);
+        if (need > 0 && (!workspace || workspace_bytes < need))
+            return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
+            return fail(BF_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+        return multipass_forward(p, mp, tw2, input, output, workspace, in_view, out_view, 0, mp.npass, stream);
+    }
     return launch_generic_fw(p, sc, 0, sc.per * sc.nblocks, tw2, tw4, input, in_view, output,
                              out_view, stream);
 }
@@ -311,7 +496,7 @@ struct BwPlan {
     size_t boundary_bytes;  // one (B, S, n) activation plane
     size_t off_boundaries, off_gbuf, off_partials, total;
     bool fits;
-    bool fast;          // single launch of the twiddle-stationary kernel
+    bool fast;          // register-resident pass plan
 };
 
 BwPlan plan_bw(const bf_problem *p, bool base4)
@@ -322,17 +507,31 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
     const size_t row_bytes = (size_t)n * e;
     const Schedule sc = make_schedule(p, base4);
     pl.nstages = sc.per * sc.nblocks;
-    if (fast_applicable(p, base4, true)) {
-        // one launch; partial sums from every (workgroup, row slot)
-        const FastGrid g = fast_grid(p, 1, 1);
+    const PassPlan mp = build_passes(p, base4);
+    if (mp.ok && passes_addressable(p, mp, true)) {
+        // boundaries: the activation entering every pass after the first; one gradient plane
+        // that the passes update in place; partial slices sized for the widest pass.
         pl.fits = true;
         pl.fast = true;
-        pl.nchunks = 1;
-        pl.chunk = pl.nstages;
-        pl.nparts = g.nwg;
+        pl.nchunks = mp.npass;
         pl.slot = 2 * n;
-        pl.off_partials = 0;
-        pl.total = align256((size_t)pl.nparts * p->nstacks * pl.nstages * pl.slot * e);
+        pl.boundary_bytes = align256((size_t)p->batch * p->nstacks * row_bytes);
+        int64_t nparts = 1;
+        for (int k = 0; k < mp.npass; ++k) {
+            const Pass &q = mp.pass[k];
+            const int64_t np = q.high ? high_grid(p->batch, p->nstacks).nparts
+                                      : fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1).nwg;
+            nparts = std::max(nparts, np);
+        }
+        pl.nparts = nparts;
+        size_t off = 0;
+        pl.off_boundaries = off;
+        off += mp.npass > 1 ? (size_t)(mp.npass - 1) * pl.boundary_bytes : 0;
+        pl.off_gbuf = off;
+        off += mp.npass > 1 ? pl.boundary_bytes : 0;
+        pl.off_partials = off;
+        off += align256((size_t)nparts * p->nstacks * mp.max_nst * pl.slot * e);
+        pl.total = off;
         return pl;
     }
     pl.fits = 2 * row_bytes <= kGenericBwLds;
@@ -429,29 +628,87 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     const View di_view = make_view(p->d_input_stride, p->input_size);
     const View dense = dense_view(p->nstacks, n);
     char *ws = static_cast<char *>(workspace);
+    const size_t e_bytes = elem_bytes(p->dtype);
 
     if (pl.nstages == 0) return launch_copy_pad(p, grad, g_view, d_input, di_view, stream);
 
     if (pl.fast) {
-        const FastGrid g = fast_grid(p, 1, 1);
-        FastBwArgs a;
-        a.tw = static_cast<const float *>(tw2);
-        a.tw_stack_stride = sc.tw2_stack_stride;
-        a.x_in = static_cast<const float *>(input);
-        a.x_view = x_view;
-        a.g_out = static_cast<const float *>(grad);
-        a.g_view = g_view;
-        a.g_in = static_cast<float *>(d_input);
-        a.gi_view = di_view;
-        a.partial = reinterpret_cast<float *>(ws + pl.off_partials);
-        a.batch = p->batch;
-        a.ngroups = g.ngroups;
-        a.groups_per_wg = g.groups_per_wg;
-        const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks);
-        BF_FAST_DISPATCH(launch_fast_bw_t, a, grid, stream);
-        BF_HIP_CHECK(hipGetLastError());
-        rc = launch_reduce(p, sc, 0, pl.nstages, pl.nparts, ws + pl.off_partials, pl.slot, d_tw2, d_tw4, stream);
-        if (rc) return rc;
+        const PassPlan mp = build_passes(p, base4);
+        const int P = mp.npass;
+        auto boundary = [&](int k) { return ws + pl.off_boundaries + (size_t)(k - 1) * pl.boundary_bytes; };
+        // forward replay: boundary k = activation entering pass k (k >= 1)
+        for (int k = 0; k + 1 < P; ++k) {
+            rc = multipass_forward(p, mp, tw2, k == 0 ? input : boundary(k), boundary(k + 1), nullptr,
+                                   k == 0 ? x_view : dense, dense, k, k + 1, stream);
+            if (rc) return rc;
+        }
+        const View dn_view = make_view(p->d_input_stride, std::min(p->input_size, n));
+        for (int k = P - 1; k >= 0; --k) {
+            const Pass &q = mp.pass[k];
+            const void *xin = k == 0 ? input : boundary(k);
+            const View xv = k == 0 ? x_view : dense;
+            const void *gout = k == P - 1 ? grad : ws + pl.off_gbuf;
+            const View gv = k == P - 1 ? g_view : dense;
+            void *gin = k == 0 ? d_input : ws + pl.off_gbuf;
+            const View giv = k == 0 ? dn_view : dense;
+            int64_t nparts = 0;
+            if (q.high) {
+                const HighGrid g = high_grid(p->batch, p->nstacks);
+                HighArgs a = {};
+                a.tw = tw2;
+                a.tw_stack_stride = sc.tw2_stack_stride;
+                a.tw_stage_stride = (n / 2) * 4;
+                fill_stage_table(a.tw_stage, 4, q);
+                a.x_in = xin;
+                a.x_view = xv;
+                a.g_out = gout;
+                a.g_view = gv;
+                a.g_in = gin;
+                a.gi_view = giv;
+                a.partial = ws + pl.off_partials;
+                a.partial_slot = pl.slot;
+                a.batch = p->batch;
+                a.rows_per_wg = g.rows_per_wg;
+                nparts = g.nparts;
+                const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, 1024 / kHighThreads);
+                rc = launch_high<float>(q, true, a, grid, stream);
+                if (rc) return rc;
+            } else {
+                const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1);
+                FastBwArgs a = {};
+                a.tw = static_cast<const float *>(tw2);
+                a.tw_stack_stride = sc.tw2_stack_stride;
+                a.tw_stage_stride = (n / 2) * 4;
+                fill_stage_table(a.tw_stage, kFastMaxStages, q);
+                a.partial_slot = pl.slot;
+                a.x_in = static_cast<const float *>(xin);
+                a.x_view = xv;
+                a.g_out = static_cast<const float *>(gout);
+                a.g_view = gv;
+                a.g_in = static_cast<float *>(gin);
+                a.gi_view = giv;
+                a.partial = reinterpret_cast<float *>(ws + pl.off_partials);
+                a.batch = p->batch;
+                a.ngroups = g.ngroups;
+                a.groups_per_wg = g.groups_per_wg;
+                nparts = g.nwg;
+                const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)mp.chunks);
+                BF_FAST_DISPATCH(launch_fast_bw_t, q, a, grid, stream);
+                BF_HIP_CHECK(hipGetLastError());
+            }
+            rc = launch_reduce(p, sc, q.t0, q.t1, nparts, ws + pl.off_partials, pl.slot, d_tw2, d_tw4, stream);
+            if (rc) return rc;
+        }
+        if (p->input_size > n) {
+            // input wider than n: those columns get a zero gradient
+            View tail = di_view;
+            tail.width = p->input_size - n;
+            View none = tail;
+            none.width = 0;
+            char *base = static_cast<char *>(d_input) + (size_t)n * p->d_input_stride[2] * e_bytes;
+            rc = launch_copy_pad(p, base, none, base, tail, stream);
+            if (rc) return rc;
+        }
         return BF_OK;
     }
 
@@ -509,10 +766,16 @@ int bf_hip_version(void) { return HIP_VERSION; }
 
 const char *bf_last_error(void) { return g_last_error.c_str(); }
 
-int bf_butterfly_multiply_fw(const bf_problem *p, const void *twiddle, const void *input,
-                             void *output, void *stream)
+size_t bf_butterfly_multiply_fw_workspace_bytes(const bf_problem *p)
 {
-    return forward(p, false, twiddle, nullptr, input, output, stream);
+    if (check_problem(p, false)) return 0;
+    return forward_workspace(p, false);
+}
+
+int bf_butterfly_multiply_fw(const bf_problem *p, const void *twiddle, const void *input,
+                             void *output, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return forward(p, false, twiddle, nullptr, input, output, workspace, workspace_bytes, stream);
 }
 
 size_t bf_butterfly_multiply_bw_workspace_bytes(const bf_problem *p)
@@ -532,7 +795,7 @@ int bf_butterfly_multiply_bw(const bf_problem *p, const void *twiddle, const voi
 int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4, const void *twiddle2,
                                    const void *input, void *output, void *stream)
 {
-    return forward(p, true, twiddle2, twiddle4, input, output, stream);
+    return forward(p, true, twiddle2, twiddle4, input, output, nullptr, 0, stream);
 }
 
 size_t bf_butterfly_multiply_base4_bw_workspace_bytes(const bf_problem *p)

@@ -107,7 +107,9 @@ Tensor butterfly_multiply_fw(const Tensor twiddle, const Tensor input, bool incr
     if (output_size_val < s.n) output = output.slice(2, 0, output_size_val);
     bf_problem p = make_problem(s, x, increasing_stride, output_size_val, "butterfly_multiply_fw");
     set_strides(p.output_stride, output);
-    check_rc(bf_butterfly_multiply_fw(&p, tw.data_ptr(), x.data_ptr(), output.data_ptr(),
+    const size_t ws_bytes = bf_butterfly_multiply_fw_workspace_bytes(&p);
+    Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+    check_rc(bf_butterfly_multiply_fw(&p, tw.data_ptr(), x.data_ptr(), output.data_ptr(), ws.data_ptr(), ws_bytes,
                                       current_stream()),
              "butterfly_multiply_fw");
     return output;

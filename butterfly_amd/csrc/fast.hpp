@@ -208,9 +208,16 @@ __device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, int voff, in
     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
 }
 
+constexpr int kFastMaxStages = 20;
+
+// Rows longer than 1024 are handled as independent 1024-element chunks (blockIdx.z) for the
+// stages that pair bits below 10: chunk c of stage s uses the factor slice starting at pair
+// c * 512, and its d_twiddle sums land at the same place in the partial slice.
 struct FastFwArgs {
-    const float *tw;           // factors of the first block of this launch, stack 0
+    const float *tw;           // twiddle tensor, stack 0
     int64_t tw_stack_stride;
+    int64_t tw_stage_stride;   // floats between consecutive stages: (n_full / 2) * 4
+    int tw_stage[kFastMaxStages];  // global stage number of every local stage
     const float *in;
     View in_view;
     float *out;
@@ -231,11 +238,13 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     __shared__ float lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
+    const int chunk = blockIdx.z;
     const FastCoords c = fast_coords<L>(t);
+    const int col = (chunk << L) + c.eA;  // column of this thread's element in the full row
 
     float ta[NS], tb[NS];
     {
-        const float *twp = a.tw + stack * a.tw_stack_stride;
+        const float *twp = a.tw + stack * a.tw_stack_stride + (int64_t)chunk * (n / 2) * 4;
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
             constexpr int bit = P::bit(s);
@@ -243,7 +252,7 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
             const int e = lay ? c.eB : c.eA;
             const int r = (e >> bit) & 1;
             const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
-            const float *T = twp + ((int64_t)s * (n / 2) + i) * 4;
+            const float *T = twp + a.tw_stage[s] * a.tw_stage_stride + i * 4;
             ta[s] = T[3 * r];   // T[r][r]
             tb[s] = T[r + 1];   // T[r][1 - r]
         });
@@ -258,8 +267,8 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     const __amdgpu_buffer_rsrc_t out_rs = make_rsrc(a.out + g0 * SLOTS * a.out_view.sb + stack * a.out_view.ss);
     const int in_row = (int)(a.in_view.sb * 4), out_row = (int)(a.out_view.sb * 4);
     // thread-constant part of the offsets; the row group adds a wave-uniform part
-    const int in_thr = c.eA < a.in_view.width ? c.slot * in_row + (int)(c.eA * a.in_view.se * 4) : kOob;
-    const int out_thr = c.eA < a.out_view.width ? c.slot * out_row + (int)(c.eA * a.out_view.se * 4) : kOob;
+    const int in_thr = col < a.in_view.width ? c.slot * in_row + (int)(col * a.in_view.se * 4) : kOob;
+    const int out_thr = col < a.out_view.width ? c.slot * out_row + (int)(col * a.out_view.se * 4) : kOob;
 
     auto load_rows = [&](int grel, float (&v)[R]) {
 #pragma unroll
@@ -323,13 +332,16 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
 struct FastBwArgs {
     const float *tw;
     int64_t tw_stack_stride;
+    int64_t tw_stage_stride;
+    int tw_stage[kFastMaxStages];
+    int64_t partial_slot;      // floats per stage in a partial slice: 2 * n_full
     const float *x_in;
     View x_view;
     const float *g_out;
     View g_view;
     float *g_in;
-    View gi_view;              // columns in [n, width) are zero-filled
-    float *partial;            // (gridDim.x, S, NS, 2 n)
+    View gi_view;
+    float *partial;            // (gridDim.x, S, NS, partial_slot)
     int64_t batch;
     int64_t ngroups;
     int64_t groups_per_wg;
@@ -394,11 +406,13 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     __shared__ float lds_carry[Q::DEFER ? kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
+    const int chunk = blockIdx.z;
     const FastCoords c = fast_coords<L>(t);
+    const int col = (chunk << L) + c.eA;  // column of this thread's element in the full row
 
     float ta[NS], tb[NS], acc_self[NS], acc_cross[NS];
     {
-        const float *twp = a.tw + stack * a.tw_stack_stride;
+        const float *twp = a.tw + stack * a.tw_stack_stride + (int64_t)chunk * (n / 2) * 4;
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
             constexpr int bit = P::bit(s);
@@ -406,7 +420,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             const int e = lay ? c.eB : c.eA;
             const int r = (e >> bit) & 1;
             const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
-            const float *T = twp + ((int64_t)s * (n / 2) + i) * 4;
+            const float *T = twp + a.tw_stage[s] * a.tw_stage_stride + i * 4;
             ta[s] = T[3 * r];
             tb[s] = T[r + 1];
             acc_self[s] = 0.0f;
@@ -423,9 +437,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const __amdgpu_buffer_rsrc_t g_rs = make_rsrc(a.g_out + g0 * SLOTS * a.g_view.sb + stack * a.g_view.ss);
     const __amdgpu_buffer_rsrc_t gi_rs = make_rsrc(a.g_in + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
     const int x_row = (int)(a.x_view.sb * 4), g_row = (int)(a.g_view.sb * 4), gi_row = (int)(a.gi_view.sb * 4);
-    const int x_thr = c.eA < a.x_view.width ? c.slot * x_row + (int)(c.eA * a.x_view.se * 4) : kOob;
-    const int g_thr = c.eA < a.g_view.width ? c.slot * g_row + (int)(c.eA * a.g_view.se * 4) : kOob;
-    const int gi_thr = c.eA < a.gi_view.width ? c.slot * gi_row + (int)(c.eA * a.gi_view.se * 4) : kOob;
+    const int x_thr = col < a.x_view.width ? c.slot * x_row + (int)(col * a.x_view.se * 4) : kOob;
+    const int g_thr = col < a.g_view.width ? c.slot * g_row + (int)(col * a.g_view.se * 4) : kOob;
+    const int gi_thr = col < a.gi_view.width ? c.slot * gi_row + (int)(col * a.gi_view.se * 4) : kOob;
 
     auto group_ok = [&](int grp) { return grp >= 0 && grp * SLOTS + c.slot < rows_valid; };
     auto load_x = [&](int grp) { return buf_load(x_rs, group_ok(grp) ? x_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row); };
@@ -437,9 +451,6 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         const bool ok = group_ok(grp);
         const int soff = (grp < 0 ? 0 : grp) * SLOTS * gi_row;
         buf_store(gi_rs, ok ? gi_thr : kOob, soff, gval);
-        // input wider than n: those columns get a zero gradient
-        for (int64_t j = n + c.eA; j < a.gi_view.width; j += n)
-            buf_store(gi_rs, ok ? c.slot * gi_row + (int)(j * a.gi_view.se * 4) : kOob, soff, 0.0f);
     };
 
     // `carry` holds the previous group's input gradient still in layout B (DEFER only)
@@ -528,7 +539,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const FastCoords c2 = fast_coords<L>(t2);
     // One partial slice per workgroup.  When the workgroup holds several rows at once
     // (n < 1024) the per-row-slot sums are first added through LDS in ascending slot order.
-    float *part = a.partial + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * (2 * n);
+    float *part = a.partial + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * a.partial_slot +
+                  (int64_t)chunk * (n / 2) * 4;
     if constexpr (SLOTS == 1) {
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
@@ -537,7 +549,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             const int e = lay ? c2.eB : c2.eA;
             const int r = (e >> bit) & 1;
             const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
-            float *d = part + (int64_t)s * (2 * n) + i * 4;
+            float *d = part + (int64_t)s * a.partial_slot + i * 4;
             d[3 * r] = acc_self[s];    // dT[r][r]
             d[r + 1] = acc_cross[s];   // dT[r][1 - r]
         });
@@ -560,7 +572,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 const int r = (eo >> bit) & 1;
                 const int i = ((eo >> (bit + 1)) << bit) | (eo & ((1 << bit) - 1));
                 // j = 0: dT[r][r], j = 1: dT[r][1 - r]
-                part[(int64_t)s * (2 * n) + i * 4 + (j ? r + 1 : 3 * r)] = sum;
+                part[(int64_t)s * a.partial_slot + i * 4 + (j ? r + 1 : 3 * r)] = sum;
             }
         });
     }

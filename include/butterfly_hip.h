@@ -63,7 +63,11 @@ const char *bf_last_error(void);
  * csrc/cpu/butterfly_cpu.cpp:17-66, csrc/cuda/butterfly_cuda.cu:349-416).
  *   twiddle (S, nb, log_n, n/2, 2, 2) dense.                                          */
 int bf_butterfly_multiply_fw(const bf_problem *p, const void *twiddle, const void *input,
-                             void *output, void *stream);
+                             void *output, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Workspace the forward call needs, in bytes: zero when the whole schedule runs in one
+ * launch (n <= 1024 with at most two blocks), one (B, S, n) activation otherwise.          */
+size_t bf_butterfly_multiply_fw_workspace_bytes(const bf_problem *p);
 
 /* Workspace the backward call needs for this problem, in bytes. */
 size_t bf_butterfly_multiply_bw_workspace_bytes(const bf_problem *p);

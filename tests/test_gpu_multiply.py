@@ -94,6 +94,42 @@ def test_register_resident_kernels_all_sizes(L):
                 assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL, (L, nb, inc, B, S, I, O)
 
 
+MULTIPASS_CASES = [
+    # B, S, L, nb, I, O, inc -- more than two blocks and rows of 2048 / 4096 (chunked + high-bit passes)
+    (40, 2, 9, 3, None, None, True),
+    (40, 2, 9, 4, None, None, False),
+    (33, 1, 10, 5, 1000, 900, False),
+    (21, 2, 11, 1, None, None, True),
+    (21, 2, 11, 1, None, None, False),
+    (21, 1, 11, 2, None, None, True),
+    (21, 1, 11, 2, 2000, 1500, False),
+    (13, 2, 12, 1, None, None, True),
+    (13, 2, 12, 1, None, None, False),
+    (13, 1, 12, 2, None, None, True),
+    (13, 1, 12, 2, None, None, False),
+    (10, 2, 12, 3, 4092, 2046, True),
+    (10, 2, 12, 3, 2 * 4096 + 7, 4091, False),
+    (300, 1, 12, 2, None, None, True),
+]
+
+
+@pytest.mark.parametrize("case", MULTIPASS_CASES, ids=lambda c: f"B{c[0]}-S{c[1]}-L{c[2]}-nb{c[3]}-I{c[4]}-O{c[5]}-inc{int(c[6])}")
+def test_multi_launch_schedules(case):
+    from butterfly_amd import _capi
+    B, S, L, nb, I, O, inc = case
+    say("multipass case", case)
+    rng = np.random.default_rng(900 + L * 13 + nb)
+    tw, x, g = make_case(rng, np.float32, B, S, L, nb, I, O)
+    y_ref = oracle.butterfly_fw(tw, x, inc, O)
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+    y = _capi.multiply_fw(dev(tw), dev(x), inc, O)
+    dtw, dx = _capi.multiply_bw(dev(tw), dev(x), dev(g), inc)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
 def test_c_abi_strided_operands():
     """Stride-0 stack broadcast (what Butterfly.pre_process hands over), a transposed input
     and a non-contiguous gradient."""

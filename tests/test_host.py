@@ -21,7 +21,7 @@ def header_functions():
 def test_library_exports_every_declared_symbol():
     from butterfly_amd import _capi
     names = header_functions()
-    assert len(names) >= 9
+    assert len(names) >= 10
     assert sorted(_capi.SYMBOLS) == names
     L = _capi.lib()
     for name in names:
@@ -37,17 +37,17 @@ def test_c_abi_rejects_bad_problems_on_the_host():
     p.dtype, p.batch, p.nstacks, p.log_n, p.nblocks = 7, 1, 1, 3, 1
     p.input_size = p.output_size = 8
     null = ctypes.c_void_p(0)
-    assert L.bf_butterfly_multiply_fw(ctypes.byref(p), null, null, null, null) == -1
+    assert L.bf_butterfly_multiply_fw(ctypes.byref(p), null, null, null, null, 0, null) == -1
     assert b"dtype" in L.bf_last_error()
     p.dtype, p.output_size = 0, 9
-    assert L.bf_butterfly_multiply_fw(ctypes.byref(p), null, null, null, null) == -1
+    assert L.bf_butterfly_multiply_fw(ctypes.byref(p), null, null, null, null, 0, null) == -1
     assert b"output_size" in L.bf_last_error()
     p.output_size, p.log_n = 8, 31
-    assert L.bf_butterfly_multiply_fw(ctypes.byref(p), null, null, null, null) == -1
+    assert L.bf_butterfly_multiply_fw(ctypes.byref(p), null, null, null, null, 0, null) == -1
     p.log_n = 3
     p.input_stride[2] = -1
     assert L.bf_butterfly_multiply_bw(ctypes.byref(p), null, null, null, null, null, null, 0, null) == -1
-    assert L.bf_butterfly_multiply_fw(None, null, null, null, null) == -1
+    assert L.bf_butterfly_multiply_fw(None, null, null, null, null, 0, null) == -1
     # workspace query is pure host arithmetic
     p.input_stride[2] = 1
     p.batch, p.log_n, p.nblocks = 16384, 10, 2
