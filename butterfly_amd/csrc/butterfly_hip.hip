@@ -145,8 +145,9 @@ constexpr int kNumCU = 256;     // MI355X
 #endif
 constexpr int kFastFwRows = BF_FAST_FW_ROWS;  // row groups in flight per forward workgroup
 constexpr int kFastFwWgPerCu = BF_FAST_FW_WGS;  // forward workgroups resident per compute unit
+constexpr int kFastFwRowsComplex = 2;       // complex64: half as many (LDS and registers double)
 
-// ---- register-resident multi-pass path (float, base-2, n <= 4096) ---------------------------
+// ---- register-resident multi-pass path (float and complex64, base-2, n <= 4096) ---------------------------
 //
 // The flat stage list is cut into passes, one kernel launch each:
 //   * a LOW pass runs up to 20 consecutive stages that pair element bits below 10 with the
@@ -159,9 +160,9 @@ constexpr int kFastFwWgPerCu = BF_FAST_FW_WGS;  // forward workgroups resident p
 
 // Largest byte offset one workgroup forms into an operand with these strides; the fast
 // kernels address through 32-bit offsets and need it below 2 GiB.
-bool span_ok(const int64_t stride[3], int64_t rows, int64_t width)
+bool span_ok(const int64_t stride[3], int64_t rows, int64_t width, size_t elem)
 {
-    const double bytes = 4.0 * ((double)rows * (double)stride[0] + (double)width * (double)stride[2]);
+    const double bytes = (double)elem * ((double)rows * (double)stride[0] + (double)width * (double)stride[2]);
     return bytes < 2147483000.0;
 }
 
@@ -193,16 +194,18 @@ PassPlan build_passes(const bf_problem *p, bool base4)
 {
     PassPlan pl;
     const int L = (int)p->log_n;
-    if (base4 || p->dtype != BF_F32 || L < 1 || L > 12 || p->nblocks < 1 || p->batch <= 0 || p->nstacks <= 0 ||
+    if (base4 || L < 1 || L > 12 || p->nblocks < 1 || p->batch <= 0 || p->nstacks <= 0 ||
         p->input_size <= 0 || p->output_size <= 0)
         return pl;
     const int NS = L * (int)p->nblocks;
+    // complex64 needs twice the registers per stage: one block per LOW pass
+    const int max_nb = p->dtype == BF_C64 ? 1 : 2;
     if (L <= 10) {
-        for (int k = 0; k < p->nblocks; k += 2) {
+        for (int k = 0; k < p->nblocks; k += max_nb) {
             if (pl.npass == 40) return pl;
             Pass &q = pl.pass[pl.npass++];
             q = Pass{};
-            q.NB = std::min<int>(2, (int)p->nblocks - k);
+            q.NB = std::min<int>(max_nb, (int)p->nblocks - k);
             q.t0 = k * L;
             q.t1 = (k + q.NB) * L;
             q.L = L;
@@ -218,7 +221,7 @@ PassPlan build_passes(const bf_problem *p, bool base4)
             q.t0 = t;
             const bool high = stage_bit(p, t) >= 10;
             int u = t;
-            while (u < NS && (stage_bit(p, u) >= 10) == high) ++u;
+            while (u < NS && (stage_bit(p, u) >= 10) == high && (high || u - t < 10 * max_nb)) ++u;
             q.t1 = u;
             q.high = high;
             if (high) {
@@ -239,6 +242,8 @@ PassPlan build_passes(const bf_problem *p, bool base4)
     pl.ok = true;
     return pl;
 }
+
+int fw_rows(const bf_problem *p) { return p->dtype == BF_C64 ? kFastFwRowsComplex : kFastFwRows; }
 
 struct FastGrid {
     int64_t slots, ngroups, nwg, groups_per_wg;
@@ -281,27 +286,41 @@ bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
     for (int k = 0; k < pl.npass; ++k) {
         const Pass &q = pl.pass[k];
         if (q.high) continue;
-        const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, backward ? 1 : kFastFwRows,
+        const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, backward ? 1 : fw_rows(p),
                                      backward ? 1 : kFastFwWgPerCu);
         rows = std::max(rows, (g.groups_per_wg + kFastFwRows + 2) * g.slots);
     }
     const int64_t dense[3] = {p->nstacks * n, n, 1};
-    if (!span_ok(p->input_stride, rows, n) || !span_ok(p->output_stride, rows, n) || !span_ok(dense, rows, n))
+    const size_t e = elem_bytes(p->dtype);
+    if (!span_ok(p->input_stride, rows, n, e) || !span_ok(p->output_stride, rows, n, e) || !span_ok(dense, rows, n, e))
         return false;
-    if (backward && !span_ok(p->d_input_stride, rows, n)) return false;
+    if (backward && !span_ok(p->d_input_stride, rows, n, e)) return false;
     return true;
 }
 
 template <int L, int NB, bool INC>
-void launch_fast_fw_t(const FastFwArgs &a, dim3 grid, hipStream_t stream)
+void launch_fast_fw_t(bool cplx, const FastFwArgs &a, dim3 grid, hipStream_t stream)
 {
-    hipLaunchKernelGGL((fast_fw_kernel<L, NB, INC, kFastFwRows>), grid, dim3(kFastThreads), 0, stream, a);
+    if constexpr (NB == 1) {
+        if (cplx) {
+            hipLaunchKernelGGL((fast_fw_kernel<float2, L, NB, INC, kFastFwRowsComplex>), grid, dim3(kFastThreads), 0,
+                               stream, a);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((fast_fw_kernel<float, L, NB, INC, kFastFwRows>), grid, dim3(kFastThreads), 0, stream, a);
 }
 
 template <int L, int NB, bool INC>
-void launch_fast_bw_t(const FastBwArgs &a, dim3 grid, hipStream_t stream)
+void launch_fast_bw_t(bool cplx, const FastBwArgs &a, dim3 grid, hipStream_t stream)
 {
-    hipLaunchKernelGGL((fast_bw_kernel<L, NB, INC>), grid, dim3(kFastThreads), 0, stream, a);
+    if constexpr (NB == 1) {
+        if (cplx) {
+            hipLaunchKernelGGL((fast_bw_kernel<float2, L, NB, INC>), grid, dim3(kFastThreads), 0, stream, a);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((fast_bw_kernel<float, L, NB, INC>), grid, dim3(kFastThreads), 0, stream, a);
 }
 
 #define BF_FAST_DISPATCH(FN, Q, ...)                                                     \
@@ -380,24 +399,25 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
             a.batch = p->batch;
             a.rows_per_wg = g.rows_per_wg;
             const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, 1024 / kHighThreads);
-            const int rc = launch_high<float>(q, false, a, grid, stream);
+            const int rc = p->dtype == BF_C64 ? launch_high<float2>(q, false, a, grid, stream)
+                                              : launch_high<float>(q, false, a, grid, stream);
             if (rc) return rc;
         } else {
-            const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, kFastFwRows, kFastFwWgPerCu);
+            const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, fw_rows(p), kFastFwWgPerCu);
             FastFwArgs a = {};
-            a.tw = static_cast<const float *>(tw);
+            a.tw = tw;
             a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
             a.tw_stage_stride = (n / 2) * 4;
             fill_stage_table(a.tw_stage, kFastMaxStages, q);
-            a.in = static_cast<const float *>(src);
+            a.in = src;
             a.in_view = sv;
-            a.out = static_cast<float *>(dst);
+            a.out = dst;
             a.out_view = dv;
             a.batch = p->batch;
             a.ngroups = g.ngroups;
             a.groups_per_wg = g.groups_per_wg;
             const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)pl.chunks);
-            BF_FAST_DISPATCH(launch_fast_fw_t, q, a, grid, stream);
+            BF_FAST_DISPATCH(launch_fast_fw_t, q, p->dtype == BF_C64, a, grid, stream);
             BF_HIP_CHECK(hipGetLastError());
         }
     }
@@ -671,29 +691,30 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                 a.rows_per_wg = g.rows_per_wg;
                 nparts = g.nparts;
                 const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, 1024 / kHighThreads);
-                rc = launch_high<float>(q, true, a, grid, stream);
+                rc = p->dtype == BF_C64 ? launch_high<float2>(q, true, a, grid, stream)
+                                        : launch_high<float>(q, true, a, grid, stream);
                 if (rc) return rc;
             } else {
                 const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1);
                 FastBwArgs a = {};
-                a.tw = static_cast<const float *>(tw2);
+                a.tw = tw2;
                 a.tw_stack_stride = sc.tw2_stack_stride;
                 a.tw_stage_stride = (n / 2) * 4;
                 fill_stage_table(a.tw_stage, kFastMaxStages, q);
                 a.partial_slot = pl.slot;
-                a.x_in = static_cast<const float *>(xin);
+                a.x_in = xin;
                 a.x_view = xv;
-                a.g_out = static_cast<const float *>(gout);
+                a.g_out = gout;
                 a.g_view = gv;
-                a.g_in = static_cast<float *>(gin);
+                a.g_in = gin;
                 a.gi_view = giv;
-                a.partial = reinterpret_cast<float *>(ws + pl.off_partials);
+                a.partial = ws + pl.off_partials;
                 a.batch = p->batch;
                 a.ngroups = g.ngroups;
                 a.groups_per_wg = g.groups_per_wg;
                 nparts = g.nwg;
                 const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)mp.chunks);
-                BF_FAST_DISPATCH(launch_fast_bw_t, q, a, grid, stream);
+                BF_FAST_DISPATCH(launch_fast_bw_t, q, p->dtype == BF_C64, a, grid, stream);
                 BF_HIP_CHECK(hipGetLastError());
             }
             rc = launch_reduce(p, sc, q.t0, q.t1, nparts, ws + pl.off_partials, pl.slot, d_tw2, d_tw4, stream);

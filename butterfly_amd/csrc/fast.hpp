@@ -1,4 +1,4 @@
-// Twiddle-stationary kernels for base-2 float rows of n <= 1024.
+// Twiddle-stationary kernels for base-2 rows of n <= 1024, float and complex64.
 //
 // One workgroup of 1024 threads (16 wavefronts) owns a group of 1024 / n rows at a time and
 // keeps every 2x2 factor it needs in registers for the whole launch: thread t holds one
@@ -127,12 +127,33 @@ __device__ __forceinline__ float partner(float v, int bperm_addr)
         return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(bperm_addr, __builtin_bit_cast(int, v)));
 }
 
+template <int K>
+__device__ __forceinline__ float2 partner(float2 v, int bperm_addr)
+{
+    return make_float2(partner<K>(v.x, bperm_addr), partner<K>(v.y, bperm_addr));
+}
+
 // acc += g * x, pinned where it is written: the accumulators live across the whole row loop
 // and the compiler otherwise sinks these to the end of the iteration, which keeps every
 // stage's operands alive and overflows the register file.
 __device__ __forceinline__ void fmac_pinned(float &acc, float g, float x)
 {
     asm volatile("v_fmac_f32_e32 %0, %1, %2" : "+v"(acc) : "v"(g), "v"(x));
+}
+
+// acc -= g * x, pinned
+__device__ __forceinline__ void fnmac_pinned(float &acc, float g, float x)
+{
+    asm volatile("v_fma_f32 %0, -%1, %2, %0" : "+v"(acc) : "v"(g), "v"(x));
+}
+
+// acc += g * conj(x), pinned
+__device__ __forceinline__ void fmac_pinned(float2 &acc, float2 g, float2 x)
+{
+    fmac_pinned(acc.x, g.x, x.x);
+    fmac_pinned(acc.x, g.y, x.y);
+    fmac_pinned(acc.y, g.y, x.x);
+    fnmac_pinned(acc.y, g.x, x.y);
 }
 
 // acc += g * (x held by the partner thread), for the DPP exchange kinds: one v_fmac with a
@@ -154,6 +175,45 @@ __device__ __forceinline__ void fmac_partner_dpp(float &acc, float g, float x)
     else
         asm volatile("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1"
                      : "+v"(acc) : "v"(x), "v"(g));
+}
+
+// The three products of a backward stage, for one element and exchange kind K.
+//   self  += g * conj(x)            cross += g * conj(x of the partner)
+//   g     <- conj(ta) * g + (conj(tb) * g formed by the partner from its own tb)
+template <int K>
+__device__ __forceinline__ void bw_products(float &self, float &cross, float &g, float x, float ta, float tb,
+                                            int bperm_addr)
+{
+    fmac_pinned(self, g, x);
+    if constexpr (K < 4) fmac_partner_dpp<K>(cross, g, x);
+    else fmac_pinned(cross, g, partner<K>(x, bperm_addr));
+    const float m = tb * g;
+    if constexpr (K < 4) g = ta * g + partner<K>(m, bperm_addr);
+    else g = fmaf(ta, g, partner<K>(m, bperm_addr));
+}
+
+template <int K>
+__device__ __forceinline__ void bw_products(float2 &self, float2 &cross, float2 &g, float2 x, float2 ta,
+                                            float2 tb, int bperm_addr)
+{
+    fmac_pinned(self, g, x);
+    fmac_pinned(cross, g, partner<K>(x, bperm_addr));
+    const float2 m = mul(conj_of(tb), g);
+    g = add(mul(conj_of(ta), g), partner<K>(m, bperm_addr));
+}
+
+// Forward stage for one element: ta * v + tb * (v of the partner).
+template <int K>
+__device__ __forceinline__ float fw_product(float v, float ta, float tb, int bperm_addr)
+{
+    const float p = tb * partner<K>(v, bperm_addr);
+    return fmaf(ta, v, p);
+}
+
+template <int K>
+__device__ __forceinline__ float2 fw_product(float2 v, float2 ta, float2 tb, int bperm_addr)
+{
+    return mac(mul(ta, v), tb, partner<K>(v, bperm_addr));
 }
 
 // Per-thread coordinates in both layouts.
@@ -198,9 +258,18 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base)
 }
 
 // voff: per-thread byte offset (range-checked); soff: wave-uniform byte offset added on top.
-__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int voff, int soff)
+template <typename T>
+__device__ __forceinline__ T buf_load(__amdgpu_buffer_rsrc_t r, int voff, int soff)
 {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+    } else {
+        typedef unsigned v2u __attribute__((ext_vector_type(2)));
+        // (bit-casting a vector element in place reads element 0 for both: go through scalars)
+        const v2u raw = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+        const unsigned lo = raw.x, hi = raw.y;
+        return make_float2(__uint_as_float(lo), __uint_as_float(hi));
+    }
 }
 
 __device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, int voff, int soff, float v)
@@ -208,86 +277,110 @@ __device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, int voff, in
     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
 }
 
+__device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, int voff, int soff, float2 v)
+{
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    v2u raw;
+    const float fx = v.x, fy = v.y;
+    raw.x = __float_as_uint(fx);
+    raw.y = __float_as_uint(fy);
+    __builtin_amdgcn_raw_buffer_store_b64(raw, r, voff, soff, 0);
+}
+
 constexpr int kFastMaxStages = 20;
 
 // Rows longer than 1024 are handled as independent 1024-element chunks (blockIdx.z) for the
 // stages that pair bits below 10: chunk c of stage s uses the factor slice starting at pair
 // c * 512, and its d_twiddle sums land at the same place in the partial slice.
+// All element counts and strides below are in scalars of the kernel's type (float or
+// complex64).
 struct FastFwArgs {
-    const float *tw;           // twiddle tensor, stack 0
+    const void *tw;            // twiddle tensor, stack 0
     int64_t tw_stack_stride;
-    int64_t tw_stage_stride;   // floats between consecutive stages: (n_full / 2) * 4
+    int64_t tw_stage_stride;   // scalars between consecutive stages: (n_full / 2) * 4
     int tw_stage[kFastMaxStages];  // global stage number of every local stage
-    const float *in;
+    const void *in;
     View in_view;
-    float *out;
+    void *out;
     View out_view;
     int64_t batch;
     int64_t ngroups;           // ceil(batch / SLOTS)
     int64_t groups_per_wg;
 };
 
-template <int L, int NB, bool INC, int R>
+// Loads the two factor entries each thread needs for every stage.
+template <typename T, int L, int NB, bool INC>
+__device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, int64_t stage_stride,
+                                             const int (&tw_stage)[kFastMaxStages], int chunk,
+                                             const FastCoords &c, T (&ta)[L * NB], T (&tb)[L * NB])
+{
+    using P = FastPlan<L, NB, INC>;
+    constexpr int n = 1 << L;
+    const T *twp = reinterpret_cast<const T *>(tw) + stack_off + (int64_t)chunk * (n / 2) * 4;
+    static_for<0, P::NS>([&](auto S) {
+        constexpr int s = S;
+        constexpr int bit = P::bit(s);
+        constexpr int lay = P::layout(s);
+        const int e = lay ? c.eB : c.eA;
+        const int r = (e >> bit) & 1;
+        const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
+        const T *Tm = twp + tw_stage[s] * stage_stride + i * 4;
+        ta[s] = Tm[3 * r];   // T[r][r]
+        tb[s] = Tm[r + 1];   // T[r][1 - r]
+    });
+}
+
 #ifndef BF_FAST_FW_WAVES
 #define BF_FAST_FW_WAVES 4
 #endif
+template <typename T, int L, int NB, bool INC, int R>
 __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel(FastFwArgs a)
 {
     using P = FastPlan<L, NB, INC>;
-    constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
-    __shared__ float lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
+    constexpr int NS = P::NS, SLOTS = P::SLOTS;
+    constexpr int EB = (int)sizeof(T);
+    __shared__ T lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
     const FastCoords c = fast_coords<L>(t);
     const int col = (chunk << L) + c.eA;  // column of this thread's element in the full row
 
-    float ta[NS], tb[NS];
-    {
-        const float *twp = a.tw + stack * a.tw_stack_stride + (int64_t)chunk * (n / 2) * 4;
-        static_for<0, NS>([&](auto S) {
-            constexpr int s = S;
-            constexpr int bit = P::bit(s);
-            constexpr int lay = P::layout(s);
-            const int e = lay ? c.eB : c.eA;
-            const int r = (e >> bit) & 1;
-            const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
-            const float *T = twp + a.tw_stage[s] * a.tw_stage_stride + i * 4;
-            ta[s] = T[3 * r];   // T[r][r]
-            tb[s] = T[r + 1];   // T[r][1 - r]
-        });
-    }
+    T ta[NS], tb[NS];
+    load_factors<T, L, NB, INC>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, c, ta, tb);
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
     const int ng = (int)(g1 - g0);
     const int64_t row_end = g1 * SLOTS < a.batch ? g1 * SLOTS : a.batch;
     const int rows_valid = (int)(row_end - g0 * SLOTS);
-    const __amdgpu_buffer_rsrc_t in_rs = make_rsrc(a.in + g0 * SLOTS * a.in_view.sb + stack * a.in_view.ss);
-    const __amdgpu_buffer_rsrc_t out_rs = make_rsrc(a.out + g0 * SLOTS * a.out_view.sb + stack * a.out_view.ss);
-    const int in_row = (int)(a.in_view.sb * 4), out_row = (int)(a.out_view.sb * 4);
+    const __amdgpu_buffer_rsrc_t in_rs =
+        make_rsrc(reinterpret_cast<const T *>(a.in) + g0 * SLOTS * a.in_view.sb + stack * a.in_view.ss);
+    const __amdgpu_buffer_rsrc_t out_rs =
+        make_rsrc(reinterpret_cast<T *>(a.out) + g0 * SLOTS * a.out_view.sb + stack * a.out_view.ss);
+    const int in_row = (int)(a.in_view.sb * EB), out_row = (int)(a.out_view.sb * EB);
     // thread-constant part of the offsets; the row group adds a wave-uniform part
-    const int in_thr = col < a.in_view.width ? c.slot * in_row + (int)(col * a.in_view.se * 4) : kOob;
-    const int out_thr = col < a.out_view.width ? c.slot * out_row + (int)(col * a.out_view.se * 4) : kOob;
+    const int in_thr = col < a.in_view.width ? c.slot * in_row + (int)(col * a.in_view.se * EB) : kOob;
+    const int out_thr = col < a.out_view.width ? c.slot * out_row + (int)(col * a.out_view.se * EB) : kOob;
 
-    auto load_rows = [&](int grel, float (&v)[R]) {
+    auto load_rows = [&](int grel, T (&v)[R]) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
-            v[r] = buf_load(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
+            v[r] = buf_load<T>(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
         }
     };
 
-    float nxt[R];
+    T nxt[R];
     load_rows(0, nxt);
     // R stores that the range check discards.  They put the same "loads, then stores" history
     // in front of the first iteration as every later iteration has, so the wait for the
     // prefetched rows at the top of the loop is emitted as "all but the newest R operations"
     // and does not also wait for the previous iteration's stores to be acknowledged.
 #pragma unroll
-    for (int r = 0; r < R; ++r) buf_store(out_rs, kOob, 4 * r, 0.0f);
+    for (int r = 0; r < R; ++r) buf_store(out_rs, kOob, EB * r, zero_of(T()));
     for (int grel = 0; grel < ng; grel += R) {
-        float v[R];
+        T v[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) v[r] = nxt[r];
         load_rows(grel + R, nxt);
@@ -298,7 +391,7 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
             if constexpr (P::layout(s) != P::layout_before(s)) {
                 constexpr int par = P::fw_transposes_before(s) & 1;
                 constexpr int to_b = P::layout(s);
-                float *buf = lds + par * R * kFastRowWords;
+                T *buf = lds + par * R * kFastRowWords;
                 const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
 #pragma unroll
                 for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
@@ -307,14 +400,11 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
                 for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];
             }
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const float p = tb[s] * partner<K>(v[r], c.bperm_addr);
-                v[r] = fmaf(ta[s], v[r], p);
-            }
+            for (int r = 0; r < R; ++r) v[r] = fw_product<K>(v[r], ta[s], tb[s], c.bperm_addr);
         });
         if constexpr (P::layout(NS - 1) != 0) {
             constexpr int par = P::fw_transposes_before(NS) & 1;
-            float *buf = lds + par * R * kFastRowWords;
+            T *buf = lds + par * R * kFastRowWords;
 #pragma unroll
             for (int r = 0; r < R; ++r) buf[r * kFastRowWords + c.fB] = v[r];
             __syncthreads();
@@ -330,18 +420,18 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
 }
 
 struct FastBwArgs {
-    const float *tw;
+    const void *tw;
     int64_t tw_stack_stride;
     int64_t tw_stage_stride;
     int tw_stage[kFastMaxStages];
-    int64_t partial_slot;      // floats per stage in a partial slice: 2 * n_full
-    const float *x_in;
+    int64_t partial_slot;      // scalars per stage in a partial slice: 2 * n_full
+    const void *x_in;
     View x_view;
-    const float *g_out;
+    const void *g_out;
     View g_view;
-    float *g_in;
+    void *g_in;
     View gi_view;
-    float *partial;            // (gridDim.x, S, NS, partial_slot)
+    void *partial;             // (gridDim.x, S, NS, partial_slot)
     int64_t batch;
     int64_t ngroups;
     int64_t groups_per_wg;
@@ -351,7 +441,7 @@ struct FastBwArgs {
 // row i + 1 (producing its stage inputs) together with the reverse sweep of row i (consuming
 // the stage inputs produced one iteration earlier).  The two walks change layout at mirrored
 // points, so they share every barrier, and their transposes travel through LDS as one
-// 64-bit (x, g) pair.  Two independent dependency chains per thread also hide the DPP and
+// (x, g) pair.  Two independent dependency chains per thread also hide the DPP and
 // LDS latencies that a single chain exposes.
 template <int L, int NB, bool INC>
 struct BwPipe {
@@ -396,89 +486,96 @@ struct BwPipe {
     }
 };
 
-template <int L, int NB, bool INC>
+// (x, g) pair that travels through LDS as one access
+template <typename T> struct PairOf;
+template <> struct PairOf<float> { typedef float2 type; };
+template <> struct PairOf<float2> { typedef float4 type; };
+__device__ __forceinline__ float2 make_pair(float x, float g) { return make_float2(x, g); }
+__device__ __forceinline__ float4 make_pair(float2 x, float2 g) { return make_float4(x.x, x.y, g.x, g.y); }
+__device__ __forceinline__ float pair_x(float2 p) { return p.x; }
+__device__ __forceinline__ float pair_g(float2 p) { return p.y; }
+__device__ __forceinline__ float2 pair_x(float4 p) { return make_float2(p.x, p.y); }
+__device__ __forceinline__ float2 pair_g(float4 p) { return make_float2(p.z, p.w); }
+
+template <typename T, int L, int NB, bool INC>
 __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 {
     using P = FastPlan<L, NB, INC>;
     using Q = BwPipe<L, NB, INC>;
+    using Pair = typename PairOf<T>::type;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
-    __shared__ float2 lds[P::NSWAP > 0 ? 2 * kFastRowWords : 1];
-    __shared__ float lds_carry[Q::DEFER ? kFastRowWords : 1];
+    constexpr int EB = (int)sizeof(T);
+    __shared__ Pair lds[P::NSWAP > 0 ? 2 * kFastRowWords : 1];
+    __shared__ T lds_carry[Q::DEFER ? kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
     const FastCoords c = fast_coords<L>(t);
     const int col = (chunk << L) + c.eA;  // column of this thread's element in the full row
 
-    float ta[NS], tb[NS], acc_self[NS], acc_cross[NS];
-    {
-        const float *twp = a.tw + stack * a.tw_stack_stride + (int64_t)chunk * (n / 2) * 4;
-        static_for<0, NS>([&](auto S) {
-            constexpr int s = S;
-            constexpr int bit = P::bit(s);
-            constexpr int lay = P::layout(s);
-            const int e = lay ? c.eB : c.eA;
-            const int r = (e >> bit) & 1;
-            const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
-            const float *T = twp + a.tw_stage[s] * a.tw_stage_stride + i * 4;
-            ta[s] = T[3 * r];
-            tb[s] = T[r + 1];
-            acc_self[s] = 0.0f;
-            acc_cross[s] = 0.0f;
-        });
-    }
+    T ta[NS], tb[NS], acc_self[NS], acc_cross[NS];
+    load_factors<T, L, NB, INC>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, c, ta, tb);
+    static_for<0, NS>([&](auto S) {
+        acc_self[S] = zero_of(T());
+        acc_cross[S] = zero_of(T());
+    });
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
     const int ng = (int)(g1 - g0);
     const int64_t row_end = g1 * SLOTS < a.batch ? g1 * SLOTS : a.batch;
     const int rows_valid = (int)(row_end - g0 * SLOTS);
-    const __amdgpu_buffer_rsrc_t x_rs = make_rsrc(a.x_in + g0 * SLOTS * a.x_view.sb + stack * a.x_view.ss);
-    const __amdgpu_buffer_rsrc_t g_rs = make_rsrc(a.g_out + g0 * SLOTS * a.g_view.sb + stack * a.g_view.ss);
-    const __amdgpu_buffer_rsrc_t gi_rs = make_rsrc(a.g_in + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
-    const int x_row = (int)(a.x_view.sb * 4), g_row = (int)(a.g_view.sb * 4), gi_row = (int)(a.gi_view.sb * 4);
-    const int x_thr = col < a.x_view.width ? c.slot * x_row + (int)(col * a.x_view.se * 4) : kOob;
-    const int g_thr = col < a.g_view.width ? c.slot * g_row + (int)(col * a.g_view.se * 4) : kOob;
-    const int gi_thr = col < a.gi_view.width ? c.slot * gi_row + (int)(col * a.gi_view.se * 4) : kOob;
+    const __amdgpu_buffer_rsrc_t x_rs =
+        make_rsrc(reinterpret_cast<const T *>(a.x_in) + g0 * SLOTS * a.x_view.sb + stack * a.x_view.ss);
+    const __amdgpu_buffer_rsrc_t g_rs =
+        make_rsrc(reinterpret_cast<const T *>(a.g_out) + g0 * SLOTS * a.g_view.sb + stack * a.g_view.ss);
+    const __amdgpu_buffer_rsrc_t gi_rs =
+        make_rsrc(reinterpret_cast<T *>(a.g_in) + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
+    const int x_row = (int)(a.x_view.sb * EB), g_row = (int)(a.g_view.sb * EB), gi_row = (int)(a.gi_view.sb * EB);
+    const int x_thr = col < a.x_view.width ? c.slot * x_row + (int)(col * a.x_view.se * EB) : kOob;
+    const int g_thr = col < a.g_view.width ? c.slot * g_row + (int)(col * a.g_view.se * EB) : kOob;
+    const int gi_thr = col < a.gi_view.width ? c.slot * gi_row + (int)(col * a.gi_view.se * EB) : kOob;
 
     auto group_ok = [&](int grp) { return grp >= 0 && grp * SLOTS + c.slot < rows_valid; };
-    auto load_x = [&](int grp) { return buf_load(x_rs, group_ok(grp) ? x_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row); };
-    auto load_g = [&](int grp) { return buf_load(g_rs, group_ok(grp) ? g_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * g_row); };
-
-    // One pipelined iteration: forward replay of group it + 1 into `nxt`, reverse sweep of
-    // group it out of `cur`.  vF / gv enter holding the freshly loaded x and g.
-    auto store_grad = [&](int grp, float gval) {
-        const bool ok = group_ok(grp);
-        const int soff = (grp < 0 ? 0 : grp) * SLOTS * gi_row;
-        buf_store(gi_rs, ok ? gi_thr : kOob, soff, gval);
+    auto load_x = [&](int grp) {
+        return buf_load<T>(x_rs, group_ok(grp) ? x_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row);
+    };
+    auto load_g = [&](int grp) {
+        return buf_load<T>(g_rs, group_ok(grp) ? g_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * g_row);
+    };
+    auto store_grad = [&](int grp, T gval) {
+        buf_store(gi_rs, group_ok(grp) ? gi_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * gi_row, gval);
     };
 
-    // `carry` holds the previous group's input gradient still in layout B (DEFER only)
-    // FLIP alternates between the two unrolled calls so that LDS buffers keep alternating
-    // across iterations when the number of phases is odd.
-    auto iteration = [&](auto FLIP, int it, float vF, float gv, float &carry, float (&cur)[NS], float (&nxt)[NS]) {
+    // One pipelined iteration: forward replay of group it + 1 into `nxt`, reverse sweep of
+    // group it out of `cur`; vF / gv enter holding the freshly loaded x and g.  `carry` holds
+    // the previous group's input gradient still in layout B (DEFER only).  FLIP alternates
+    // between the two unrolled calls so that LDS buffers keep alternating across iterations
+    // when the number of phases is odd.
+    auto iteration = [&](auto FLIP, int it, T vF, T gv, T &carry, T (&cur)[NS], T (&nxt)[NS]) {
         constexpr int flip = decltype(FLIP)::value;
         static_for<0, Q::K + 1>([&](auto KK) {
             constexpr int k = KK;
             if constexpr (k >= 1) {
                 constexpr bool hasF = k <= Q::nF, hasB = k <= Q::nB;
                 constexpr int to_b = k & 1;  // both walks start in layout A and alternate
-                float2 *buf = lds + ((k + flip * Q::K) & 1) * kFastRowWords;
+                Pair *buf = lds + ((k + flip * Q::K) & 1) * kFastRowWords;
+                T *bufs = reinterpret_cast<T *>(buf);
                 const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
-                if constexpr (hasF && hasB) buf[wr] = make_float2(vF, gv);
-                else if constexpr (hasF) buf[wr].x = vF;
-                else buf[wr].y = gv;
+                if constexpr (hasF && hasB) buf[wr] = make_pair(vF, gv);
+                else if constexpr (hasF) bufs[2 * wr] = vF;
+                else bufs[2 * wr + 1] = gv;
                 if constexpr (Q::DEFER && k == 1) lds_carry[c.fB] = carry;
                 __syncthreads();
                 if constexpr (Q::DEFER && k == 1) store_grad(it - 1, lds_carry[c.fA]);
                 if constexpr (hasF && hasB) {
-                    const float2 v2 = buf[rd];
-                    vF = v2.x;
-                    gv = v2.y;
+                    const Pair v2 = buf[rd];
+                    vF = pair_x(v2);
+                    gv = pair_g(v2);
                 } else if constexpr (hasF) {
-                    vF = buf[rd].x;
+                    vF = bufs[2 * rd];
                 } else {
-                    gv = buf[rd].y;
+                    gv = bufs[2 * rd + 1];
                 }
             }
             constexpr int cf = Q::f_count(k), cb = Q::b_count(k);
@@ -486,27 +583,14 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             static_for<0, (cf > cb ? cf : cb)>([&](auto J) {
                 constexpr int j = J;
                 if constexpr (j < cb) {
-                    // reverse stage s: uses the gradient before it passes through the stage
+                    // reverse stage: uses the gradient before it passes through the stage
                     constexpr int s = b0 - j;
-                    constexpr int Kd = P::kind(s);
-                    const float xs = cur[s];
-                    fmac_pinned(acc_self[s], gv, xs);
-                    if constexpr (Kd < 4) fmac_partner_dpp<Kd>(acc_cross[s], gv, xs);
-                    else fmac_pinned(acc_cross[s], gv, partner<Kd>(xs, c.bperm_addr));
-                    // d_x[r] = T[r][r] g[r] + T[1-r][r] g[1-r]; the partner forms the second
-                    // product from its own factor entry and it is fetched.
-                    const float m = tb[s] * gv;
-                    if constexpr (Kd < 4) gv = ta[s] * gv + partner<Kd>(m, c.bperm_addr);
-                    else gv = fmaf(ta[s], gv, partner<Kd>(m, c.bperm_addr));
+                    bw_products<P::kind(s)>(acc_self[s], acc_cross[s], gv, cur[s], ta[s], tb[s], c.bperm_addr);
                 }
                 if constexpr (j < cf) {
                     constexpr int s = f0 + j;
-                    constexpr int Kd = P::kind(s);
                     nxt[s] = vF;
-                    if constexpr (s + 1 < NS) {
-                        const float p = tb[s] * partner<Kd>(vF, c.bperm_addr);
-                        vF = fmaf(ta[s], vF, p);
-                    }
+                    if constexpr (s + 1 < NS) vF = fw_product<P::kind(s)>(vF, ta[s], tb[s], c.bperm_addr);
                 }
             });
         });
@@ -514,16 +598,16 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         else store_grad(it, gv);
     };
 
-    float actP[NS], actQ[NS];
-    static_for<0, NS>([&](auto S) { actP[S] = 0.0f; });
+    T actP[NS], actQ[NS];
+    static_for<0, NS>([&](auto S) { actP[S] = zero_of(T()); });
     // iteration it pairs group it + 1 (forward) with group it (reverse); it = -1 .. ng - 1
-    float x0 = load_x(0), gm = load_g(-1);
-    float x1 = load_x(1), gp = load_g(0);
-    float carry = 0.0f;
+    T x0 = load_x(0), gm = load_g(-1);
+    T x1 = load_x(1), gp = load_g(0);
+    T carry = zero_of(T());
     // with a deferred closing transpose one more (empty) iteration flushes the last group
     const int it_end = Q::DEFER ? ng + 1 : ng;
     for (int it = -1; it < it_end; it += 2) {
-        const float xa = x0, ga = gm, xb = x1, gb = gp;
+        const T xa = x0, ga = gm, xb = x1, gb = gp;
         x0 = load_x(it + 3);
         gm = load_g(it + 2);
         x1 = load_x(it + 4);
@@ -539,8 +623,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const FastCoords c2 = fast_coords<L>(t2);
     // One partial slice per workgroup.  When the workgroup holds several rows at once
     // (n < 1024) the per-row-slot sums are first added through LDS in ascending slot order.
-    float *part = a.partial + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * a.partial_slot +
-                  (int64_t)chunk * (n / 2) * 4;
+    T *part = reinterpret_cast<T *>(a.partial) + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * a.partial_slot +
+              (int64_t)chunk * (n / 2) * 4;
     if constexpr (SLOTS == 1) {
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
@@ -549,12 +633,12 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             const int e = lay ? c2.eB : c2.eA;
             const int r = (e >> bit) & 1;
             const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
-            float *d = part + (int64_t)s * a.partial_slot + i * 4;
+            T *d = part + (int64_t)s * a.partial_slot + i * 4;
             d[3 * r] = acc_self[s];    // dT[r][r]
             d[r + 1] = acc_cross[s];   // dT[r][1 - r]
         });
     } else {
-        __shared__ float red[2 * 1024];
+        __shared__ T red[2 * 1024];
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
             constexpr int bit = P::bit(s);
@@ -566,9 +650,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             __syncthreads();
             if (t2 < 2 * n) {
                 const int eo = t2 >> 1, j = t2 & 1;
-                float sum = red[t2];
+                T sum = red[t2];
 #pragma unroll 4
-                for (int sl = 1; sl < SLOTS; ++sl) sum += red[sl * 2 * n + t2];
+                for (int sl = 1; sl < SLOTS; ++sl) sum = add(sum, red[sl * 2 * n + t2]);
                 const int r = (eo >> bit) & 1;
                 const int i = ((eo >> (bit + 1)) << bit) | (eo & ((1 << bit) - 1));
                 // j = 0: dT[r][r], j = 1: dT[r][1 - r]

@@ -130,6 +130,40 @@ def test_multi_launch_schedules(case):
     assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
 
 
+COMPLEX_FAST_CASES = [
+    # B, S, L, nb, I, O, inc
+    (37, 2, 1, 2, None, None, True),
+    (37, 2, 3, 3, None, None, False),
+    (300, 1, 5, 2, 29, 20, True),
+    (50, 2, 6, 1, None, None, False),
+    (50, 2, 8, 2, None, None, True),
+    (40, 1, 9, 3, None, None, False),
+    (33, 2, 10, 1, None, None, True),
+    (33, 1, 10, 2, 1000, 1001, False),
+    (9, 2, 11, 2, None, None, True),
+    (9, 1, 12, 1, None, None, True),
+    (9, 1, 12, 2, None, None, False),
+    (5, 2, 12, 3, 4092, 2046, True),
+]
+
+
+@pytest.mark.parametrize("case", COMPLEX_FAST_CASES, ids=lambda c: f"B{c[0]}-S{c[1]}-L{c[2]}-nb{c[3]}-I{c[4]}-O{c[5]}-inc{int(c[6])}")
+def test_complex_register_resident_kernels(case):
+    from butterfly_amd import _capi
+    B, S, L, nb, I, O, inc = case
+    say("complex case", case)
+    rng = np.random.default_rng(1300 + L * 17 + nb)
+    tw, x, g = make_case(rng, np.complex64, B, S, L, nb, I, O)
+    y_ref = oracle.butterfly_fw(tw, x, inc, O)
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+    y = _capi.multiply_fw(dev(tw), dev(x), inc, O)
+    dtw, dx = _capi.multiply_bw(dev(tw), dev(x), dev(g), inc)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
 def test_c_abi_strided_operands():
     """Stride-0 stack broadcast (what Butterfly.pre_process hands over), a transposed input
     and a non-contiguous gradient."""
