@@ -17,7 +17,8 @@ SYMBOLS = [
     "bf_version", "bf_hip_version", "bf_last_error",
     "bf_butterfly_multiply_fw", "bf_butterfly_multiply_fw_workspace_bytes",
     "bf_butterfly_multiply_bw_workspace_bytes", "bf_butterfly_multiply_bw",
-    "bf_butterfly_multiply_base4_fw", "bf_butterfly_multiply_base4_bw_workspace_bytes",
+    "bf_butterfly_multiply_base4_fw", "bf_butterfly_multiply_base4_fw_workspace_bytes",
+    "bf_butterfly_multiply_base4_bw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw",
 ]
 
@@ -58,7 +59,9 @@ def lib():
         L.bf_butterfly_multiply_bw_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_bw_workspace_bytes.restype = sz
         L.bf_butterfly_multiply_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, sz, vp]
-        L.bf_butterfly_multiply_base4_fw.argtypes = [pp, vp, vp, vp, vp, vp]
+        L.bf_butterfly_multiply_base4_fw.argtypes = [pp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_base4_fw_workspace_bytes.argtypes = [pp]
+        L.bf_butterfly_multiply_base4_fw_workspace_bytes.restype = sz
         L.bf_butterfly_multiply_base4_bw_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_base4_bw_workspace_bytes.restype = sz
         L.bf_butterfly_multiply_base4_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
@@ -148,8 +151,10 @@ def multiply_base4_fw(twiddle4, twiddle2, input, increasing_stride, output_size=
     p = make_problem(input, log_n, nb, increasing_stride, O)
     out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
     p.output_stride = _strides(out)
+    nbytes = lib().bf_butterfly_multiply_base4_fw_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_base4_fw(ctypes.byref(p), _ptr(twiddle4), _ptr(twiddle2),
-                                                _ptr(input), _ptr(out), _stream()))
+                                                _ptr(input), _ptr(out), _ptr(ws), nbytes, _stream()))
     return out
 
 

@@ -16,6 +16,7 @@
 #include "generic.hpp"
 #include "fast.hpp"
 #include "high.hpp"
+#include "fast4.hpp"
 
 namespace {
 
@@ -424,6 +425,77 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
     return BF_OK;
 }
 
+// ---- base-4 register-resident path (float, even log_n <= 10): one launch per block -----------
+
+constexpr int kFast4FwRows = 4;
+
+bool fast4_ok(const bf_problem *p, bool base4, bool backward)
+{
+    if (!base4 || p->dtype != BF_F32 || p->log_n < 2 || p->log_n > 10 || (p->log_n & 1) || p->nblocks < 1 ||
+        p->batch <= 0 || p->nstacks <= 0 || p->input_size <= 0 || p->output_size <= 0)
+        return false;
+    const int64_t n = (int64_t)1 << p->log_n;
+    const FastGrid g = fast_grid(p->batch, (int)p->log_n, p->nstacks, backward ? 1 : kFast4FwRows, 1);
+    const int64_t rows = (g.groups_per_wg + kFast4FwRows + 2) * g.slots;
+    const int64_t dense[3] = {p->nstacks * n, n, 1};
+    if (!span_ok(p->input_stride, rows, n, 4) || !span_ok(p->output_stride, rows, n, 4) || !span_ok(dense, rows, n, 4))
+        return false;
+    if (backward && !span_ok(p->d_input_stride, rows, n, 4)) return false;
+    return true;
+}
+
+template <int L, bool INC>
+void launch_fast4_t(bool backward, const Fast4Args &a, dim3 grid, hipStream_t stream)
+{
+    if (backward) hipLaunchKernelGGL((fast4_bw_kernel<L, INC>), grid, dim3(kFastThreads), 0, stream, a);
+    else hipLaunchKernelGGL((fast4_fw_kernel<L, INC, kFast4FwRows>), grid, dim3(kFastThreads), 0, stream, a);
+}
+
+int launch_fast4(int L, bool inc, bool backward, const Fast4Args &a, dim3 grid, hipStream_t stream)
+{
+    switch (L * 2 + (inc ? 1 : 0)) {
+        case 2 * 2 + 0: launch_fast4_t<2, false>(backward, a, grid, stream); break;
+        case 2 * 2 + 1: launch_fast4_t<2, true>(backward, a, grid, stream); break;
+        case 4 * 2 + 0: launch_fast4_t<4, false>(backward, a, grid, stream); break;
+        case 4 * 2 + 1: launch_fast4_t<4, true>(backward, a, grid, stream); break;
+        case 6 * 2 + 0: launch_fast4_t<6, false>(backward, a, grid, stream); break;
+        case 6 * 2 + 1: launch_fast4_t<6, true>(backward, a, grid, stream); break;
+        case 8 * 2 + 0: launch_fast4_t<8, false>(backward, a, grid, stream); break;
+        case 8 * 2 + 1: launch_fast4_t<8, true>(backward, a, grid, stream); break;
+        case 10 * 2 + 0: launch_fast4_t<10, false>(backward, a, grid, stream); break;
+        case 10 * 2 + 1: launch_fast4_t<10, true>(backward, a, grid, stream); break;
+        default: return fail(BF_ERR_UNSUPPORTED, "no base-4 kernel for this shape");
+    }
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
+}
+
+// forward of blocks [first, last) through the base-4 kernels; `scratch` as in multipass_forward
+int fast4_forward(const bf_problem *p, const void *tw4, const void *input, void *output, void *scratch,
+                  const View &in_view, const View &out_view, int first, int last, hipStream_t stream)
+{
+    const int64_t n = (int64_t)1 << p->log_n;
+    const int L = (int)p->log_n;
+    const View dense = dense_view(p->nstacks, n);
+    const FastGrid g = fast_grid(p->batch, L, p->nstacks, kFast4FwRows, 1);
+    for (int k = first; k < last; ++k) {
+        Fast4Args a = {};
+        a.tw4 = static_cast<const float *>(tw4) + (int64_t)k * (L / 2) * (n / 4) * 16;
+        a.tw_stack_stride = p->nblocks * (L / 2) * (n / 4) * 16;
+        a.x_in = static_cast<const float *>(k == first ? input : scratch);
+        a.x_view = k == first ? in_view : dense;
+        a.x_out = static_cast<float *>(k == last - 1 ? output : scratch);
+        a.xo_view = k == last - 1 ? out_view : dense;
+        a.batch = p->batch;
+        a.ngroups = g.ngroups;
+        a.groups_per_wg = g.groups_per_wg;
+        const bool inc = (p->increasing_stride != 0) != ((k & 1) != 0);
+        const int rc = launch_fast4(L, inc, false, a, dim3((unsigned)g.nwg, (unsigned)p->nstacks), stream);
+        if (rc) return rc;
+    }
+    return BF_OK;
+}
+
 // ---- generic forward ----------------------------------------------------------------------
 
 int launch_generic_fw(const bf_problem *p, const Schedule &sc, int t0, int t1, const void *tw2,
@@ -466,6 +538,10 @@ int launch_generic_fw(const bf_problem *p, const Schedule &sc, int t0, int t1, c
 // Workspace of the forward call: one dense activation when the pass plan has several passes.
 size_t forward_workspace(const bf_problem *p, bool base4)
 {
+    if (fast4_ok(p, base4, false)) {
+        const int64_t n4 = (int64_t)1 << p->log_n;
+        return p->nblocks > 1 ? align256((size_t)p->batch * p->nstacks * n4 * 4) : 0;
+    }
     const PassPlan mp = build_passes(p, base4);
     if (!mp.ok || mp.npass <= 1 || !passes_addressable(p, mp, false)) return 0;
     const int64_t n = (int64_t)1 << p->log_n;
@@ -492,6 +568,12 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
     }
     const View in_view = make_view(p->input_stride, std::min(p->input_size, n));
     const View out_view = make_view(p->output_stride, p->output_size);
+    if (fast4_ok(p, base4, false)) {
+        const size_t need = forward_workspace(p, base4);
+        if (need > 0 && (!workspace || workspace_bytes < need))
+            return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        return fast4_forward(p, tw4, input, output, workspace, in_view, out_view, 0, (int)p->nblocks, stream);
+    }
     const PassPlan mp = build_passes(p, base4);
     if (mp.ok && passes_addressable(p, mp, false)) {
         const size_t need = forward_workspace(p, base4);
@@ -517,6 +599,7 @@ struct BwPlan {
     size_t off_boundaries, off_gbuf, off_partials, total;
     bool fits;
     bool fast;          // register-resident pass plan
+    bool fast4;         // base-4 register-resident kernels, one launch per block
 };
 
 BwPlan plan_bw(const bf_problem *p, bool base4)
@@ -527,6 +610,23 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
     const size_t row_bytes = (size_t)n * e;
     const Schedule sc = make_schedule(p, base4);
     pl.nstages = sc.per * sc.nblocks;
+    if (fast4_ok(p, base4, true)) {
+        pl.fits = true;
+        pl.fast4 = true;
+        pl.nchunks = (int)p->nblocks;
+        pl.slot = 4 * n;
+        pl.boundary_bytes = align256((size_t)p->batch * p->nstacks * row_bytes);
+        pl.nparts = fast_grid(p->batch, (int)p->log_n, p->nstacks, 1, 1).nwg;
+        size_t off = 0;
+        pl.off_boundaries = off;
+        off += p->nblocks > 1 ? (size_t)(p->nblocks - 1) * pl.boundary_bytes : 0;
+        pl.off_gbuf = off;
+        off += p->nblocks > 1 ? pl.boundary_bytes : 0;
+        pl.off_partials = off;
+        off += align256((size_t)pl.nparts * p->nstacks * (p->log_n / 2) * pl.slot * e);
+        pl.total = off;
+        return pl;
+    }
     const PassPlan mp = build_passes(p, base4);
     if (mp.ok && passes_addressable(p, mp, true)) {
         // boundaries: the activation entering every pass after the first; one gradient plane
@@ -651,6 +751,51 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     const size_t e_bytes = elem_bytes(p->dtype);
 
     if (pl.nstages == 0) return launch_copy_pad(p, grad, g_view, d_input, di_view, stream);
+
+    if (pl.fast4) {
+        const int L = (int)p->log_n;
+        const int P = (int)p->nblocks;
+        const int per = L / 2;
+        auto boundary = [&](int k) { return ws + pl.off_boundaries + (size_t)(k - 1) * pl.boundary_bytes; };
+        for (int k = 0; k + 1 < P; ++k) {
+            rc = fast4_forward(p, tw4, k == 0 ? input : boundary(k), boundary(k + 1), nullptr,
+                               k == 0 ? x_view : dense, dense, k, k + 1, stream);
+            if (rc) return rc;
+        }
+        const View dn_view = make_view(p->d_input_stride, std::min(p->input_size, n));
+        const FastGrid g = fast_grid(p->batch, L, p->nstacks, 1, 1);
+        for (int k = P - 1; k >= 0; --k) {
+            Fast4Args a = {};
+            a.tw4 = static_cast<const float *>(tw4) + (int64_t)k * per * (n / 4) * 16;
+            a.tw_stack_stride = sc.tw4_stack_stride;
+            a.x_in = static_cast<const float *>(k == 0 ? input : boundary(k));
+            a.x_view = k == 0 ? x_view : dense;
+            a.g_out = static_cast<const float *>(k == P - 1 ? grad : ws + pl.off_gbuf);
+            a.g_view = k == P - 1 ? g_view : dense;
+            a.g_in = static_cast<float *>(k == 0 ? d_input : ws + pl.off_gbuf);
+            a.gi_view = k == 0 ? dn_view : dense;
+            a.partial = reinterpret_cast<float *>(ws + pl.off_partials);
+            a.batch = p->batch;
+            a.ngroups = g.ngroups;
+            a.groups_per_wg = g.groups_per_wg;
+            const bool inc = (p->increasing_stride != 0) != ((k & 1) != 0);
+            rc = launch_fast4(L, inc, true, a, dim3((unsigned)g.nwg, (unsigned)p->nstacks), stream);
+            if (rc) return rc;
+            rc = launch_reduce(p, sc, k * per, (k + 1) * per, g.nwg, ws + pl.off_partials, pl.slot, d_tw2, d_tw4,
+                               stream);
+            if (rc) return rc;
+        }
+        if (p->input_size > n) {
+            View tail = di_view;
+            tail.width = p->input_size - n;
+            View none = tail;
+            none.width = 0;
+            char *base = static_cast<char *>(d_input) + (size_t)n * p->d_input_stride[2] * e_bytes;
+            rc = launch_copy_pad(p, base, none, base, tail, stream);
+            if (rc) return rc;
+        }
+        return BF_OK;
+    }
 
     if (pl.fast) {
         const PassPlan mp = build_passes(p, base4);
@@ -813,10 +958,17 @@ int bf_butterfly_multiply_bw(const bf_problem *p, const void *twiddle, const voi
                     workspace_bytes, stream);
 }
 
-int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4, const void *twiddle2,
-                                   const void *input, void *output, void *stream)
+size_t bf_butterfly_multiply_base4_fw_workspace_bytes(const bf_problem *p)
 {
-    return forward(p, true, twiddle2, twiddle4, input, output, nullptr, 0, stream);
+    if (check_problem(p, false)) return 0;
+    return forward_workspace(p, true);
+}
+
+int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4, const void *twiddle2,
+                                   const void *input, void *output, void *workspace, size_t workspace_bytes,
+                                   void *stream)
+{
+    return forward(p, true, twiddle2, twiddle4, input, output, workspace, workspace_bytes, stream);
 }
 
 size_t bf_butterfly_multiply_base4_bw_workspace_bytes(const bf_problem *p)

@@ -222,8 +222,10 @@ Tensor butterfly_multiply_base4_fw(const Tensor twiddle4, const Tensor twiddle2,
     if (output_size_val < s.n) output = output.slice(2, 0, output_size_val);
     bf_problem p = make_problem(s, x, increasing_stride, output_size_val, "butterfly_multiply_base4_fw");
     set_strides(p.output_stride, output);
-    check_rc(bf_butterfly_multiply_base4_fw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(),
-                                            output.data_ptr(), current_stream()),
+    const size_t ws_bytes = bf_butterfly_multiply_base4_fw_workspace_bytes(&p);
+    Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+    check_rc(bf_butterfly_multiply_base4_fw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(), output.data_ptr(),
+                                            ws.data_ptr(), ws_bytes, current_stream()),
              "butterfly_multiply_base4_fw");
     return output;
 }

@@ -1,0 +1,298 @@
+// Twiddle-stationary kernels for base-4 float rows, n = 2^L <= 1024 with L even: one block of
+// L / 2 radix-4 stages per launch.
+//
+// Same ownership as fast.hpp: 1024 threads, one element per thread and row, factors in
+// registers for the whole launch.  A radix-4 stage couples the four elements that differ in
+// an aligned bit pair (2j, 2j+1); the three partners are reached with
+//   pair on phi bits (0,1): quad_perm [1,0,3,2] / [2,3,0,1] / [3,2,1,0]
+//   pair on phi bits (2,3): row_half_mirror / row_mirror / row_ror:8
+//   pair on lane bits (4,5): ds_swizzle xor 16, ds_bpermute xor 32 / xor 48
+// and pairs (6,7), (8,9) after the LDS transpose into layout B, where they sit on the phi
+// bits.  Each thread keeps its own ROW of the 4x4 factor (forward, d_twiddle) and its own
+// COLUMN (for d_x): 12 instructions per element and radix-4 stage in the backward pass.
+#pragma once
+
+#include "fast.hpp"
+
+namespace bf {
+
+template <int L, bool INC>
+struct Plan4 {
+    static_assert(L % 2 == 0 && L >= 2 && L <= 10, "base-4 fast path needs an even log_n <= 10");
+    static constexpr int NS = L / 2;
+    static constexpr int NSWAP = L > 6 ? L - 6 : 0;
+    static constexpr int SLOTS = 1024 >> L;
+    // low bit of the bit pair coupled by stage s
+    static constexpr int bit(int s) { return 2 * (INC ? s : NS - 1 - s); }
+    static constexpr int layout(int s)
+    {
+        int cur = 0;
+        for (int j = 0; j <= s; ++j) {
+            const int b = bit(j);
+            if (b >= 6) cur = 1;
+            else if (b < NSWAP) cur = 0;
+        }
+        return cur;
+    }
+    static constexpr int layout_before(int s) { return s == 0 ? 0 : layout(s - 1); }
+    static constexpr int layout_after(int s) { return s == NS - 1 ? 0 : layout(s + 1); }
+    // exchange kind: 0 = phi bits (0,1), 1 = phi bits (2,3), 2 = lane bits (4,5)
+    static constexpr int kind(int s)
+    {
+        const int b = bit(s);
+        return (b >= 6 ? b - 6 : b) / 2;
+    }
+};
+
+// value held by the thread whose element differs by mask M (1, 2, 3) in the stage's bit pair
+template <int KQ, int M>
+__device__ __forceinline__ float partner4(float v, int lane)
+{
+    if constexpr (KQ == 0) {
+        if constexpr (M == 1) return dpp_move<0xB1>(v);        // quad_perm [1,0,3,2]
+        else if constexpr (M == 2) return dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+        else return dpp_move<0x1B>(v);                         // quad_perm [3,2,1,0]
+    } else if constexpr (KQ == 1) {
+        if constexpr (M == 1) return dpp_move<0x141>(v);       // row_half_mirror: lane ^ 7
+        else if constexpr (M == 2) return dpp_move<0x140>(v);  // row_mirror:      lane ^ 15
+        else return dpp_move<0x128>(v);                        // row_ror:8:       lane ^ 8
+    } else {
+        if constexpr (M == 1)
+            return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+        else
+            return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ (16 * M)) << 2,
+                                                                          __builtin_bit_cast(int, v)));
+    }
+}
+
+struct Fast4Args {
+    const float *tw4;          // factors of this block, stack 0: (L/2, n/4, 4, 4)
+    int64_t tw_stack_stride;
+    const float *x_in;
+    View x_view;
+    float *x_out;              // forward output
+    View xo_view;
+    const float *g_out;        // backward
+    View g_view;
+    float *g_in;
+    View gi_view;
+    float *partial;            // (gridDim.x, S, L/2, 4 n)
+    int64_t batch;
+    int64_t ngroups;
+    int64_t groups_per_wg;
+};
+
+template <int L, bool INC, bool WITH_COLUMN>
+struct Factors4 {
+    static constexpr int NS = L / 2;
+    float row[NS][4];  // row[s][m] = T[r][r ^ m]
+    float colm[WITH_COLUMN ? NS : 1][4];  // colm[s][m] = T[r ^ m][r]
+
+    __device__ __forceinline__ void load(const float *tw, const FastCoords &c)
+    {
+        using P = Plan4<L, INC>;
+        constexpr int n = 1 << L;
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            constexpr int b = P::bit(s);
+            constexpr int lay = P::layout(s);
+            const int e = lay ? c.eB : c.eA;
+            const int r = (e >> b) & 3;
+            const int q = ((e >> (b + 2)) << b) | (e & ((1 << b) - 1));
+            const float *T = tw + ((int64_t)s * (n / 4) + q) * 16;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                row[s][m] = T[r * 4 + (r ^ m)];
+                if constexpr (WITH_COLUMN) colm[s][m] = T[(r ^ m) * 4 + r];
+            }
+        });
+    }
+};
+
+template <int L, bool INC, int R>
+__global__ __launch_bounds__(kFastThreads) void fast4_fw_kernel(Fast4Args a)
+{
+    using P = Plan4<L, INC>;
+    constexpr int NS = P::NS, SLOTS = P::SLOTS;
+    __shared__ float lds[P::NSWAP > 0 ? R * kFastRowWords : 1];
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int stack = blockIdx.y;
+    const FastCoords c = fast_coords<L>(t);
+
+    Factors4<L, INC, false> f;
+    f.load(a.tw4 + stack * a.tw_stack_stride, c);
+
+    const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
+    const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
+    const int ng = (int)(g1 - g0);
+    const int64_t row_end = g1 * SLOTS < a.batch ? g1 * SLOTS : a.batch;
+    const int rows_valid = (int)(row_end - g0 * SLOTS);
+    const __amdgpu_buffer_rsrc_t in_rs = make_rsrc(a.x_in + g0 * SLOTS * a.x_view.sb + stack * a.x_view.ss);
+    const __amdgpu_buffer_rsrc_t out_rs = make_rsrc(a.x_out + g0 * SLOTS * a.xo_view.sb + stack * a.xo_view.ss);
+    const int in_row = (int)(a.x_view.sb * 4), out_row = (int)(a.xo_view.sb * 4);
+    const int in_thr = c.eA < a.x_view.width ? c.slot * in_row + (int)(c.eA * a.x_view.se * 4) : kOob;
+    const int out_thr = c.eA < a.xo_view.width ? c.slot * out_row + (int)(c.eA * a.xo_view.se * 4) : kOob;
+
+    auto load_rows = [&](int grel, float (&v)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
+            v[r] = buf_load<float>(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
+        }
+    };
+    auto transpose = [&](float (&v)[R], int to_b) {
+        const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
+        __syncthreads();  // the previous transpose's reads are done
+#pragma unroll
+        for (int r = 0; r < R; ++r) lds[r * kFastRowWords + wr] = v[r];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; ++r) v[r] = lds[r * kFastRowWords + rd];
+    };
+
+    float nxt[R];
+    load_rows(0, nxt);
+    for (int grel = 0; grel < ng; grel += R) {
+        float v[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) v[r] = nxt[r];
+        load_rows(grel + R, nxt);
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            constexpr int KQ = P::kind(s);
+            if constexpr (P::layout(s) != P::layout_before(s)) transpose(v, P::layout(s));
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float y = f.row[s][0] * v[r];
+                y = fmaf(f.row[s][1], partner4<KQ, 1>(v[r], lane), y);
+                y = fmaf(f.row[s][2], partner4<KQ, 2>(v[r], lane), y);
+                y = fmaf(f.row[s][3], partner4<KQ, 3>(v[r], lane), y);
+                v[r] = y;
+            }
+        });
+        if constexpr (P::layout(NS - 1) != 0) transpose(v, 0);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
+            buf_store(out_rs, ok ? out_thr : kOob, (grel + r) * SLOTS * out_row, v[r]);
+        }
+    }
+}
+
+template <int L, bool INC>
+__global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
+{
+    using P = Plan4<L, INC>;
+    constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
+    __shared__ float lds[P::NSWAP > 0 ? kFastRowWords : 1];
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int stack = blockIdx.y;
+    const FastCoords c = fast_coords<L>(t);
+
+    Factors4<L, INC, true> f;
+    f.load(a.tw4 + stack * a.tw_stack_stride, c);
+    float acc[NS][4];  // acc[s][m] = sum g * (x of the partner at mask m) = dT[r][r ^ m]
+    static_for<0, NS>([&](auto S) {
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[S][m] = 0.0f;
+    });
+
+    const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
+    const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
+    const int ng = (int)(g1 - g0);
+    const int64_t row_end = g1 * SLOTS < a.batch ? g1 * SLOTS : a.batch;
+    const int rows_valid = (int)(row_end - g0 * SLOTS);
+    const __amdgpu_buffer_rsrc_t x_rs = make_rsrc(a.x_in + g0 * SLOTS * a.x_view.sb + stack * a.x_view.ss);
+    const __amdgpu_buffer_rsrc_t g_rs = make_rsrc(a.g_out + g0 * SLOTS * a.g_view.sb + stack * a.g_view.ss);
+    const __amdgpu_buffer_rsrc_t gi_rs = make_rsrc(a.g_in + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
+    const int x_row = (int)(a.x_view.sb * 4), g_row = (int)(a.g_view.sb * 4), gi_row = (int)(a.gi_view.sb * 4);
+    const int x_thr = c.eA < a.x_view.width ? c.slot * x_row + (int)(c.eA * a.x_view.se * 4) : kOob;
+    const int g_thr = c.eA < a.g_view.width ? c.slot * g_row + (int)(c.eA * a.g_view.se * 4) : kOob;
+    const int gi_thr = c.eA < a.gi_view.width ? c.slot * gi_row + (int)(c.eA * a.gi_view.se * 4) : kOob;
+
+    auto transpose = [&](float v, int to_b) -> float {
+        const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
+        __syncthreads();
+        lds[wr] = v;
+        __syncthreads();
+        return lds[rd];
+    };
+    auto row_ok = [&](int grp) { return grp * SLOTS + c.slot < rows_valid; };
+
+    float nx = buf_load<float>(x_rs, row_ok(0) ? x_thr : kOob, 0);
+    float ngr = buf_load<float>(g_rs, row_ok(0) ? g_thr : kOob, 0);
+    for (int grel = 0; grel < ng; ++grel) {
+        float v = nx, gv = ngr;
+        nx = buf_load<float>(x_rs, row_ok(grel + 1) ? x_thr : kOob, (grel + 1) * SLOTS * x_row);
+        ngr = buf_load<float>(g_rs, row_ok(grel + 1) ? g_thr : kOob, (grel + 1) * SLOTS * g_row);
+        float act[NS];
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            constexpr int KQ = P::kind(s);
+            if constexpr (P::layout(s) != P::layout_before(s)) v = transpose(v, P::layout(s));
+            act[s] = v;
+            if constexpr (s + 1 < NS) {
+                float y = f.row[s][0] * v;
+                y = fmaf(f.row[s][1], partner4<KQ, 1>(v, lane), y);
+                y = fmaf(f.row[s][2], partner4<KQ, 2>(v, lane), y);
+                y = fmaf(f.row[s][3], partner4<KQ, 3>(v, lane), y);
+                v = y;
+            }
+        });
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = NS - 1 - S;
+            constexpr int KQ = P::kind(s);
+            if constexpr (P::layout(s) != P::layout_after(s)) gv = transpose(gv, P::layout(s));
+            const float xs = act[s];
+            fmac_pinned(acc[s][0], gv, xs);
+            fmac_pinned(acc[s][1], gv, partner4<KQ, 1>(xs, lane));
+            fmac_pinned(acc[s][2], gv, partner4<KQ, 2>(xs, lane));
+            fmac_pinned(acc[s][3], gv, partner4<KQ, 3>(xs, lane));
+            // d_x[c] = sum_r T[r][c] g[r]: own column of the factor, partners' gradients
+            float d = f.colm[s][0] * gv;
+            d = fmaf(f.colm[s][1], partner4<KQ, 1>(gv, lane), d);
+            d = fmaf(f.colm[s][2], partner4<KQ, 2>(gv, lane), d);
+            d = fmaf(f.colm[s][3], partner4<KQ, 3>(gv, lane), d);
+            gv = d;
+        });
+        if constexpr (P::layout(0) != 0) gv = transpose(gv, 0);
+        buf_store(gi_rs, row_ok(grel) ? gi_thr : kOob, grel * SLOTS * gi_row, gv);
+    }
+
+    int t2 = t;
+    asm volatile("" : "+v"(t2));
+    const FastCoords c2 = fast_coords<L>(t2);
+    float *part = a.partial + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * (4 * n);
+    __shared__ float red[SLOTS > 1 ? 4 * 1024 : 1];
+    static_for<0, NS>([&](auto S) {
+        constexpr int s = S;
+        constexpr int b = P::bit(s);
+        constexpr int lay = P::layout(s);
+        const int e = lay ? c2.eB : c2.eA;
+        if constexpr (SLOTS == 1) {
+            const int r = (e >> b) & 3;
+            const int q = ((e >> (b + 2)) << b) | (e & ((1 << b) - 1));
+            float *d = part + (int64_t)s * (4 * n) + q * 16 + r * 4;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) d[r ^ m] = acc[s][m];
+        } else {
+            // add the row slots of this workgroup in ascending order, then one thread per entry
+            __syncthreads();
+#pragma unroll
+            for (int m = 0; m < 4; ++m) red[(c2.slot * n + e) * 4 + m] = acc[s][m];
+            __syncthreads();
+            for (int o = t2; o < 4 * n; o += kFastThreads) {
+                float sum = red[o];
+                for (int sl = 1; sl < SLOTS; ++sl) sum += red[sl * 4 * n + o];
+                const int eo = o >> 2, m = o & 3;
+                const int r = (eo >> b) & 3;
+                const int q = ((eo >> (b + 2)) << b) | (eo & ((1 << b) - 1));
+                part[(int64_t)s * (4 * n) + q * 16 + r * 4 + (r ^ m)] = sum;
+            }
+        }
+    });
+}
+
+}  // namespace bf

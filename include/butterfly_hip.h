@@ -90,7 +90,9 @@ int bf_butterfly_multiply_bw(const bf_problem *p, const void *twiddle, const voi
  * (torch_butterfly/multiply_base4.py:7-41), which the reference runs as PyTorch ops. */
 int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4,
                                    const void *twiddle2, const void *input, void *output,
-                                   void *stream);
+                                   void *workspace, size_t workspace_bytes, void *stream);
+
+size_t bf_butterfly_multiply_base4_fw_workspace_bytes(const bf_problem *p);
 
 size_t bf_butterfly_multiply_base4_bw_workspace_bytes(const bf_problem *p);
 

@@ -226,6 +226,31 @@ def test_c_abi_base4_matches_oracle(case):
     assert rel_err(d2.cpu().numpy(), d2_ref) < BW_TOL
 
 
+@pytest.mark.parametrize("L", [2, 4, 6, 8, 10])
+def test_base4_register_resident_kernels(L):
+    """Even log_n <= 10 in float runs on the base-4 twiddle-stationary kernels: every size,
+    both stride orders, one to three blocks, ragged batch, padded input, sliced output."""
+    from butterfly_amd import _capi
+    n = 1 << L
+    rng = np.random.default_rng(1700 + L)
+    for nb in (1, 2, 3):
+        for inc in (True, False):
+            for B, S, I, O in [(1, 1, n, n), (37, 2, n, n), (300, 1, n - 1, n - 1), (19, 4, n + 5, n // 2)]:
+                say("base4 fast case", L, nb, inc, B, S, I, O)
+                tw4 = (randn(rng, (S, nb, L // 2, n // 4, 4, 4), np.float32) / 2).astype(np.float32)
+                tw2 = np.zeros((S, nb, 0, n // 2, 2, 2), np.float32)
+                x = randn(rng, (B, S, I), np.float32)
+                g = randn(rng, (B, S, O), np.float32)
+                y_ref = oracle.butterfly_base4_fw(tw4, tw2, x, inc, O)
+                d4_ref, _, dx_ref = oracle.butterfly_base4_bw(tw4, tw2, x, g, inc)
+                y = _capi.multiply_base4_fw(dev(tw4), dev(tw2), dev(x), inc, O)
+                d4, _, dx = _capi.multiply_base4_bw(dev(tw4), dev(tw2), dev(x), dev(g), inc)
+                torch.cuda.synchronize()
+                assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL, (L, nb, inc, B, S, I, O)
+                assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL, (L, nb, inc, B, S, I, O)
+                assert rel_err(d4.cpu().numpy(), d4_ref) < BW_TOL, (L, nb, inc, B, S, I, O)
+
+
 def test_operators_match_oracle_and_autograd():
     """torch.ops.torch_butterfly.* end to end: views returned, autograd wired, lazy conj
     and transposed twiddle views accepted."""
