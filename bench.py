@@ -1,16 +1,20 @@
-"""Headline benchmark: butterfly_multiply forward + backward, batch 16384, n = 1024, fp32,
-nblocks = 2, decreasing stride first, on one MI355X, through torch.ops.torch_butterfly.
+"""Benchmark of the butterfly multiply on one MI355X, through torch.ops.torch_butterfly.
 
-    python bench.py [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--steps K] [--warmup W] [--config cfg2] [--no-cpu-baseline] [--calibrate-copy]
 
-Prints one JSON line.  ``value`` is algorithmic bytes (5 row-passes + twiddle traffic) per
-second over the K timed forward+backward steps with operands resident in HBM.  ``roofline``
-describes the dominant call, the backward pass, timed with device events on the launch
-stream.  ``cpu_baseline`` is the single-threaded reference C++ (or, where that build is
-absent, the repo's CPU restatement) timed on this host.
+The default workload (cfg2) is the headline one: forward + backward, batch 16384, n = 1024,
+fp32, nblocks = 2, decreasing stride first.  The other configurations of the baseline list
+(cfg1, cfg3, cfg4, cfg5) can be selected with --config.  One JSON line is printed.
+
+``value`` is algorithmic bytes (2 row passes forward, 3 backward, plus twiddle traffic) per
+second over the K timed steps, operands resident in HBM.  ``roofline`` describes the
+dominant call (the backward pass where there is one), timed with device events on the launch
+stream.  ``cpu_baseline`` is the single-threaded reference C++ (or, for base-4 and where the
+reference build is absent, the repo's CPU restatement) timed on this host on a bounded sample.
 """
 import argparse
 import json
+import math
 import os
 import subprocess
 import sys
@@ -20,51 +24,120 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-METRIC = "butterfly_multiply fwd+bwd GB/s & % HBM peak, batch 16384 n=1024 fp32"
 HBM_PEAK_GBS = 8000.0
-BW_TRAFFIC_BYTES = 289.4e6
+# HBM bytes per backward call of cfg2 (main kernel + reduce) from rocprofv3 FETCH_SIZE / WRITE_SIZE
+# scaled by a 64 MiB copy; see profiles/butterfly_fw_bw_cfg2_hbm_traffic.md
+CFG2_BW_TRAFFIC_BYTES = 289.4e6
 
-BATCH, NSTACKS, LOG_N, NBLOCKS, INCREASING = 16384, 1, 10, 2, False
+CONFIGS = {
+    # name: batch, nstacks, log_n, nblocks, increasing_stride, complex, base4, backward, cpu sample batch
+    "cfg1": dict(batch=2048, nstacks=1, log_n=10, nblocks=1, inc=True, cplx=False, base4=False, bw=False,
+                 cpu_batch=2048,
+                 metric="butterfly_multiply_fw GB/s, batch 2048 n=1024 fp32",
+                 workload="cfg1: butterfly_multiply_fw, input (2048,1,1024) fp32 N(0,1), twiddle (1,1,10,512,2,2) "
+                          "N(0,1/2), increasing_stride=True, forward only"),
+    "cfg2": dict(batch=16384, nstacks=1, log_n=10, nblocks=2, inc=False, cplx=False, base4=False, bw=True,
+                 cpu_batch=16384,
+                 metric="butterfly_multiply fwd+bwd GB/s & % HBM peak, batch 16384 n=1024 fp32",
+                 workload="cfg2: butterfly_multiply fw+bw, input (16384,1,1024) fp32 N(0,1), twiddle "
+                          "(1,2,10,512,2,2) N(0,1/2), increasing_stride=False, grad N(0,1)"),
+    "cfg3": dict(batch=8192, nstacks=1, log_n=12, nblocks=1, inc=True, cplx=True, base4=False, bw=True,
+                 cpu_batch=256,
+                 metric="butterfly_multiply fwd+bwd GB/s, complex64 FFT twiddles, batch 8192 n=4096",
+                 workload="cfg3: butterfly_multiply fw+bw complex64, normalised DFT twiddles (1,1,12,2048,2,2), "
+                          "input (8192,1,4096) bit-reversed outside the op, increasing_stride=True"),
+    "cfg4": dict(batch=16384, nstacks=4, log_n=8, nblocks=1, inc=True, cplx=False, base4=True, bw=True,
+                 cpu_batch=2048,
+                 metric="butterfly_multiply_base4 fwd+bwd GB/s, batch 16384 nstacks 4 n=256 fp32",
+                 workload="cfg4: butterfly_multiply_base4 fw+bw, input (16384,4,256) fp32 N(0,1), twiddle4 "
+                          "(4,1,4,64,4,4) N(0,1/4), increasing_stride=True"),
+    "cfg5": dict(batch=32768, nstacks=1, log_n=12, nblocks=2, inc=True, cplx=False, base4=False, bw=True,
+                 cpu_batch=1024,
+                 metric="butterfly_multiply fwd+bwd GB/s (op level), batch 32768 n=4096 fp32 nblocks 2",
+                 workload="cfg5 (op level): butterfly_multiply fw+bw of Butterfly(4096, 4096, nblocks=2), input "
+                          "(32768,1,4096) fp32 N(0,1), ortho twiddle (1,2,12,2048,2,2), increasing_stride=True"),
+}
 
 
-def algorithmic_bytes():
-    n = 1 << LOG_N
-    row = NSTACKS * n * 4
-    twiddle = NSTACKS * NBLOCKS * LOG_N * (n // 2) * 4 * 4
-    fw = 2 * row * BATCH + twiddle                 # read input, write output, read twiddle
-    bw = 3 * row * BATCH + 2 * twiddle             # read input + grad, write d_input; twiddle in, d_twiddle out
-    return fw, bw
+def algorithmic_bytes(c):
+    n = 1 << c["log_n"]
+    e = 8 if c["cplx"] else 4
+    row = c["nstacks"] * n * e
+    twiddle = c["nstacks"] * c["nblocks"] * c["log_n"] * (n // 2) * 4 * e
+    fw = 2 * row * c["batch"] + twiddle            # read input, write output, read twiddle
+    bw = 3 * row * c["batch"] + 2 * twiddle        # read input + grad, write d_input; twiddle in, d_twiddle out
+    return fw, (bw if c["bw"] else 0)
 
 
-def cpu_baseline():
-    """Reference csrc/cpu path (one thread) on the full workload, best of 3."""
+def cpu_baseline(name, c):
+    """Reference csrc/cpu path (one thread) on `cpu_batch` rows of the workload, best of 3."""
+    fw_b, bw_b = algorithmic_bytes(c)
+    scale = c["cpu_batch"] / c["batch"]
     ref_so = os.path.join(ROOT, "oracle", "_ref", "_butterfly_ref.so")
-    fw_b, bw_b = algorithmic_bytes()
-    if os.path.isfile(ref_so):
+    if os.path.isfile(ref_so) and not c["base4"]:
         out = subprocess.check_output(
-            [sys.executable, os.path.join(ROOT, "oracle", "ref_runner.py"), "time", str(BATCH), str(NSTACKS),
-             str(LOG_N), str(NBLOCKS), str(int(INCREASING)), "0", "3"], text=True)
+            [sys.executable, os.path.join(ROOT, "oracle", "ref_runner.py"), "time", str(c["cpu_batch"]),
+             str(c["nstacks"]), str(c["log_n"]), str(c["nblocks"]), str(int(c["inc"])), str(int(c["cplx"])), "3"],
+            text=True)
         r = json.loads(out.strip().splitlines()[-1])
         fw_s, bw_s, kind = r["fw_s"], r["bw_s"], "reference"
     else:
         import numpy as np
         from oracle import oracle
         rng = np.random.default_rng(0)
-        n = 1 << LOG_N
-        tw = (rng.standard_normal((NSTACKS, NBLOCKS, LOG_N, n // 2, 2, 2)) / np.sqrt(2)).astype(np.float32)
-        x = rng.standard_normal((BATCH, NSTACKS, n)).astype(np.float32)
-        g = rng.standard_normal((BATCH, NSTACKS, n)).astype(np.float32)
+        n, L, S, nb, B = 1 << c["log_n"], c["log_n"], c["nstacks"], c["nblocks"], c["cpu_batch"]
+        dt = np.complex64 if c["cplx"] else np.float32
+
+        def rnd(shape):
+            a = rng.standard_normal(shape)
+            if c["cplx"]:
+                a = (a + 1j * rng.standard_normal(shape)) / math.sqrt(2)
+            return a.astype(dt)
+
+        x, g = rnd((B, S, n)), rnd((B, S, n))
+        if c["base4"]:
+            tw4 = (rnd((S, nb, L // 2, n // 4, 4, 4)) / 2).astype(dt)
+            tw2 = (rnd((S, nb, L % 2, n // 2, 2, 2)) / math.sqrt(2)).astype(dt)
+            fw = lambda: oracle.butterfly_base4_fw(tw4, tw2, x, c["inc"])
+            bw = lambda: oracle.butterfly_base4_bw(tw4, tw2, x, g, c["inc"])
+        else:
+            tw = (rnd((S, nb, L, n // 2, 2, 2)) / math.sqrt(2)).astype(dt)
+            fw = lambda: oracle.butterfly_fw(tw, x, c["inc"])
+            bw = lambda: oracle.butterfly_bw(tw, x, g, c["inc"])
         fw_s = bw_s = float("inf")
         for _ in range(3):
-            t0 = time.perf_counter(); oracle.butterfly_fw(tw, x, INCREASING)
-            t1 = time.perf_counter(); oracle.butterfly_bw(tw, x, g, INCREASING)
+            t0 = time.perf_counter(); fw()
+            t1 = time.perf_counter()
+            if c["bw"]:
+                bw()
             t2 = time.perf_counter()
             fw_s, bw_s = min(fw_s, t1 - t0), min(bw_s, t2 - t1)
         kind = "port"
-    total = fw_s + bw_s
-    return {"value": (fw_b + bw_b) / total / 1e9, "unit": "GB/s", "cores": 1, "kind": kind,
-            "sample": f"full workload, batch {BATCH}, best of 3 (fw {fw_s * 1e3:.0f} ms, bw {bw_s * 1e3:.0f} ms)",
-            "rows_per_s": BATCH / total}
+    total = fw_s + (bw_s if c["bw"] else 0.0)
+    return {"value": (fw_b + bw_b) * scale / total / 1e9, "unit": "GB/s", "cores": 1, "kind": kind,
+            "sample": f"{c['cpu_batch']} of {c['batch']} rows of the workload, best of 3 "
+                      f"(fw {fw_s * 1e3:.0f} ms, bw {bw_s * 1e3:.0f} ms)",
+            "rows_per_s": c["cpu_batch"] / total}
+
+
+def make_operands(c, torch, dev):
+    n, L, S, nb, B = 1 << c["log_n"], c["log_n"], c["nstacks"], c["nblocks"], c["batch"]
+    dtype = torch.complex64 if c["cplx"] else torch.float32
+    if c["base4"]:
+        tw4 = (torch.randn(S, nb, L // 2, n // 4, 4, 4, dtype=dtype) / 2).to(dev)
+        tw2 = (torch.randn(S, nb, L % 2, n // 2, 2, 2, dtype=dtype) / 2 ** 0.5).to(dev)
+        tws = (tw4, tw2)
+    elif c["cplx"]:
+        from butterfly_amd import special
+        tws = (special.fft(n, normalized=True, with_br_perm=False).twiddle.detach().to(dev),)
+    elif nb == 2 and L == 12:
+        import butterfly_amd
+        tws = (butterfly_amd.Butterfly(n, n, bias=True, init="ortho", nblocks=2).twiddle.detach().to(dev),)
+    else:
+        tws = ((torch.randn(S, nb, L, n // 2, 2, 2, dtype=dtype) / 2 ** 0.5).to(dev),)
+    x = torch.randn(B, S, n, dtype=dtype).to(dev)
+    grad = torch.randn(B, S, n, dtype=dtype).to(dev)
+    return tws, x, grad
 
 
 def main():
@@ -72,75 +145,82 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="cfg2", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run plain 64 MiB device copies (a kernel of known traffic, for scaling "
+                    help="also run plain device copies of the input (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU; --gpus must be 1 (rows shard trivially, see DESIGN.md)")
+    c = CONFIGS[args.config]
 
     import torch
     import butterfly_amd  # noqa: F401
     ops = torch.ops.torch_butterfly
     assert torch.cuda.is_available(), "bench.py needs a HIP device"
     torch.manual_seed(0)
-    n = 1 << LOG_N
     dev = torch.device("cuda:0")
-    twiddle = (torch.randn(NSTACKS, NBLOCKS, LOG_N, n // 2, 2, 2) / 2 ** 0.5).to(dev)
-    x = torch.randn(BATCH, NSTACKS, n).to(dev)
-    grad = torch.randn(BATCH, NSTACKS, n).to(dev)
+    tws, x, grad = make_operands(c, torch, dev)
+    inc = c["inc"]
 
-    def step():
-        y = ops.butterfly_multiply_fw(twiddle, x, INCREASING, None)
-        dtw, dx = ops.butterfly_multiply_bw(twiddle, x, grad, INCREASING)
-        return y, dtw, dx
+    if c["base4"]:
+        fw_call = lambda: ops.butterfly_multiply_base4_fw(tws[0], tws[1], x, inc, None)
+        bw_call = lambda: ops.butterfly_multiply_base4_bw(tws[0], tws[1], x, grad, inc)
+    else:
+        fw_call = lambda: ops.butterfly_multiply_fw(tws[0], x, inc, None)
+        bw_call = lambda: ops.butterfly_multiply_bw(tws[0], x, grad, inc)
 
     for _ in range(args.warmup):
-        step()
+        fw_call()
+        if c["bw"]:
+            bw_call()
     torch.cuda.synchronize()
     if args.calibrate_copy:
         dst = torch.empty_like(x)
         for _ in range(5):
             dst.copy_(x)
         torch.cuda.synchronize()
-    fw_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    bw_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    fw_ev = [(ev(), ev()) for _ in range(args.steps)]
+    bw_ev = [(ev(), ev()) for _ in range(args.steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
         fw_ev[i][0].record()
-        ops.butterfly_multiply_fw(twiddle, x, INCREASING, None)
+        fw_call()
         fw_ev[i][1].record()
-        bw_ev[i][0].record()
-        ops.butterfly_multiply_bw(twiddle, x, grad, INCREASING)
-        bw_ev[i][1].record()
+        if c["bw"]:
+            bw_ev[i][0].record()
+            bw_call()
+            bw_ev[i][1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     fw_ms = sum(a.elapsed_time(b) for a, b in fw_ev) / args.steps
-    bw_ms = sum(a.elapsed_time(b) for a, b in bw_ev) / args.steps
+    bw_ms = sum(a.elapsed_time(b) for a, b in bw_ev) / args.steps if c["bw"] else 0.0
     ms_per_step = wall * 1e3 / args.steps
-    fw_b, bw_b = algorithmic_bytes()
+    fw_b, bw_b = algorithmic_bytes(c)
     value = (fw_b + bw_b) / (ms_per_step * 1e-3) / 1e9
-    bw_gbs = bw_b / (bw_ms * 1e-3) / 1e9
+    if c["bw"]:
+        dom_name, dom_b, dom_ms = "backward call (all its launches incl. the partial-sum reduce)", bw_b, bw_ms
+    else:
+        dom_name, dom_b, dom_ms = "forward call", fw_b, fw_ms
+    dom_gbs = dom_b / (dom_ms * 1e-3) / 1e9
     line = {
-        "metric": METRIC, "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "metric": c["metric"], "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "cfg2: butterfly_multiply fw+bw, input (16384,1,1024) fp32 N(0,1), twiddle "
-                               "(1,2,10,512,2,2) N(0,1/2), increasing_stride=False, grad N(0,1)"},
+        "vs_baseline": None, "dtype": "c64" if c["cplx"] else "f32", "data": "synthetic",
+        "config": {"workload": c["workload"]},
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
-        "rows_per_s": BATCH / (ms_per_step * 1e-3),
+        "rows_per_s": c["batch"] / (ms_per_step * 1e-3),
         "fw_ms": fw_ms, "bw_ms": bw_ms,
         "fw_GBps": fw_b / (fw_ms * 1e-3) / 1e9,
-        "roofline": {"bound": "hbm", "kernel": "butterfly_multiply_bw (main kernel + partial-sum reduce)",
-                     "achieved": bw_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bw_gbs / HBM_PEAK_GBS,
-                     # HBM bytes per backward call (main kernel + reduce) from rocprofv3 FETCH_SIZE /
-                     # WRITE_SIZE scaled by a 64 MiB copy; see profiles/butterfly_fw_bw_cfg2_hbm_traffic.md
-                     "traffic": BW_TRAFFIC_BYTES},
+        "roofline": {"bound": "hbm", "kernel": dom_name, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": dom_gbs / HBM_PEAK_GBS,
+                     "traffic": CFG2_BW_TRAFFIC_BYTES if args.config == "cfg2" else None},
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline()
+        line["cpu_baseline"] = cpu_baseline(args.config, c)
     print(json.dumps(line), flush=True)
 
 

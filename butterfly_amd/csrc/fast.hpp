@@ -330,6 +330,34 @@ __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, 
     });
 }
 
+// Moves the R values a thread holds (one per row in flight) through LDS: written at word
+// `wr`, read back at word `rd` after a barrier.  Four float rows travel as one 128-bit access.
+template <typename T, int R>
+__device__ __forceinline__ void transpose_rows(T *buf, int wr, int rd, T (&v)[R])
+{
+    if constexpr (sizeof(T) == 4 && R % 4 == 0) {
+        float4 *b4 = reinterpret_cast<float4 *>(buf);
+#pragma unroll
+        for (int r = 0; r < R; r += 4)
+            b4[(r / 4) * kFastRowWords + wr] = make_float4(v[r], v[r + 1], v[r + 2], v[r + 3]);
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; r += 4) {
+            const float4 q = b4[(r / 4) * kFastRowWords + rd];
+            v[r] = q.x;
+            v[r + 1] = q.y;
+            v[r + 2] = q.z;
+            v[r + 3] = q.w;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];
+    }
+}
+
 #ifndef BF_FAST_FW_WAVES
 #define BF_FAST_FW_WAVES 4
 #endif
@@ -339,7 +367,7 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     using P = FastPlan<L, NB, INC>;
     constexpr int NS = P::NS, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
-    __shared__ T lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
+    __shared__ __align__(16) T lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
@@ -393,11 +421,7 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
                 constexpr int to_b = P::layout(s);
                 T *buf = lds + par * R * kFastRowWords;
                 const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
-#pragma unroll
-                for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
-                __syncthreads();
-#pragma unroll
-                for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];
+                transpose_rows<T, R>(buf, wr, rd, v);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) v[r] = fw_product<K>(v[r], ta[s], tb[s], c.bperm_addr);
@@ -405,11 +429,7 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
         if constexpr (P::layout(NS - 1) != 0) {
             constexpr int par = P::fw_transposes_before(NS) & 1;
             T *buf = lds + par * R * kFastRowWords;
-#pragma unroll
-            for (int r = 0; r < R; ++r) buf[r * kFastRowWords + c.fB] = v[r];
-            __syncthreads();
-#pragma unroll
-            for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + c.fA];
+            transpose_rows<T, R>(buf, c.fB, c.fA, v);
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
