@@ -525,8 +525,14 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     using Pair = typename PairOf<T>::type;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
+    // complex64 at 9-10 stages does not fit 128 registers with both factor entries resident:
+    // the off-diagonal entries then live in LDS, one private slot per thread and stage.
+    constexpr bool TB_LDS = sizeof(T) == 8 && NS >= 9;
     __shared__ Pair lds[P::NSWAP > 0 ? 2 * kFastRowWords : 1];
     __shared__ T lds_carry[Q::DEFER ? kFastRowWords : 1];
+    constexpr int NTA = TB_LDS ? NS / 2 : 0;  // diagonal entries of the first stages live there too
+    __shared__ T lds_tb[TB_LDS ? NS * kFastThreads : 1];
+    __shared__ T lds_ta[NTA > 0 ? NTA * kFastThreads : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
@@ -538,7 +544,17 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     static_for<0, NS>([&](auto S) {
         acc_self[S] = zero_of(T());
         acc_cross[S] = zero_of(T());
+        if constexpr (TB_LDS) lds_tb[S * kFastThreads + t] = tb[S];
+        if constexpr (S < NTA) lds_ta[S * kFastThreads + t] = ta[S];
     });
+    auto tb_of = [&](auto S) -> T {
+        if constexpr (TB_LDS) return lds_tb[S * kFastThreads + t];
+        else return tb[S];
+    };
+    auto ta_of = [&](auto S) -> T {
+        if constexpr (S < NTA) return lds_ta[S * kFastThreads + t];
+        else return ta[S];
+    };
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
@@ -605,12 +621,15 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 if constexpr (j < cb) {
                     // reverse stage: uses the gradient before it passes through the stage
                     constexpr int s = b0 - j;
-                    bw_products<P::kind(s)>(acc_self[s], acc_cross[s], gv, cur[s], ta[s], tb[s], c.bperm_addr);
+                    bw_products<P::kind(s)>(acc_self[s], acc_cross[s], gv, cur[s], ta_of(std::integral_constant<int, s>{}),
+                                            tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
                 }
                 if constexpr (j < cf) {
                     constexpr int s = f0 + j;
                     nxt[s] = vF;
-                    if constexpr (s + 1 < NS) vF = fw_product<P::kind(s)>(vF, ta[s], tb[s], c.bperm_addr);
+                    if constexpr (s + 1 < NS)
+                        vF = fw_product<P::kind(s)>(vF, ta_of(std::integral_constant<int, s>{}),
+                                                    tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
                 }
             });
         });
@@ -621,19 +640,34 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     T actP[NS], actQ[NS];
     static_for<0, NS>([&](auto S) { actP[S] = zero_of(T()); });
     // iteration it pairs group it + 1 (forward) with group it (reverse); it = -1 .. ng - 1
-    T x0 = load_x(0), gm = load_g(-1);
-    T x1 = load_x(1), gp = load_g(0);
     T carry = zero_of(T());
     // with a deferred closing transpose one more (empty) iteration flushes the last group
     const int it_end = Q::DEFER ? ng + 1 : ng;
-    for (int it = -1; it < it_end; it += 2) {
-        const T xa = x0, ga = gm, xb = x1, gb = gp;
-        x0 = load_x(it + 3);
-        gm = load_g(it + 2);
-        x1 = load_x(it + 4);
-        gp = load_g(it + 3);
-        iteration(std::integral_constant<int, 0>{}, it, xa, ga, carry, actP, actQ);
-        iteration(std::integral_constant<int, 1>{}, it + 1, xb, gb, carry, actQ, actP);
+    if constexpr (sizeof(T) == 4) {
+        // operands are fetched two iterations ahead
+        T x0 = load_x(0), gm = load_g(-1);
+        T x1 = load_x(1), gp = load_g(0);
+        for (int it = -1; it < it_end; it += 2) {
+            const T xa = x0, ga = gm, xb = x1, gb = gp;
+            x0 = load_x(it + 3);
+            gm = load_g(it + 2);
+            x1 = load_x(it + 4);
+            gp = load_g(it + 3);
+            iteration(std::integral_constant<int, 0>{}, it, xa, ga, carry, actP, actQ);
+            iteration(std::integral_constant<int, 1>{}, it + 1, xb, gb, carry, actQ, actP);
+        }
+    } else {
+        // complex64: an iteration is long enough to cover the fetch, and four more registers
+        // held across a whole iteration would not fit
+        T x0 = load_x(0), gm = load_g(-1);
+        for (int it = -1; it < it_end; it += 2) {
+            const T xa = x0, ga = gm;
+            const T x1 = load_x(it + 2), gp = load_g(it + 1);
+            iteration(std::integral_constant<int, 0>{}, it, xa, ga, carry, actP, actQ);
+            x0 = load_x(it + 3);
+            gm = load_g(it + 2);
+            iteration(std::integral_constant<int, 1>{}, it + 1, x1, gp, carry, actQ, actP);
+        }
     }
 
     // Recompute the coordinates from a laundered thread id: sharing them with the prologue
@@ -658,7 +692,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             d[r + 1] = acc_cross[s];   // dT[r][1 - r]
         });
     } else {
-        __shared__ T red[2 * 1024];
+        // (the factor slots in LDS are dead by now and serve as the staging area)
+        __shared__ T red_own[TB_LDS ? 1 : 2 * 1024];
+        T *red = TB_LDS ? lds_tb : red_own;
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
             constexpr int bit = P::bit(s);
