@@ -181,23 +181,23 @@ def main():
         for _ in range(5):
             dst.copy_(x)
         torch.cuda.synchronize()
-    ev = lambda: torch.cuda.Event(enable_timing=True)
-    fw_ev = [(ev(), ev()) for _ in range(args.steps)]
-    bw_ev = [(ev(), ev()) for _ in range(args.steps)]
+    # One event between consecutive calls: the end of a call is the start of the next one.
+    per_step = 2 if c["bw"] else 1
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(per_step * args.steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    marks[0].record()
     for i in range(args.steps):
-        fw_ev[i][0].record()
         fw_call()
-        fw_ev[i][1].record()
+        marks[per_step * i + 1].record()
         if c["bw"]:
-            bw_ev[i][0].record()
             bw_call()
-            bw_ev[i][1].record()
+            marks[per_step * i + 2].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    fw_ms = sum(a.elapsed_time(b) for a, b in fw_ev) / args.steps
-    bw_ms = sum(a.elapsed_time(b) for a, b in bw_ev) / args.steps if c["bw"] else 0.0
+    span = lambda j: marks[j].elapsed_time(marks[j + 1])
+    fw_ms = sum(span(per_step * i) for i in range(args.steps)) / args.steps
+    bw_ms = sum(span(per_step * i + 1) for i in range(args.steps)) / args.steps if c["bw"] else 0.0
     ms_per_step = wall * 1e3 / args.steps
     fw_b, bw_b = algorithmic_bytes(c)
     value = (fw_b + bw_b) / (ms_per_step * 1e-3) / 1e9

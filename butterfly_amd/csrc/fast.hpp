@@ -93,17 +93,6 @@ struct FastPlan {
         int c = fw_transposes_before(NS);
         return c + (layout(NS - 1) != 0 ? 1 : 0);
     }
-    // The reverse walk starts in layout A and visits stages NS-1 .. 0; layout the running
-    // gradient is in when stage s is reached, and transposes performed before that point.
-    static constexpr int layout_after(int s) { return s == NS - 1 ? 0 : layout(s + 1); }
-    static constexpr int bw_transposes_before(int s)
-    {
-        int c = 0;
-        for (int j = NS - 1; j > s; --j) {
-            if (layout(j) != layout_after(j)) ++c;
-        }
-        return c;
-    }
 };
 
 template <int CTRL>
@@ -156,49 +145,33 @@ __device__ __forceinline__ void fmac_pinned(float2 &acc, float2 g, float2 x)
     fnmac_pinned(acc.y, g.x, x.y);
 }
 
-// acc += g * (x held by the partner thread), for the DPP exchange kinds: one v_fmac with a
-// DPP source.  The s_nop covers the two wait states a DPP read needs after a VALU write of
-// its source register.
-template <int K>
-__device__ __forceinline__ void fmac_partner_dpp(float &acc, float g, float x)
+// The three products of a backward stage, for one element and exchange kind K.  With p the
+// partner element of the pair and T the 2x2 factor:
+//   self  += g * conj(x)                 dT[me][me]
+//   cross += g_p * conj(x)               dT[p][me]: the gradient of the partner's output row
+//                                        times this thread's own input
+//   g     <- conj(T[me][me]) * g + conj(T[p][me]) * g_p
+// so one exchange (of g) serves both, and the thread needs the factor column of its element
+// (ta = T[me][me], tc = T[p][me]) rather than the row the forward stage uses.
+template <int K, typename T>
+__device__ __forceinline__ void bw_products(T &self, T &cross, T &g, T x, T ta, T tc, int bperm_addr)
 {
-    static_assert(K >= 0 && K < 4, "DPP kinds only");
-    if constexpr (K == 0)
-        asm volatile("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1"
-                     : "+v"(acc) : "v"(x), "v"(g));
-    else if constexpr (K == 1)
-        asm volatile("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1"
-                     : "+v"(acc) : "v"(x), "v"(g));
-    else if constexpr (K == 2)
-        asm volatile("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1"
-                     : "+v"(acc) : "v"(x), "v"(g));
-    else
-        asm volatile("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1"
-                     : "+v"(acc) : "v"(x), "v"(g));
-}
-
-// The three products of a backward stage, for one element and exchange kind K.
-//   self  += g * conj(x)            cross += g * conj(x of the partner)
-//   g     <- conj(ta) * g + (conj(tb) * g formed by the partner from its own tb)
-template <int K>
-__device__ __forceinline__ void bw_products(float &self, float &cross, float &g, float x, float ta, float tb,
-                                            int bperm_addr)
-{
+    const T gp = partner<K>(g, bperm_addr);
     fmac_pinned(self, g, x);
-    if constexpr (K < 4) fmac_partner_dpp<K>(cross, g, x);
-    else fmac_pinned(cross, g, partner<K>(x, bperm_addr));
-    const float m = tb * g;
-    if constexpr (K < 4) g = ta * g + partner<K>(m, bperm_addr);
-    else g = fmaf(ta, g, partner<K>(m, bperm_addr));
+    fmac_pinned(cross, gp, x);
+    g = macc(mul(conj_of(ta), g), tc, gp);
 }
 
-template <int K>
-__device__ __forceinline__ void bw_products(float2 &self, float2 &cross, float2 &g, float2 x, float2 ta,
-                                            float2 tb, int bperm_addr)
+// The same stage written with the factor row (ta = T[me][me], tb = T[me][p]) that the forward
+// replay holds anyway: two exchanges, but no third factor entry to keep.
+//   cross += g * conj(x_p)               dT[me][p]
+//   g     <- conj(ta) * g + (conj(tb) * g formed by the partner from its own tb)
+template <int K, typename T>
+__device__ __forceinline__ void bw_products_row(T &self, T &cross, T &g, T x, T ta, T tb, int bperm_addr)
 {
     fmac_pinned(self, g, x);
     fmac_pinned(cross, g, partner<K>(x, bperm_addr));
-    const float2 m = mul(conj_of(tb), g);
+    const T m = mul(conj_of(tb), g);
     g = add(mul(conj_of(ta), g), partner<K>(m, bperm_addr));
 }
 
@@ -308,11 +281,13 @@ struct FastFwArgs {
     int64_t groups_per_wg;
 };
 
-// Loads the two factor entries each thread needs for every stage.
+// Loads the factor entries each thread needs for every stage: its row (ta, tb) and, for the
+// backward kernel, the off-diagonal entry of its column (tc).
 template <typename T, int L, int NB, bool INC>
 __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, int64_t stage_stride,
                                              const int (&tw_stage)[kFastMaxStages], int chunk,
-                                             const FastCoords &c, T (&ta)[L * NB], T (&tb)[L * NB])
+                                             const FastCoords &c, T (&ta)[L * NB], T (&tb)[L * NB],
+                                             T (&tc)[L * NB], bool want_tc)
 {
     using P = FastPlan<L, NB, INC>;
     constexpr int n = 1 << L;
@@ -327,6 +302,7 @@ __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, 
         const T *Tm = twp + tw_stage[s] * stage_stride + i * 4;
         ta[s] = Tm[3 * r];   // T[r][r]
         tb[s] = Tm[r + 1];   // T[r][1 - r]
+        if (want_tc) tc[s] = Tm[2 - r];   // T[1 - r][r]
     });
 }
 
@@ -374,8 +350,9 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     const FastCoords c = fast_coords<L>(t);
     const int col = (chunk << L) + c.eA;  // column of this thread's element in the full row
 
-    T ta[NS], tb[NS];
-    load_factors<T, L, NB, INC>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, c, ta, tb);
+    T ta[NS], tb[NS], tc_unused[NS];
+    load_factors<T, L, NB, INC>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, c, ta, tb,
+                                tc_unused, false);
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
@@ -459,27 +436,45 @@ struct FastBwArgs {
 
 // Backward kernel, software-pipelined over rows: iteration i runs the forward replay of
 // row i + 1 (producing its stage inputs) together with the reverse sweep of row i (consuming
-// the stage inputs produced one iteration earlier).  The two walks change layout at mirrored
-// points, so they share every barrier, and their transposes travel through LDS as one
-// (x, g) pair.  Two independent dependency chains per thread also hide the DPP and
-// LDS latencies that a single chain exposes.
-template <int L, int NB, bool INC>
+// the stage inputs produced one iteration earlier).  Both walks change layout at the same
+// phase boundaries, so they share every barrier, and where they move in the same direction
+// their transposes travel through LDS as one (x, g) pair.  Two independent dependency chains
+// per thread also hide the DPP and LDS latencies that a single chain exposes.
+//
+// DIRECT: the operands arrive in LDS (see fast_bw_kernel) and each walk starts in the layout
+// of its first stage; otherwise they arrive in registers in layout A.
+template <int L, int NB, bool INC, bool DIRECT>
 struct BwPipe {
     using P = FastPlan<L, NB, INC>;
     static constexpr int NS = P::NS;
-    static constexpr int nF = P::fw_transposes_before(NS);
-    static constexpr int nB = P::bw_transposes_before(-1) + (P::layout(0) != 0 ? 1 : 0);
-    // When the reverse walk ends in layout B and the forward walk has no transpose left to
-    // pair with, the closing transpose of the reverse walk is carried into the next
-    // iteration and rides on that iteration's first barrier.
-    static constexpr bool DEFER = P::layout(0) != 0 && nF < nB && nB >= 2;
-    static constexpr int K = DEFER ? nB - 1 : (nF > nB ? nF : nB);  // phases 0..K; phase k >= 1 opens with transposes #k
-    // phase in which forward stage s / reverse stage s runs
-    static constexpr int fphase(int s) { return P::fw_transposes_before(s + 1); }
+    static constexpr int SF = DIRECT ? P::layout(0) : 0;       // layout the forward walk starts in
+    static constexpr int SB = DIRECT ? P::layout(NS - 1) : 0;  // layout the reverse walk starts in
+    // phase in which forward stage s / reverse stage s runs = layout changes up to and
+    // including the one in front of it
+    static constexpr int fphase(int s)
+    {
+        int c = 0, cur = SF;
+        for (int j = 0; j <= s; ++j)
+            if (P::layout(j) != cur) { ++c; cur = P::layout(j); }
+        return c;
+    }
     static constexpr int bphase(int s)
     {
-        return P::bw_transposes_before(s) + (P::layout(s) != P::layout_after(s) ? 1 : 0);
+        int c = 0, cur = SB;
+        for (int j = NS - 1; j >= s; --j)
+            if (P::layout(j) != cur) { ++c; cur = P::layout(j); }
+        return c;
     }
+    static constexpr int nF = fphase(NS - 1);
+    static constexpr int nB = bphase(0) + (P::layout(0) != 0 ? 1 : 0);  // + closing transpose back to A
+    // layout of each walk during phase k
+    static constexpr int flay(int k) { return SF ^ (k & 1); }
+    static constexpr int blay(int k) { return SB ^ (k & 1); }
+    // When the reverse walk ends in layout B and the forward walk has no transpose left to
+    // share a barrier with, the closing transpose of the reverse walk is carried into the
+    // next iteration and rides on that iteration's first barrier.
+    static constexpr bool DEFER = P::layout(0) != 0 && nF < nB && nB >= 2;
+    static constexpr int K = DEFER ? nB - 1 : (nF > nB ? nF : nB);  // phases 0..K; phase k >= 1 opens with transposes #k
     static constexpr int f_count(int k)
     {
         int c = 0;
@@ -517,30 +512,81 @@ __device__ __forceinline__ float pair_g(float2 p) { return p.y; }
 __device__ __forceinline__ float2 pair_x(float4 p) { return make_float2(p.x, p.y); }
 __device__ __forceinline__ float2 pair_g(float4 p) { return make_float2(p.z, p.w); }
 
+// ---- rows fetched straight into LDS -----------------------------------------------------------
+// A buffer load with the LDS modifier writes the dword each lane fetches to LDS at
+// M0 + 4 * lane: no register holds the row while it is in flight, and the thread that later
+// needs an element reads it from LDS in whatever layout its first stage wants.  Lanes whose
+// offset is out of range write zero.  The compiler does not see these loads (it would wait
+// for them at the next LDS access of any kind); the kernel waits for them itself.
+typedef int BufDesc __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ BufDesc make_desc(const void *base)
+{
+    const unsigned long long a = (unsigned long long)base;
+    BufDesc d;
+    d.x = (int)(unsigned)a;
+    d.y = (int)((a >> 32) & 0xffff);
+    d.z = (int)0x80000000u;
+    d.w = 0x00020000;
+    return d;
+}
+
+// lds_addr: LDS byte address the wavefront's 64 dwords start at (wave-uniform)
+__device__ __forceinline__ void load_row_to_lds(BufDesc desc, unsigned lds_addr, int voff, int soff)
+{
+    int keep_m0;
+    asm volatile("s_mov_b32 %0, m0\n\t"
+                 "s_mov_b32 m0, %1\n\t"
+                 "s_nop 0\n\t"
+                 "buffer_load_dword %2, %3, %4 offen lds\n\t"
+                 "s_mov_b32 m0, %0"
+                 : "=&s"(keep_m0)
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(desc), "s"(soff)
+                 : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_rows_in_lds()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+typedef __attribute__((address_space(3))) float LdsFloat;
+
 template <typename T, int L, int NB, bool INC>
 __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 {
     using P = FastPlan<L, NB, INC>;
-    using Q = BwPipe<L, NB, INC>;
+    constexpr int W = (int)sizeof(T) / 4;
+    // float rows are fetched straight into LDS; complex64 has no LDS to spare for that at
+    // 9-10 stages and fetches into registers
+    constexpr bool DIRECT = W == 1;
+    using Q = BwPipe<L, NB, INC, DIRECT>;
     using Pair = typename PairOf<T>::type;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
-    // complex64 at 9-10 stages does not fit 128 registers with both factor entries resident:
-    // the off-diagonal entries then live in LDS, one private slot per thread and stage.
-    constexpr bool TB_LDS = sizeof(T) == 8 && NS >= 9;
-    __shared__ Pair lds[P::NSWAP > 0 ? 2 * kFastRowWords : 1];
+    // Three factor entries per stage (the row for the forward replay, the column for the
+    // reverse sweep) do not fit 128 registers next to the sums for long schedules: the
+    // off-diagonal row entries, which only the replay reads, then live in LDS, one private
+    // slot per thread and stage; complex64 at 9-10 stages also keeps half of the diagonal
+    // entries there.
+    constexpr bool COL = !(W == 2 && NS >= 9);  // reverse sweep written with the factor column
+    constexpr bool TB_LDS = NS * W > 10;
+    constexpr int NTA = (W == 2 && NS >= 9) ? NS / 2 : 0;
+    __shared__ Pair lds[Q::K > 0 ? 2 * kFastRowWords : 1];
     __shared__ T lds_carry[Q::DEFER ? kFastRowWords : 1];
-    constexpr int NTA = TB_LDS ? NS / 2 : 0;  // diagonal entries of the first stages live there too
     __shared__ T lds_tb[TB_LDS ? NS * kFastThreads : 1];
     __shared__ T lds_ta[NTA > 0 ? NTA * kFastThreads : 1];
+    __shared__ float lds_rows[DIRECT ? 8 * kFastRowWords : 1];  // x slots 0..3, output-gradient slots 4..7
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
     const FastCoords c = fast_coords<L>(t);
     const int col = (chunk << L) + c.eA;  // column of this thread's element in the full row
 
-    T ta[NS], tb[NS], acc_self[NS], acc_cross[NS];
-    load_factors<T, L, NB, INC>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, c, ta, tb);
+    T ta[NS], tb[NS], tc[NS], acc_self[NS], acc_cross[NS];
+    load_factors<T, L, NB, INC>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, c, ta, tb, tc,
+                                COL);
     static_for<0, NS>([&](auto S) {
         acc_self[S] = zero_of(T());
         acc_cross[S] = zero_of(T());
@@ -561,57 +607,96 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const int ng = (int)(g1 - g0);
     const int64_t row_end = g1 * SLOTS < a.batch ? g1 * SLOTS : a.batch;
     const int rows_valid = (int)(row_end - g0 * SLOTS);
-    const __amdgpu_buffer_rsrc_t x_rs =
-        make_rsrc(reinterpret_cast<const T *>(a.x_in) + g0 * SLOTS * a.x_view.sb + stack * a.x_view.ss);
-    const __amdgpu_buffer_rsrc_t g_rs =
-        make_rsrc(reinterpret_cast<const T *>(a.g_out) + g0 * SLOTS * a.g_view.sb + stack * a.g_view.ss);
+    const T *x_base = reinterpret_cast<const T *>(a.x_in) + g0 * SLOTS * a.x_view.sb + stack * a.x_view.ss;
+    const T *g_base = reinterpret_cast<const T *>(a.g_out) + g0 * SLOTS * a.g_view.sb + stack * a.g_view.ss;
     const __amdgpu_buffer_rsrc_t gi_rs =
         make_rsrc(reinterpret_cast<T *>(a.g_in) + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
     const int x_row = (int)(a.x_view.sb * EB), g_row = (int)(a.g_view.sb * EB), gi_row = (int)(a.gi_view.sb * EB);
+    const int gi_thr = col < a.gi_view.width ? c.slot * gi_row + (int)(col * a.gi_view.se * EB) : kOob;
+    auto group_ok = [&](int grp) { return grp >= 0 && grp * SLOTS + c.slot < rows_valid; };
+    auto store_grad = [&](int grp, T gval) {
+        buf_store(gi_rs, group_ok(grp) ? gi_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * gi_row, gval);
+    };
+
+    // --- operand fetch, register flavour: thread t holds its layout-A element
+    const __amdgpu_buffer_rsrc_t x_rs = make_rsrc(x_base), g_rs = make_rsrc(g_base);
     const int x_thr = col < a.x_view.width ? c.slot * x_row + (int)(col * a.x_view.se * EB) : kOob;
     const int g_thr = col < a.g_view.width ? c.slot * g_row + (int)(col * a.g_view.se * EB) : kOob;
-    const int gi_thr = col < a.gi_view.width ? c.slot * gi_row + (int)(col * a.gi_view.se * EB) : kOob;
-
-    auto group_ok = [&](int grp) { return grp >= 0 && grp * SLOTS + c.slot < rows_valid; };
     auto load_x = [&](int grp) {
         return buf_load<T>(x_rs, group_ok(grp) ? x_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row);
     };
     auto load_g = [&](int grp) {
         return buf_load<T>(g_rs, group_ok(grp) ? g_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * g_row);
     };
-    auto store_grad = [&](int grp, T gval) {
-        buf_store(gi_rs, group_ok(grp) ? gi_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * gi_row, gval);
+    // --- operand fetch, LDS flavour: lane l of wavefront w fetches element 64 w + l of the row
+    // group, which lands at the padded word 65 w + l of the slot
+    const BufDesc x_desc = make_desc(x_base), g_desc = make_desc(g_base);
+    const int slot_d = t >> L, col_d = (chunk << L) + (t & (n - 1));
+    const int x_dma = col_d < a.x_view.width ? slot_d * x_row + (int)(col_d * a.x_view.se * EB) : kOob;
+    const int g_dma = col_d < a.g_view.width ? slot_d * g_row + (int)(col_d * a.g_view.se * EB) : kOob;
+    const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
+    auto group_ok_d = [&](int grp) { return grp >= 0 && grp * SLOTS + slot_d < rows_valid; };
+    // x of group grp -> x slot (grp & 3); output gradient of group grp -> gradient slot (grp & 3).
+    // Rows are requested AHEAD iterations before they are read: one is enough when the wait
+    // for them sits late in the iteration (behind two or more barriers), otherwise two.
+    constexpr int AHEAD = Q::K >= 2 ? 1 : 2;
+    auto fetch_x = [&](int grp) {
+        load_row_to_lds(x_desc, rows_addr + (grp & 3) * kFastRowWords * 4, group_ok_d(grp) ? x_dma : kOob,
+                        (grp < 0 ? 0 : grp) * SLOTS * x_row);
+    };
+    auto fetch_g = [&](int grp) {
+        load_row_to_lds(g_desc, rows_addr + (4 + (grp & 3)) * kFastRowWords * 4, group_ok_d(grp) ? g_dma : kOob,
+                        (grp < 0 ? 0 : grp) * SLOTS * g_row);
     };
 
     // One pipelined iteration: forward replay of group it + 1 into `nxt`, reverse sweep of
-    // group it out of `cur`; vF / gv enter holding the freshly loaded x and g.  `carry` holds
-    // the previous group's input gradient still in layout B (DEFER only).  FLIP alternates
-    // between the two unrolled calls so that LDS buffers keep alternating across iterations
-    // when the number of phases is odd.
+    // group it out of `cur`.  Register flavour: vF / gv enter holding the freshly loaded x and
+    // g.  LDS flavour: they are read from the row slots, and the rows of a later iteration
+    // are requested; the rows of the next iteration must have landed, for every wavefront,
+    // before it starts, so each wavefront waits for its own share of them just before the
+    // last barrier of this iteration.  `carry` holds the previous group's input gradient still in layout B (DEFER
+    // only).  FLIP alternates between the two unrolled calls: it gives the parity of `it` at
+    // compile time and keeps the LDS buffers alternating when the number of phases is odd.
     auto iteration = [&](auto FLIP, int it, T vF, T gv, T &carry, T (&cur)[NS], T (&nxt)[NS]) {
         constexpr int flip = decltype(FLIP)::value;
+        // Memory operations issued after the requests the wait is for and before the wait: this
+        // iteration's store when it comes first and, if those requests were made one iteration
+        // earlier, that iteration's store and this iteration's two requests.
+        constexpr int YOUNGER = ((Q::DEFER && Q::K > 1) ? 1 : 0) + (AHEAD == 2 ? 3 : 0);
+        if constexpr (DIRECT) {
+            fetch_x(it + 1 + AHEAD);
+            fetch_g(it + AHEAD);
+            const float xv = lds_rows[((it + 1) & 3) * kFastRowWords + (Q::SF ? c.fB : c.fA)];
+            const float gr = lds_rows[(4 + (it & 3)) * kFastRowWords + (Q::SB ? c.fB : c.fA)];
+            vF = xv;
+            gv = gr;
+        }
         static_for<0, Q::K + 1>([&](auto KK) {
             constexpr int k = KK;
             if constexpr (k >= 1) {
                 constexpr bool hasF = k <= Q::nF, hasB = k <= Q::nB;
-                constexpr int to_b = k & 1;  // both walks start in layout A and alternate
+                constexpr bool paired = hasF && hasB && Q::flay(k) == Q::blay(k);
                 Pair *buf = lds + ((k + flip * Q::K) & 1) * kFastRowWords;
                 T *bufs = reinterpret_cast<T *>(buf);
-                const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
-                if constexpr (hasF && hasB) buf[wr] = make_pair(vF, gv);
-                else if constexpr (hasF) bufs[2 * wr] = vF;
-                else bufs[2 * wr + 1] = gv;
+                const int wrF = Q::flay(k) ? c.fA : c.fB, rdF = Q::flay(k) ? c.fB : c.fA;
+                const int wrB = Q::blay(k) ? c.fA : c.fB, rdB = Q::blay(k) ? c.fB : c.fA;
+                if constexpr (paired) {
+                    buf[wrF] = make_pair(vF, gv);
+                } else {
+                    if constexpr (hasF) bufs[2 * wrF] = vF;
+                    if constexpr (hasB) bufs[2 * wrB + 1] = gv;
+                }
                 if constexpr (Q::DEFER && k == 1) lds_carry[c.fB] = carry;
+                if constexpr (DIRECT && k == Q::K) wait_rows_in_lds<YOUNGER>();
                 __syncthreads();
                 if constexpr (Q::DEFER && k == 1) store_grad(it - 1, lds_carry[c.fA]);
-                if constexpr (hasF && hasB) {
-                    const Pair v2 = buf[rd];
+                if constexpr (paired) {
+                    const Pair v2 = buf[rdF];
                     vF = pair_x(v2);
                     gv = pair_g(v2);
-                } else if constexpr (hasF) {
-                    vF = bufs[2 * rd];
                 } else {
-                    gv = bufs[2 * rd + 1];
+                    if constexpr (hasF) vF = bufs[2 * rdF];
+                    if constexpr (hasB) gv = bufs[2 * rdB + 1];
                 }
             }
             constexpr int cf = Q::f_count(k), cb = Q::b_count(k);
@@ -621,8 +706,13 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 if constexpr (j < cb) {
                     // reverse stage: uses the gradient before it passes through the stage
                     constexpr int s = b0 - j;
-                    bw_products<P::kind(s)>(acc_self[s], acc_cross[s], gv, cur[s], ta_of(std::integral_constant<int, s>{}),
-                                            tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
+                    if constexpr (COL)
+                        bw_products<P::kind(s)>(acc_self[s], acc_cross[s], gv, cur[s],
+                                                ta_of(std::integral_constant<int, s>{}), tc[s], c.bperm_addr);
+                    else
+                        bw_products_row<P::kind(s)>(acc_self[s], acc_cross[s], gv, cur[s],
+                                                    ta_of(std::integral_constant<int, s>{}),
+                                                    tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
                 }
                 if constexpr (j < cf) {
                     constexpr int s = f0 + j;
@@ -633,6 +723,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 }
             });
         });
+        if constexpr (DIRECT && Q::K == 0) wait_rows_in_lds<3>();
         if constexpr (Q::DEFER) carry = gv;
         else store_grad(it, gv);
     };
@@ -643,19 +734,20 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     T carry = zero_of(T());
     // with a deferred closing transpose one more (empty) iteration flushes the last group
     const int it_end = Q::DEFER ? ng + 1 : ng;
-    if constexpr (sizeof(T) == 4) {
-        // operands are fetched two iterations ahead
-        T x0 = load_x(0), gm = load_g(-1);
-        T x1 = load_x(1), gp = load_g(0);
-        for (int it = -1; it < it_end; it += 2) {
-            const T xa = x0, ga = gm, xb = x1, gb = gp;
-            x0 = load_x(it + 3);
-            gm = load_g(it + 2);
-            x1 = load_x(it + 4);
-            gp = load_g(it + 3);
-            iteration(std::integral_constant<int, 0>{}, it, xa, ga, carry, actP, actQ);
-            iteration(std::integral_constant<int, 1>{}, it + 1, xb, gb, carry, actQ, actP);
+    if constexpr (DIRECT) {
+        fetch_x(0);
+        fetch_g(-1);  // nothing to sweep yet: a row of zeros
+        if constexpr (AHEAD == 2) {
+            fetch_x(1);
+            fetch_g(0);
         }
+        wait_rows_in_lds<0>();
+        __syncthreads();
+        for (int it = -1; it < it_end; it += 2) {
+            iteration(std::integral_constant<int, 0>{}, it, zero_of(T()), zero_of(T()), carry, actP, actQ);
+            iteration(std::integral_constant<int, 1>{}, it + 1, zero_of(T()), zero_of(T()), carry, actQ, actP);
+        }
+        wait_rows_in_lds<0>();  // requests past the last group (they fetch nothing)
     } else {
         // complex64: an iteration is long enough to cover the fetch, and four more registers
         // held across a whole iteration would not fit
@@ -689,7 +781,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
             T *d = part + (int64_t)s * a.partial_slot + i * 4;
             d[3 * r] = acc_self[s];    // dT[r][r]
-            d[r + 1] = acc_cross[s];   // dT[r][1 - r]
+            d[COL ? 2 - r : r + 1] = acc_cross[s];   // dT[1 - r][r] (column form) or dT[r][1 - r]
         });
     } else {
         // (the factor slots in LDS are dead by now and serve as the staging area)
@@ -711,8 +803,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 for (int sl = 1; sl < SLOTS; ++sl) sum = add(sum, red[sl * 2 * n + t2]);
                 const int r = (eo >> bit) & 1;
                 const int i = ((eo >> (bit + 1)) << bit) | (eo & ((1 << bit) - 1));
-                // j = 0: dT[r][r], j = 1: dT[r][1 - r]
-                part[(int64_t)s * a.partial_slot + i * 4 + (j ? r + 1 : 3 * r)] = sum;
+                // j = 0: dT[r][r], j = 1: dT[1 - r][r] (column form) or dT[r][1 - r]
+                part[(int64_t)s * a.partial_slot + i * 4 + (j ? (COL ? 2 - r : r + 1) : 3 * r)] = sum;
             }
         });
     }
