@@ -72,7 +72,8 @@ struct FastPlan {
         }
         return cur;
     }
-    static constexpr int layout_before(int s) { return s == 0 ? 0 : layout(s - 1); }
+    // (`start`: layout the walk is in before its first stage; A when rows arrive in registers)
+    static constexpr int layout_before(int s, int start = 0) { return s == 0 ? start : layout(s - 1); }
     // exchange kind: 0..3 DPP pattern for phi bit, 4 swizzle xor 16, 5 bpermute xor 32
     static constexpr int kind(int s)
     {
@@ -80,17 +81,17 @@ struct FastPlan {
         return b >= 6 ? b - 6 : b;
     }
     // LDS transposes performed before stage s of a forward walk (for buffer parity)
-    static constexpr int fw_transposes_before(int s)
+    static constexpr int fw_transposes_before(int s, int start = 0)
     {
-        int c = 0, cur = 0;
+        int c = 0, cur = start;
         for (int j = 0; j < s; ++j) {
             if (layout(j) != cur) { ++c; cur = layout(j); }
         }
         return c;
     }
-    static constexpr int fw_transposes_total()
+    static constexpr int fw_transposes_total(int start = 0)
     {
-        int c = fw_transposes_before(NS);
+        int c = fw_transposes_before(NS, start);
         return c + (layout(NS - 1) != 0 ? 1 : 0);
     }
 };
@@ -260,6 +261,47 @@ __device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, int voff, in
     __builtin_amdgcn_raw_buffer_store_b64(raw, r, voff, soff, 0);
 }
 
+// ---- rows fetched straight into LDS -----------------------------------------------------------
+// A buffer load with the LDS modifier writes the dword each lane fetches to LDS at
+// M0 + 4 * lane: no register holds the row while it is in flight, and the thread that later
+// needs an element reads it from LDS in whatever layout its first stage wants.  Lanes whose
+// offset is out of range write zero.  The compiler does not see these loads (it would wait
+// for them at the next LDS access of any kind); the kernel waits for them itself.
+typedef int BufDesc __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ BufDesc make_desc(const void *base)
+{
+    const unsigned long long a = (unsigned long long)base;
+    BufDesc d;
+    d.x = (int)(unsigned)a;
+    d.y = (int)((a >> 32) & 0xffff);
+    d.z = (int)0x80000000u;
+    d.w = 0x00020000;
+    return d;
+}
+
+// lds_addr: LDS byte address the wavefront's 64 dwords start at (wave-uniform)
+__device__ __forceinline__ void load_row_to_lds(BufDesc desc, unsigned lds_addr, int voff, int soff)
+{
+    int keep_m0;
+    asm volatile("s_mov_b32 %0, m0\n\t"
+                 "s_mov_b32 m0, %1\n\t"
+                 "s_nop 0\n\t"
+                 "buffer_load_dword %2, %3, %4 offen lds\n\t"
+                 "s_mov_b32 m0, %0"
+                 : "=&s"(keep_m0)
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(desc), "s"(soff)
+                 : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_rows_in_lds()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+typedef __attribute__((address_space(3))) float LdsFloat;
+
 constexpr int kFastMaxStages = 20;
 
 // Rows longer than 1024 are handled as independent 1024-element chunks (blockIdx.z) for the
@@ -308,7 +350,9 @@ __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, 
 
 // Moves the R values a thread holds (one per row in flight) through LDS: written at word
 // `wr`, read back at word `rd` after a barrier.  Four float rows travel as one 128-bit access.
-template <typename T, int R>
+// WAIT: the wavefront first waits for the rows it has requested into LDS, so that the barrier
+// also publishes those.
+template <typename T, int R, bool WAIT = false>
 __device__ __forceinline__ void transpose_rows(T *buf, int wr, int rd, T (&v)[R])
 {
     if constexpr (sizeof(T) == 4 && R % 4 == 0) {
@@ -316,6 +360,7 @@ __device__ __forceinline__ void transpose_rows(T *buf, int wr, int rd, T (&v)[R]
 #pragma unroll
         for (int r = 0; r < R; r += 4)
             b4[(r / 4) * kFastRowWords + wr] = make_float4(v[r], v[r + 1], v[r + 2], v[r + 3]);
+        if constexpr (WAIT) wait_rows_in_lds<0>();
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < R; r += 4) {
@@ -328,6 +373,7 @@ __device__ __forceinline__ void transpose_rows(T *buf, int wr, int rd, T (&v)[R]
     } else {
 #pragma unroll
         for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
+        if constexpr (WAIT) wait_rows_in_lds<0>();
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];
@@ -341,9 +387,15 @@ template <typename T, int L, int NB, bool INC, int R>
 __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel(FastFwArgs a)
 {
     using P = FastPlan<L, NB, INC>;
-    constexpr int NS = P::NS, SLOTS = P::SLOTS;
+    constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
-    __shared__ __align__(16) T lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
+    // float rows are fetched straight into LDS, one iteration (R row groups) ahead, and the
+    // walk starts in the layout of its first stage; complex64 rows arrive in registers, layout A
+    constexpr bool DIRECT = sizeof(T) == 4;
+    constexpr int SF = DIRECT ? P::layout(0) : 0;
+    constexpr int TT = P::fw_transposes_total(SF);  // barriers per iteration
+    __shared__ __align__(16) T lds[TT > 0 ? 2 * R * kFastRowWords : 1];
+    __shared__ float lds_rows[DIRECT ? 2 * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
@@ -359,8 +411,8 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     const int ng = (int)(g1 - g0);
     const int64_t row_end = g1 * SLOTS < a.batch ? g1 * SLOTS : a.batch;
     const int rows_valid = (int)(row_end - g0 * SLOTS);
-    const __amdgpu_buffer_rsrc_t in_rs =
-        make_rsrc(reinterpret_cast<const T *>(a.in) + g0 * SLOTS * a.in_view.sb + stack * a.in_view.ss);
+    const T *in_base = reinterpret_cast<const T *>(a.in) + g0 * SLOTS * a.in_view.sb + stack * a.in_view.ss;
+    const __amdgpu_buffer_rsrc_t in_rs = make_rsrc(in_base);
     const __amdgpu_buffer_rsrc_t out_rs =
         make_rsrc(reinterpret_cast<T *>(a.out) + g0 * SLOTS * a.out_view.sb + stack * a.out_view.ss);
     const int in_row = (int)(a.in_view.sb * EB), out_row = (int)(a.out_view.sb * EB);
@@ -375,45 +427,80 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
             v[r] = buf_load<T>(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
         }
     };
+    // LDS flavour: lane l of wavefront w fetches element 64 w + l of each row group, which lands
+    // at the padded word 65 w + l of the group's slot; `set` alternates between iterations
+    const BufDesc in_desc = make_desc(in_base);
+    const int slot_d = t >> L, col_d = (chunk << L) + (t & (n - 1));
+    const int in_dma = col_d < a.in_view.width ? slot_d * in_row + (int)(col_d * a.in_view.se * EB) : kOob;
+    const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
+    auto fetch_rows = [&](int grel, int set) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const bool ok = (grel + r) * SLOTS + slot_d < rows_valid;
+            load_row_to_lds(in_desc, rows_addr + (set * R + r) * kFastRowWords * 4, ok ? in_dma : kOob,
+                            (grel + r) * SLOTS * in_row);
+        }
+    };
 
     T nxt[R];
-    load_rows(0, nxt);
-    // R stores that the range check discards.  They put the same "loads, then stores" history
-    // in front of the first iteration as every later iteration has, so the wait for the
-    // prefetched rows at the top of the loop is emitted as "all but the newest R operations"
-    // and does not also wait for the previous iteration's stores to be acknowledged.
+    if constexpr (DIRECT) {
+        fetch_rows(0, 0);
+        wait_rows_in_lds<0>();
+        __syncthreads();
+    } else {
+        load_rows(0, nxt);
+        // R stores that the range check discards.  They put the same "loads, then stores"
+        // history in front of the first iteration as every later iteration has, so the wait for
+        // the prefetched rows at the top of the loop is emitted as "all but the newest R
+        // operations" and does not also wait for the previous iteration's stores to be
+        // acknowledged.
 #pragma unroll
-    for (int r = 0; r < R; ++r) buf_store(out_rs, kOob, EB * r, zero_of(T()));
+        for (int r = 0; r < R; ++r) buf_store(out_rs, kOob, EB * r, zero_of(T()));
+    }
     for (int grel = 0; grel < ng; grel += R) {
         T v[R];
+        if constexpr (DIRECT) {
+            const int set = (grel / R) & 1;
+            fetch_rows(grel + R, set ^ 1);
 #pragma unroll
-        for (int r = 0; r < R; ++r) v[r] = nxt[r];
-        load_rows(grel + R, nxt);
+            for (int r = 0; r < R; ++r) {
+                const float x = lds_rows[(set * R + r) * kFastRowWords + (SF ? c.fB : c.fA)];
+                v[r] = x;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r) v[r] = nxt[r];
+            load_rows(grel + R, nxt);
+        }
 
+        // The rows requested above must be in LDS, for every wavefront, when the next
+        // iteration starts: each wavefront waits for its own just before the last barrier.
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
             constexpr int K = P::kind(s);
-            if constexpr (P::layout(s) != P::layout_before(s)) {
-                constexpr int par = P::fw_transposes_before(s) & 1;
+            if constexpr (P::layout(s) != P::layout_before(s, SF)) {
+                constexpr int nth = P::fw_transposes_before(s, SF);  // transposes done so far
                 constexpr int to_b = P::layout(s);
-                T *buf = lds + par * R * kFastRowWords;
+                T *buf = lds + (nth & 1) * R * kFastRowWords;
                 const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
-                transpose_rows<T, R>(buf, wr, rd, v);
+                transpose_rows<T, R, DIRECT && nth + 1 == TT>(buf, wr, rd, v);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) v[r] = fw_product<K>(v[r], ta[s], tb[s], c.bperm_addr);
         });
         if constexpr (P::layout(NS - 1) != 0) {
-            constexpr int par = P::fw_transposes_before(NS) & 1;
-            T *buf = lds + par * R * kFastRowWords;
-            transpose_rows<T, R>(buf, c.fB, c.fA, v);
+            constexpr int nth = P::fw_transposes_before(NS, SF);
+            T *buf = lds + (nth & 1) * R * kFastRowWords;
+            transpose_rows<T, R, DIRECT>(buf, c.fB, c.fA, v);
         }
+        if constexpr (DIRECT && TT == 0) wait_rows_in_lds<0>();
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
             buf_store(out_rs, ok ? out_thr : kOob, (grel + r) * SLOTS * out_row, v[r]);
         }
     }
+    if constexpr (DIRECT) wait_rows_in_lds<0>();  // requests past the last group (they fetch nothing)
 }
 
 struct FastBwArgs {
@@ -511,47 +598,6 @@ __device__ __forceinline__ float pair_x(float2 p) { return p.x; }
 __device__ __forceinline__ float pair_g(float2 p) { return p.y; }
 __device__ __forceinline__ float2 pair_x(float4 p) { return make_float2(p.x, p.y); }
 __device__ __forceinline__ float2 pair_g(float4 p) { return make_float2(p.z, p.w); }
-
-// ---- rows fetched straight into LDS -----------------------------------------------------------
-// A buffer load with the LDS modifier writes the dword each lane fetches to LDS at
-// M0 + 4 * lane: no register holds the row while it is in flight, and the thread that later
-// needs an element reads it from LDS in whatever layout its first stage wants.  Lanes whose
-// offset is out of range write zero.  The compiler does not see these loads (it would wait
-// for them at the next LDS access of any kind); the kernel waits for them itself.
-typedef int BufDesc __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ BufDesc make_desc(const void *base)
-{
-    const unsigned long long a = (unsigned long long)base;
-    BufDesc d;
-    d.x = (int)(unsigned)a;
-    d.y = (int)((a >> 32) & 0xffff);
-    d.z = (int)0x80000000u;
-    d.w = 0x00020000;
-    return d;
-}
-
-// lds_addr: LDS byte address the wavefront's 64 dwords start at (wave-uniform)
-__device__ __forceinline__ void load_row_to_lds(BufDesc desc, unsigned lds_addr, int voff, int soff)
-{
-    int keep_m0;
-    asm volatile("s_mov_b32 %0, m0\n\t"
-                 "s_mov_b32 m0, %1\n\t"
-                 "s_nop 0\n\t"
-                 "buffer_load_dword %2, %3, %4 offen lds\n\t"
-                 "s_mov_b32 m0, %0"
-                 : "=&s"(keep_m0)
-                 : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(desc), "s"(soff)
-                 : "memory");
-}
-
-template <int N>
-__device__ __forceinline__ void wait_rows_in_lds()
-{
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-typedef __attribute__((address_space(3))) float LdsFloat;
 
 template <typename T, int L, int NB, bool INC>
 __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
