@@ -16,6 +16,7 @@
 #include "generic.hpp"
 #include "fast.hpp"
 #include "high.hpp"
+#include "wide.hpp"
 #include "fast4.hpp"
 
 namespace {
@@ -155,7 +156,10 @@ constexpr int kFastFwRowsComplex = 2;       // complex64: half as many (LDS and 
 //     twiddle-stationary kernels of fast.hpp (rows longer than 1024 are treated as
 //     independent 1024-element chunks);
 //   * a HIGH pass runs the stages that pair bits 10 and 11 with the streaming kernels of
-//     high.hpp.
+//     high.hpp;
+//   * the forward call alone replaces the LOW / HIGH passes of one block by a single WIDE pass
+//     (wide.hpp) where the factors of a whole block fit the registers: float at n = 2048 and
+//     4096, complex64 at n = 2048.
 // n <= 1024 with one or two blocks is a single LOW pass: each row is read once and written
 // once.  Longer schedules pass the activation through the workspace between launches.
 
@@ -170,6 +174,7 @@ bool span_ok(const int64_t stride[3], int64_t rows, int64_t width, size_t elem)
 struct Pass {
     int t0, t1;     // stage range [t0, t1)
     bool high;
+    bool wide;      // forward only: one whole block of a 2048- or 4096-element row (wide.hpp)
     int L, NB;      // LOW: FastPlan<L, NB, inc> on chunks of 2^L elements
     bool inc;
     int H, NST, PAT;  // HIGH: H high bits, NST stages, bit hb of PAT = high bit paired by stage s
@@ -191,7 +196,7 @@ int stage_bit(const bf_problem *p, int t)
     return inc ? idx : L - 1 - idx;
 }
 
-PassPlan build_passes(const bf_problem *p, bool base4)
+PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false)
 {
     PassPlan pl;
     const int L = (int)p->log_n;
@@ -209,6 +214,17 @@ PassPlan build_passes(const bf_problem *p, bool base4)
             q.NB = std::min<int>(max_nb, (int)p->nblocks - k);
             q.t0 = k * L;
             q.t1 = (k + q.NB) * L;
+            q.L = L;
+            q.inc = (p->increasing_stride != 0) != ((k & 1) != 0);
+        }
+    } else if (forward_only && (p->dtype == BF_F32 || L == 11)) {
+        for (int k = 0; k < p->nblocks; ++k) {
+            if (pl.npass == 40) return pl;
+            Pass &q = pl.pass[pl.npass++];
+            q = Pass{};
+            q.wide = true;
+            q.t0 = k * L;
+            q.t1 = (k + 1) * L;
             q.L = L;
             q.inc = (p->increasing_stride != 0) != ((k & 1) != 0);
         }
@@ -264,6 +280,19 @@ FastGrid fast_grid(int64_t batch, int Lk, int64_t lanes, int rows_in_flight, int
     return g;
 }
 
+// Row partition of a WIDE pass: one row at a time per workgroup.
+FastGrid wide_grid(int64_t batch, int64_t nstacks)
+{
+    FastGrid g;
+    g.slots = 1;
+    g.ngroups = batch;
+    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU / nstacks);
+    g.nwg = std::min(want, batch);
+    g.groups_per_wg = (batch + g.nwg - 1) / g.nwg;
+    g.nwg = (batch + g.groups_per_wg - 1) / g.groups_per_wg;
+    return g;
+}
+
 // Row partition of a HIGH pass (4 workgroups of 256 low positions per row partition and stack).
 struct HighGrid {
     int64_t nparts, rows_per_wg;
@@ -287,8 +316,9 @@ bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
     for (int k = 0; k < pl.npass; ++k) {
         const Pass &q = pl.pass[k];
         if (q.high) continue;
-        const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, backward ? 1 : fw_rows(p),
-                                     backward ? 1 : kFastFwWgPerCu);
+        const FastGrid g = q.wide ? wide_grid(p->batch, p->nstacks)
+                                  : fast_grid(p->batch, q.L, p->nstacks * pl.chunks, backward ? 1 : fw_rows(p),
+                                              backward ? 1 : kFastFwWgPerCu);
         rows = std::max(rows, (g.groups_per_wg + kFastFwRows + 2) * g.slots);
     }
     const int64_t dense[3] = {p->nstacks * n, n, 1};
@@ -403,6 +433,30 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
             const int rc = p->dtype == BF_C64 ? launch_high<float2>(q, false, a, grid, stream)
                                               : launch_high<float>(q, false, a, grid, stream);
             if (rc) return rc;
+        } else if (q.wide) {
+            const FastGrid g = wide_grid(p->batch, p->nstacks);
+            FastFwArgs a = {};
+            a.tw = tw;
+            a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
+            a.tw_stage_stride = (n / 2) * 4;
+            fill_stage_table(a.tw_stage, kFastMaxStages, q);
+            a.in = src;
+            a.in_view = sv;
+            a.out = dst;
+            a.out_view = dv;
+            a.batch = p->batch;
+            a.ngroups = g.ngroups;
+            a.groups_per_wg = g.groups_per_wg;
+            const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, 1);
+            const dim3 block(kFastThreads);
+            const bool cplx = p->dtype == BF_C64;
+            if (q.L == 12 && q.inc) hipLaunchKernelGGL((wide_fw_kernel<float, 12, true>), grid, block, 0, stream, a);
+            else if (q.L == 12) hipLaunchKernelGGL((wide_fw_kernel<float, 12, false>), grid, block, 0, stream, a);
+            else if (cplx && q.inc) hipLaunchKernelGGL((wide_fw_kernel<float2, 11, true>), grid, block, 0, stream, a);
+            else if (cplx) hipLaunchKernelGGL((wide_fw_kernel<float2, 11, false>), grid, block, 0, stream, a);
+            else if (q.inc) hipLaunchKernelGGL((wide_fw_kernel<float, 11, true>), grid, block, 0, stream, a);
+            else hipLaunchKernelGGL((wide_fw_kernel<float, 11, false>), grid, block, 0, stream, a);
+            BF_HIP_CHECK(hipGetLastError());
         } else {
             const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, fw_rows(p), kFastFwWgPerCu);
             FastFwArgs a = {};
@@ -542,7 +596,7 @@ size_t forward_workspace(const bf_problem *p, bool base4)
         const int64_t n4 = (int64_t)1 << p->log_n;
         return p->nblocks > 1 ? align256((size_t)p->batch * p->nstacks * n4 * 4) : 0;
     }
-    const PassPlan mp = build_passes(p, base4);
+    const PassPlan mp = build_passes(p, base4, true);
     if (!mp.ok || mp.npass <= 1 || !passes_addressable(p, mp, false)) return 0;
     const int64_t n = (int64_t)1 << p->log_n;
     return align256((size_t)p->batch * p->nstacks * n * elem_bytes(p->dtype));
@@ -574,7 +628,7 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
             return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
         return fast4_forward(p, tw4, input, output, workspace, in_view, out_view, 0, (int)p->nblocks, stream);
     }
-    const PassPlan mp = build_passes(p, base4);
+    const PassPlan mp = build_passes(p, base4, true);
     if (mp.ok && passes_addressable(p, mp, false)) {
         const size_t need = forward_workspace(p, base4);
         if (need > 0 && (!workspace || workspace_bytes < need))

@@ -350,9 +350,9 @@ __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, 
 
 // Moves the R values a thread holds (one per row in flight) through LDS: written at word
 // `wr`, read back at word `rd` after a barrier.  Four float rows travel as one 128-bit access.
-// WAIT: the wavefront first waits for the rows it has requested into LDS, so that the barrier
-// also publishes those.
-template <typename T, int R, bool WAIT = false>
+// WAIT: the wavefront first waits for the rows it has requested into LDS (all but the YOUNGER
+// newest memory operations), so that the barrier also publishes those.
+template <typename T, int R, bool WAIT = false, int YOUNGER = 0>
 __device__ __forceinline__ void transpose_rows(T *buf, int wr, int rd, T (&v)[R])
 {
     if constexpr (sizeof(T) == 4 && R % 4 == 0) {
@@ -360,7 +360,7 @@ __device__ __forceinline__ void transpose_rows(T *buf, int wr, int rd, T (&v)[R]
 #pragma unroll
         for (int r = 0; r < R; r += 4)
             b4[(r / 4) * kFastRowWords + wr] = make_float4(v[r], v[r + 1], v[r + 2], v[r + 3]);
-        if constexpr (WAIT) wait_rows_in_lds<0>();
+        if constexpr (WAIT) wait_rows_in_lds<YOUNGER>();
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < R; r += 4) {
@@ -373,7 +373,7 @@ __device__ __forceinline__ void transpose_rows(T *buf, int wr, int rd, T (&v)[R]
     } else {
 #pragma unroll
         for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
-        if constexpr (WAIT) wait_rows_in_lds<0>();
+        if constexpr (WAIT) wait_rows_in_lds<YOUNGER>();
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];

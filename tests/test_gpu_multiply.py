@@ -110,6 +110,14 @@ MULTIPASS_CASES = [
     (10, 2, 12, 3, 4092, 2046, True),
     (10, 2, 12, 3, 2 * 4096 + 7, 4091, False),
     (300, 1, 12, 2, None, None, True),
+    # many rows per workgroup: the row slots in LDS and the transpose buffers go round several times
+    (3000, 1, 10, 2, None, None, False),
+    (3000, 1, 10, 1, None, None, True),
+    (2900, 1, 10, 1, 1000, 1024, False),
+    (9000, 1, 7, 2, 100, 120, True),
+    (1500, 1, 12, 1, None, None, True),
+    (1500, 1, 12, 1, None, None, False),
+    (1300, 2, 11, 2, 2000, 2040, False),
 ]
 
 
@@ -144,6 +152,9 @@ COMPLEX_FAST_CASES = [
     (9, 1, 12, 1, None, None, True),
     (9, 1, 12, 2, None, None, False),
     (5, 2, 12, 3, 4092, 2046, True),
+    (1400, 1, 10, 1, None, None, True),
+    (700, 1, 11, 1, None, None, True),
+    (700, 1, 11, 2, None, None, False),
 ]
 
 
