@@ -343,12 +343,18 @@ void launch_fast_fw_t(bool cplx, const FastFwArgs &a, dim3 grid, hipStream_t str
 }
 
 template <int L, int NB, bool INC>
-void launch_fast_bw_t(bool cplx, const FastBwArgs &a, dim3 grid, hipStream_t stream)
+void launch_fast_bw_t(bool cplx, bool two_rows, const FastBwArgs &a, dim3 grid, hipStream_t stream)
 {
     if constexpr (NB == 1) {
         if (cplx) {
             hipLaunchKernelGGL((fast_bw_kernel<float2, L, NB, INC>), grid, dim3(kFastThreads), 0, stream, a);
             return;
+        }
+        if constexpr (L >= 7) {
+            if (two_rows) {
+                hipLaunchKernelGGL((fast_bw_kernel<float, L, NB, INC, 2>), grid, dim3(kFastThreads), 0, stream, a);
+                return;
+            }
         }
     }
     hipLaunchKernelGGL((fast_bw_kernel<float, L, NB, INC>), grid, dim3(kFastThreads), 0, stream, a);
@@ -913,7 +919,8 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                 a.groups_per_wg = g.groups_per_wg;
                 nparts = g.nwg;
                 const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)mp.chunks);
-                BF_FAST_DISPATCH(launch_fast_bw_t, q, p->dtype == BF_C64, a, grid, stream);
+                // two row groups in flight once a workgroup has enough of them to fill the pipeline
+                BF_FAST_DISPATCH(launch_fast_bw_t, q, p->dtype == BF_C64, g.groups_per_wg >= 16, a, grid, stream);
                 BF_HIP_CHECK(hipGetLastError());
             }
             rc = launch_reduce(p, sc, q.t0, q.t1, nparts, ws + pl.off_partials, pl.slot, d_tw2, d_tw4, stream);

@@ -599,11 +599,35 @@ __device__ __forceinline__ float pair_g(float2 p) { return p.y; }
 __device__ __forceinline__ float2 pair_x(float4 p) { return make_float2(p.x, p.y); }
 __device__ __forceinline__ float2 pair_g(float4 p) { return make_float2(p.z, p.w); }
 
-template <typename T, int L, int NB, bool INC>
+// The R values a thread holds for one walk (one per row group in flight) as one LDS access.
+template <typename T, int R>
+__device__ __forceinline__ void put_rows(T *base, int idx, const T (&v)[R])
+{
+    if constexpr (R == 1) base[idx] = v[0];
+    else reinterpret_cast<float2 *>(base)[idx] = make_float2(v[0], v[1]);
+}
+
+template <typename T, int R>
+__device__ __forceinline__ void get_rows(const T *base, int idx, T (&v)[R])
+{
+    if constexpr (R == 1) {
+        v[0] = base[idx];
+    } else {
+        const float2 p = reinterpret_cast<const float2 *>(base)[idx];
+        v[0] = p.x;
+        v[1] = p.y;
+    }
+}
+
+// R: row groups in flight per walk.  Two are possible where one block of float factors
+// leaves half of the registers free; each barrier and each LDS round trip then serves two
+// rows, and every thread runs four independent dependency chains instead of two.
+template <typename T, int L, int NB, bool INC, int R = 1>
 __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 {
     using P = FastPlan<L, NB, INC>;
     constexpr int W = (int)sizeof(T) / 4;
+    static_assert(R == 1 || (R == 2 && W == 1), "two row groups in flight: float only");
     // float rows are fetched straight into LDS; complex64 has no LDS to spare for that at
     // 9-10 stages and fetches into registers
     constexpr bool DIRECT = W == 1;
@@ -617,13 +641,16 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // slot per thread and stage; complex64 at 9-10 stages also keeps half of the diagonal
     // entries there.
     constexpr bool COL = !(W == 2 && NS >= 9);  // reverse sweep written with the factor column
-    constexpr bool TB_LDS = NS * W > 10;
+    constexpr bool TB_LDS = NS * W * R > 10;
     constexpr int NTA = (W == 2 && NS >= 9) ? NS / 2 : 0;
-    __shared__ Pair lds[Q::K > 0 ? 2 * kFastRowWords : 1];
-    __shared__ T lds_carry[Q::DEFER ? kFastRowWords : 1];
+    // transpose buffers: [parity][walk][rowwords][R]; where both walks move the same way and
+    // R = 1, the two walks share one access as an (x, g) pair: [parity][rowwords] pairs
+    __shared__ __align__(16) T lds[Q::K > 0 ? 4 * R * kFastRowWords : 1];
+    __shared__ __align__(16) T lds_carry[Q::DEFER ? R * kFastRowWords : 1];
     __shared__ T lds_tb[TB_LDS ? NS * kFastThreads : 1];
     __shared__ T lds_ta[NTA > 0 ? NTA * kFastThreads : 1];
-    __shared__ float lds_rows[DIRECT ? 8 * kFastRowWords : 1];  // x slots 0..3, output-gradient slots 4..7
+    // row slots: 4 sets of R for x, then 4 sets of R for the output gradient
+    __shared__ float lds_rows[DIRECT ? 8 * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
@@ -682,67 +709,86 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const int g_dma = col_d < a.g_view.width ? slot_d * g_row + (int)(col_d * a.g_view.se * EB) : kOob;
     const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
     auto group_ok_d = [&](int grp) { return grp >= 0 && grp * SLOTS + slot_d < rows_valid; };
-    // x of group grp -> x slot (grp & 3); output gradient of group grp -> gradient slot (grp & 3).
-    // Rows are requested AHEAD iterations before they are read: one is enough when the wait
-    // for them sits late in the iteration (behind two or more barriers), otherwise two.
+    // Iteration j replays the R groups R j .. R j + R - 1 (they sit in x set j & 3) and sweeps
+    // them one iteration later (output-gradient set j & 3).  Rows are requested AHEAD
+    // iterations before they are read: one is enough when the wait for them sits late in the
+    // iteration (behind two or more barriers), otherwise two.
     constexpr int AHEAD = Q::K >= 2 ? 1 : 2;
-    auto fetch_x = [&](int grp) {
-        load_row_to_lds(x_desc, rows_addr + (grp & 3) * kFastRowWords * 4, group_ok_d(grp) ? x_dma : kOob,
-                        (grp < 0 ? 0 : grp) * SLOTS * x_row);
+    auto fetch_x = [&](int j) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int grp = R * j + r;
+            load_row_to_lds(x_desc, rows_addr + ((j & 3) * R + r) * kFastRowWords * 4,
+                            group_ok_d(grp) ? x_dma : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row);
+        }
     };
-    auto fetch_g = [&](int grp) {
-        load_row_to_lds(g_desc, rows_addr + (4 + (grp & 3)) * kFastRowWords * 4, group_ok_d(grp) ? g_dma : kOob,
-                        (grp < 0 ? 0 : grp) * SLOTS * g_row);
+    auto fetch_g = [&](int j) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int grp = R * j + r;
+            load_row_to_lds(g_desc, rows_addr + ((4 + (j & 3)) * R + r) * kFastRowWords * 4,
+                            group_ok_d(grp) ? g_dma : kOob, (grp < 0 ? 0 : grp) * SLOTS * g_row);
+        }
     };
 
-    // One pipelined iteration: forward replay of group it + 1 into `nxt`, reverse sweep of
-    // group it out of `cur`.  Register flavour: vF / gv enter holding the freshly loaded x and
-    // g.  LDS flavour: they are read from the row slots, and the rows of a later iteration
-    // are requested; the rows of the next iteration must have landed, for every wavefront,
-    // before it starts, so each wavefront waits for its own share of them just before the
-    // last barrier of this iteration.  `carry` holds the previous group's input gradient still in layout B (DEFER
-    // only).  FLIP alternates between the two unrolled calls: it gives the parity of `it` at
-    // compile time and keeps the LDS buffers alternating when the number of phases is odd.
-    auto iteration = [&](auto FLIP, int it, T vF, T gv, T &carry, T (&cur)[NS], T (&nxt)[NS]) {
+    // One pipelined iteration: forward replay of the groups of iteration it + 1 into `nxt`,
+    // reverse sweep of the groups of iteration it out of `cur`.  Register flavour: vF / gv
+    // enter holding the freshly loaded x and g.  LDS flavour: they are read from the row
+    // slots, and the rows of a later iteration are requested; the rows of the next iteration
+    // must have landed, for every wavefront, before it starts, so each wavefront waits for
+    // its own share of them just before the last barrier of this iteration.  `carry` holds
+    // the previous iteration's input gradients still in layout B (DEFER only).  FLIP
+    // alternates between the two unrolled calls and keeps the LDS buffers alternating when
+    // the number of phases is odd.
+    auto iteration = [&](auto FLIP, int it, T (&vF)[R], T (&gv)[R], T (&carry)[R], T (&cur)[R][NS], T (&nxt)[R][NS]) {
         constexpr int flip = decltype(FLIP)::value;
         // Memory operations issued after the requests the wait is for and before the wait: this
-        // iteration's store when it comes first and, if those requests were made one iteration
-        // earlier, that iteration's store and this iteration's two requests.
-        constexpr int YOUNGER = ((Q::DEFER && Q::K > 1) ? 1 : 0) + (AHEAD == 2 ? 3 : 0);
+        // iteration's stores when they come first and, if those requests were made one
+        // iteration earlier, that iteration's stores and this iteration's requests.
+        constexpr int YOUNGER = ((Q::DEFER && Q::K > 1) ? R : 0) + (AHEAD == 2 ? 3 * R : 0);
         if constexpr (DIRECT) {
             fetch_x(it + 1 + AHEAD);
             fetch_g(it + AHEAD);
-            const float xv = lds_rows[((it + 1) & 3) * kFastRowWords + (Q::SF ? c.fB : c.fA)];
-            const float gr = lds_rows[(4 + (it & 3)) * kFastRowWords + (Q::SB ? c.fB : c.fA)];
-            vF = xv;
-            gv = gr;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float xv = lds_rows[(((it + 1) & 3) * R + r) * kFastRowWords + (Q::SF ? c.fB : c.fA)];
+                const float gr = lds_rows[((4 + (it & 3)) * R + r) * kFastRowWords + (Q::SB ? c.fB : c.fA)];
+                vF[r] = xv;
+                gv[r] = gr;
+            }
         }
         static_for<0, Q::K + 1>([&](auto KK) {
             constexpr int k = KK;
             if constexpr (k >= 1) {
                 constexpr bool hasF = k <= Q::nF, hasB = k <= Q::nB;
-                constexpr bool paired = hasF && hasB && Q::flay(k) == Q::blay(k);
-                Pair *buf = lds + ((k + flip * Q::K) & 1) * kFastRowWords;
-                T *bufs = reinterpret_cast<T *>(buf);
+                constexpr bool paired = R == 1 && hasF && hasB && Q::flay(k) == Q::blay(k);
+                T *half = lds + ((k + flip * Q::K) & 1) * 2 * R * kFastRowWords;
+                Pair *buf = reinterpret_cast<Pair *>(half);
+                T *bufF = half, *bufB = half + R * kFastRowWords;
                 const int wrF = Q::flay(k) ? c.fA : c.fB, rdF = Q::flay(k) ? c.fB : c.fA;
                 const int wrB = Q::blay(k) ? c.fA : c.fB, rdB = Q::blay(k) ? c.fB : c.fA;
                 if constexpr (paired) {
-                    buf[wrF] = make_pair(vF, gv);
+                    buf[wrF] = make_pair(vF[0], gv[0]);
                 } else {
-                    if constexpr (hasF) bufs[2 * wrF] = vF;
-                    if constexpr (hasB) bufs[2 * wrB + 1] = gv;
+                    if constexpr (hasF) put_rows<T, R>(bufF, wrF, vF);
+                    if constexpr (hasB) put_rows<T, R>(bufB, wrB, gv);
                 }
-                if constexpr (Q::DEFER && k == 1) lds_carry[c.fB] = carry;
+                if constexpr (Q::DEFER && k == 1) put_rows<T, R>(lds_carry, c.fB, carry);
                 if constexpr (DIRECT && k == Q::K) wait_rows_in_lds<YOUNGER>();
                 __syncthreads();
-                if constexpr (Q::DEFER && k == 1) store_grad(it - 1, lds_carry[c.fA]);
+                if constexpr (Q::DEFER && k == 1) {
+                    T done[R];
+                    get_rows<T, R>(lds_carry, c.fA, done);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) store_grad(R * (it - 1) + r, done[r]);
+                }
                 if constexpr (paired) {
                     const Pair v2 = buf[rdF];
-                    vF = pair_x(v2);
-                    gv = pair_g(v2);
+                    vF[0] = pair_x(v2);
+                    gv[0] = pair_g(v2);
                 } else {
-                    if constexpr (hasF) vF = bufs[2 * rdF];
-                    if constexpr (hasB) gv = bufs[2 * rdB + 1];
+                    if constexpr (hasF) get_rows<T, R>(bufF, rdF, vF);
+                    if constexpr (hasB) get_rows<T, R>(bufB, rdB, gv);
                 }
             }
             constexpr int cf = Q::f_count(k), cb = Q::b_count(k);
@@ -752,37 +798,50 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 if constexpr (j < cb) {
                     // reverse stage: uses the gradient before it passes through the stage
                     constexpr int s = b0 - j;
-                    if constexpr (COL)
-                        bw_products<P::kind(s)>(acc_self[s], acc_cross[s], gv, cur[s],
-                                                ta_of(std::integral_constant<int, s>{}), tc[s], c.bperm_addr);
-                    else
-                        bw_products_row<P::kind(s)>(acc_self[s], acc_cross[s], gv, cur[s],
-                                                    ta_of(std::integral_constant<int, s>{}),
-                                                    tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        if constexpr (COL)
+                            bw_products<P::kind(s)>(acc_self[s], acc_cross[s], gv[r], cur[r][s],
+                                                    ta_of(std::integral_constant<int, s>{}), tc[s], c.bperm_addr);
+                        else
+                            bw_products_row<P::kind(s)>(acc_self[s], acc_cross[s], gv[r], cur[r][s],
+                                                        ta_of(std::integral_constant<int, s>{}),
+                                                        tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
+                    }
                 }
                 if constexpr (j < cf) {
                     constexpr int s = f0 + j;
-                    nxt[s] = vF;
-                    if constexpr (s + 1 < NS)
-                        vF = fw_product<P::kind(s)>(vF, ta_of(std::integral_constant<int, s>{}),
-                                                    tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        nxt[r][s] = vF[r];
+                        if constexpr (s + 1 < NS)
+                            vF[r] = fw_product<P::kind(s)>(vF[r], ta_of(std::integral_constant<int, s>{}),
+                                                           tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
+                    }
                 }
             });
         });
-        if constexpr (DIRECT && Q::K == 0) wait_rows_in_lds<3>();
-        if constexpr (Q::DEFER) carry = gv;
-        else store_grad(it, gv);
+        if constexpr (DIRECT && Q::K == 0) wait_rows_in_lds<3 * R>();
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if constexpr (Q::DEFER) carry[r] = gv[r];
+            else store_grad(R * it + r, gv[r]);
+        }
     };
 
-    T actP[NS], actQ[NS];
-    static_for<0, NS>([&](auto S) { actP[S] = zero_of(T()); });
-    // iteration it pairs group it + 1 (forward) with group it (reverse); it = -1 .. ng - 1
-    T carry = zero_of(T());
-    // with a deferred closing transpose one more (empty) iteration flushes the last group
-    const int it_end = Q::DEFER ? ng + 1 : ng;
+    T actP[R][NS], actQ[R][NS];
+#pragma unroll
+    for (int r = 0; r < R; ++r) static_for<0, NS>([&](auto S) { actP[r][S] = zero_of(T()); });
+    // iteration it replays the groups of iteration it + 1 and sweeps its own; it = -1 .. nit - 1
+    T carry[R], vF[R], gv[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) carry[r] = vF[r] = gv[r] = zero_of(T());
+    const int nit = (ng + R - 1) / R;
+    // with a deferred closing transpose one more (empty) iteration flushes the last groups
+    const int it_end = Q::DEFER ? nit + 1 : nit;
     if constexpr (DIRECT) {
         fetch_x(0);
-        fetch_g(-1);  // nothing to sweep yet: a row of zeros
+        fetch_g(-1);  // nothing to sweep yet: rows of zeros
         if constexpr (AHEAD == 2) {
             fetch_x(1);
             fetch_g(0);
@@ -790,8 +849,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         wait_rows_in_lds<0>();
         __syncthreads();
         for (int it = -1; it < it_end; it += 2) {
-            iteration(std::integral_constant<int, 0>{}, it, zero_of(T()), zero_of(T()), carry, actP, actQ);
-            iteration(std::integral_constant<int, 1>{}, it + 1, zero_of(T()), zero_of(T()), carry, actQ, actP);
+            iteration(std::integral_constant<int, 0>{}, it, vF, gv, carry, actP, actQ);
+            iteration(std::integral_constant<int, 1>{}, it + 1, vF, gv, carry, actQ, actP);
         }
         wait_rows_in_lds<0>();  // requests past the last group (they fetch nothing)
     } else {
@@ -799,12 +858,15 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         // held across a whole iteration would not fit
         T x0 = load_x(0), gm = load_g(-1);
         for (int it = -1; it < it_end; it += 2) {
-            const T xa = x0, ga = gm;
+            vF[0] = x0;
+            gv[0] = gm;
             const T x1 = load_x(it + 2), gp = load_g(it + 1);
-            iteration(std::integral_constant<int, 0>{}, it, xa, ga, carry, actP, actQ);
+            iteration(std::integral_constant<int, 0>{}, it, vF, gv, carry, actP, actQ);
             x0 = load_x(it + 3);
             gm = load_g(it + 2);
-            iteration(std::integral_constant<int, 1>{}, it + 1, x1, gp, carry, actQ, actP);
+            vF[0] = x1;
+            gv[0] = gp;
+            iteration(std::integral_constant<int, 1>{}, it + 1, vF, gv, carry, actQ, actP);
         }
     }
 

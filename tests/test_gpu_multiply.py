@@ -112,8 +112,9 @@ MULTIPASS_CASES = [
     (300, 1, 12, 2, None, None, True),
     # many rows per workgroup: the row slots in LDS and the transpose buffers go round several times
     (3000, 1, 10, 2, None, None, False),
-    (3000, 1, 10, 1, None, None, True),
-    (2900, 1, 10, 1, 1000, 1024, False),
+    (5000, 1, 10, 1, None, None, True),
+    (4500, 1, 10, 1, 1000, 1024, False),
+    (4400, 2, 8, 1, None, 200, True),
     (9000, 1, 7, 2, 100, 120, True),
     (1500, 1, 12, 1, None, None, True),
     (1500, 1, 12, 1, None, None, False),
