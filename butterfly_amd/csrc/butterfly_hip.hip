@@ -315,7 +315,11 @@ bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
     int64_t rows = 0;
     for (int k = 0; k < pl.npass; ++k) {
         const Pass &q = pl.pass[k];
-        if (q.high) continue;
+        if (q.high) {
+            // the backward high-bit kernel forms 32-bit offsets from its workgroup's first row
+            if (backward) rows = std::max(rows, high_grid(p->batch, p->nstacks).rows_per_wg + kHighAhead + 1);
+            continue;
+        }
         const FastGrid g = q.wide ? wide_grid(p->batch, p->nstacks)
                                   : fast_grid(p->batch, q.L, p->nstacks * pl.chunks, backward ? 1 : fw_rows(p),
                                               backward ? 1 : kFastFwWgPerCu);
@@ -381,9 +385,12 @@ void launch_fast_bw_t(bool cplx, bool two_rows, const FastBwArgs &a, dim3 grid, 
 template <typename T, int H, int NST, int PAT>
 void launch_high_t(bool backward, const HighArgs &a, dim3 grid, hipStream_t stream)
 {
-    if (backward)
-        hipLaunchKernelGGL((high_bw_kernel<T, H, NST, PAT>), grid, dim3(kHighThreads), 0, stream, a);
-    else
+    if (backward) {
+        // float leaves room for 1024 threads (128 registers each), complex64 for 512
+        constexpr int THREADS = sizeof(T) == 4 ? 1024 : 512;
+        grid.z = 1024 / THREADS;
+        hipLaunchKernelGGL((high_bw_kernel<T, H, NST, PAT, THREADS>), grid, dim3(THREADS), 0, stream, a);
+    } else
         hipLaunchKernelGGL((high_fw_kernel<T, H, NST, PAT>), grid, dim3(kHighThreads), 0, stream, a);
 }
 

@@ -124,12 +124,29 @@ __global__ __launch_bounds__(kHighThreads) void high_fw_kernel(HighArgs a)
 // d_twiddle sums stay in registers across all rows of the workgroup and are written once
 // into the partial slice of this row partition (workgroups with different blockIdx.z own
 // different pair indices of the same slice).
-template <typename T, int H, int NST, int PAT>
-__global__ __launch_bounds__(kHighThreads) void high_bw_kernel(HighArgs a)
+//
+// The factors and sums leave room for three wavefronts per SIMD only, too few to keep HBM
+// busy with register prefetch, so rows are fetched straight into LDS (load_row_to_lds in
+// fast.hpp) kHighAhead rows ahead: a lane reads back exactly the dwords it fetched itself, so
+// no barrier is involved, only the wait for the wavefront's own requests.  All operands are
+// addressed with 32-bit offsets from the workgroup's first row (the host checks the span).
+// THREADS low positions per workgroup (gridDim.z = 1024 / THREADS): as many as the registers
+// allow, so that a workgroup touches long contiguous pieces of every quarter-row.
+constexpr int kHighAhead = 3;   // rows requested ahead; kHighAhead + 1 row slots in LDS
+
+template <typename T, int H, int NST, int PAT, int THREADS>
+__global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
 {
     using TW = HighTwiddle<T, H, NST, PAT>;
     constexpr int E = 1 << H;
-    const int p = blockIdx.z * kHighThreads + threadIdx.x;
+    constexpr int W = (int)sizeof(T) / 4;  // dwords per scalar: the planes of a complex row are fetched separately
+    constexpr int EB = (int)sizeof(T);
+    // complex64 rows would have to be fetched as two strided 32-bit planes, which measured
+    // slower than plain register prefetch: float only
+    constexpr bool DIRECT = W == 1;
+    constexpr int SLOT = 2 * E * W * THREADS;  // dwords per row slot: x and g, E elements, W planes
+    __shared__ float rows[DIRECT ? (kHighAhead + 1) * SLOT : 1];
+    const int p = blockIdx.z * THREADS + threadIdx.x;
     const int stack = blockIdx.y;
     TW tw;
     tw.load(a, stack, p);
@@ -143,28 +160,88 @@ __global__ __launch_bounds__(kHighThreads) void high_bw_kernel(HighArgs a)
 
     const int64_t r0 = (int64_t)blockIdx.x * a.rows_per_wg;
     const int64_t r1 = r0 + a.rows_per_wg < a.batch ? r0 + a.rows_per_wg : a.batch;
-    const T *xin = reinterpret_cast<const T *>(a.x_in) + stack * a.x_view.ss;
-    const T *gout = reinterpret_cast<const T *>(a.g_out) + stack * a.g_view.ss;
-    T *gin = reinterpret_cast<T *>(a.g_in) + stack * a.gi_view.ss;
-
-    auto load_row = [&](int64_t row, T (&x)[E], T (&g)[E]) {
+    const int nr = (int)(r1 - r0);
+    const BufDesc x_desc = make_desc(reinterpret_cast<const T *>(a.x_in) + stack * a.x_view.ss + r0 * a.x_view.sb);
+    const BufDesc g_desc = make_desc(reinterpret_cast<const T *>(a.g_out) + stack * a.g_view.ss + r0 * a.g_view.sb);
+    const __amdgpu_buffer_rsrc_t gi_rs =
+        make_rsrc(reinterpret_cast<T *>(a.g_in) + stack * a.gi_view.ss + r0 * a.gi_view.sb);
+    const int x_row = (int)(a.x_view.sb * EB), g_row = (int)(a.g_view.sb * EB), gi_row = (int)(a.gi_view.sb * EB);
+    int x_off[E], g_off[E], gi_off[E];
+#pragma unroll
+    for (int j = 0; j < E; ++j) {
+        const int col = (j << kHighLowBits) | p;
+        x_off[j] = col < a.x_view.width ? (int)(col * a.x_view.se * EB) : kOob;
+        g_off[j] = col < a.g_view.width ? (int)(col * a.g_view.se * EB) : kOob;
+        gi_off[j] = col < a.gi_view.width ? (int)(col * a.gi_view.se * EB) : kOob;
+    }
+    // slot layout, in dwords: [x | g][element j][plane][thread]; a wavefront's 64 lanes are contiguous
+    const unsigned wave_addr =
+        (unsigned)(unsigned long long)(LdsFloat *)rows + (unsigned)(threadIdx.x & ~63) * 4;
+    auto fetch_row = [&](int row) {  // row relative to r0
+        const unsigned slot_addr = wave_addr + (unsigned)(row & kHighAhead) * SLOT * 4;
 #pragma unroll
         for (int j = 0; j < E; ++j) {
-            const int col = (j << kHighLowBits) | p;
-            x[j] = (row < r1 && col < a.x_view.width) ? xin[row * a.x_view.sb + col * a.x_view.se] : zero_of(T());
-            g[j] = (row < r1 && col < a.g_view.width) ? gout[row * a.g_view.sb + col * a.g_view.se] : zero_of(T());
+#pragma unroll
+            for (int w = 0; w < W; ++w) {
+                load_row_to_lds(x_desc, slot_addr + ((0 * E + j) * W + w) * THREADS * 4,
+                                row < nr && x_off[j] != kOob ? x_off[j] + 4 * w : kOob, row * x_row);
+                load_row_to_lds(g_desc, slot_addr + ((1 * E + j) * W + w) * THREADS * 4,
+                                row < nr && g_off[j] != kOob ? g_off[j] + 4 * w : kOob, row * g_row);
+            }
+        }
+    };
+    auto read_row = [&](int row, int which, int j) -> T {
+        const float *src = rows + (row & kHighAhead) * SLOT + (which * E + j) * W * THREADS + threadIdx.x;
+        if constexpr (W == 1) return src[0];
+        else return make_float2(src[0], src[THREADS]);
+    };
+    static_assert((kHighAhead & (kHighAhead + 1)) == 0, "row slots are indexed with a mask");
+    // memory operations issued after the requests of a row and before that row is read: the
+    // requests of the kHighAhead following rows and the stores of the kHighAhead rows before it
+    constexpr int YOUNGER = kHighAhead * (2 * E * W + E);
+    static_assert(YOUNGER <= 63, "the wait counter holds 6 bits");
+
+    // register flavour: one row ahead
+    const __amdgpu_buffer_rsrc_t x_rs = make_rsrc(reinterpret_cast<const T *>(a.x_in) + stack * a.x_view.ss + r0 * a.x_view.sb);
+    const __amdgpu_buffer_rsrc_t g_rs = make_rsrc(reinterpret_cast<const T *>(a.g_out) + stack * a.g_view.ss + r0 * a.g_view.sb);
+    auto load_row = [&](int row, T (&x)[E], T (&g)[E]) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            x[j] = buf_load<T>(x_rs, row < nr ? x_off[j] : kOob, row * x_row);
+            g[j] = buf_load<T>(g_rs, row < nr ? g_off[j] : kOob, row * g_row);
         }
     };
     T nx[E], ng[E];
-    load_row(r0, nx, ng);
-    for (int64_t row = r0; row < r1; ++row) {
-        T act[NST][E], g[E];
+    if constexpr (DIRECT) {
 #pragma unroll
-        for (int j = 0; j < E; ++j) {
-            act[0][j] = nx[j];
-            g[j] = ng[j];
+        for (int r = 0; r < kHighAhead; ++r) {
+            fetch_row(r);
+            // stores that the range check discards: every row then sees the same number of
+            // younger operations, the first ones included
+#pragma unroll
+            for (int j = 0; j < E; ++j) buf_store(gi_rs, kOob, 0, zero_of(T()));
         }
-        load_row(row + 1, nx, ng);
+    } else {
+        load_row(0, nx, ng);
+    }
+    for (int row = 0; row < nr; ++row) {
+        T act[NST][E], g[E];
+        if constexpr (DIRECT) {
+            fetch_row(row + kHighAhead);
+            wait_rows_in_lds<YOUNGER>();
+#pragma unroll
+            for (int j = 0; j < E; ++j) {
+                act[0][j] = read_row(row, 0, j);
+                g[j] = read_row(row, 1, j);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < E; ++j) {
+                act[0][j] = nx[j];
+                g[j] = ng[j];
+            }
+            load_row(row + 1, nx, ng);
+        }
         static_for<0, NST - 1>([&](auto S) {
             constexpr int s = S;
             constexpr int hb = high_bit_of<PAT>(s);
@@ -193,11 +270,9 @@ __global__ __launch_bounds__(kHighThreads) void high_bw_kernel(HighArgs a)
             });
         });
 #pragma unroll
-        for (int j = 0; j < E; ++j) {
-            const int col = (j << kHighLowBits) | p;
-            if (col < a.gi_view.width) gin[row * a.gi_view.sb + col * a.gi_view.se] = g[j];
-        }
+        for (int j = 0; j < E; ++j) buf_store(gi_rs, gi_off[j], row * gi_row, g[j]);
     }
+    if constexpr (DIRECT) wait_rows_in_lds<0>();  // requests past the last row (they fetch nothing)
 
     T *part = reinterpret_cast<T *>(a.partial) + ((int64_t)blockIdx.x * gridDim.y + stack) * NST * a.partial_slot;
     static_for<0, NST>([&](auto S) {
