@@ -56,6 +56,17 @@ CONFIGS = {
                  metric="butterfly_multiply fwd+bwd GB/s (op level), batch 32768 n=4096 fp32 nblocks 2",
                  workload="cfg5 (op level): butterfly_multiply fw+bw of Butterfly(4096, 4096, nblocks=2), input "
                           "(32768,1,4096) fp32 N(0,1), ortho twiddle (1,2,12,2048,2,2), increasing_stride=True"),
+    "cfg5m": dict(batch=32768, nstacks=1, log_n=12, nblocks=2, inc=True, cplx=False, base4=False, bw=True,
+                  cpu_batch=1024, module="fused",
+                  metric="Butterfly(4096,4096,bias) module fwd+bwd GB/s, batch 32768 fp32 nblocks 2",
+                  workload="cfg5 (module level): Butterfly(4096, 4096, bias=True, init='ortho', nblocks=2) forward + "
+                           "autograd backward (d_input, d_twiddle, d_bias), input (32768,4096) fp32 N(0,1); bias "
+                           "added by the kernel that writes the output, d_bias by the library's column sum"),
+    "cfg5m-sep": dict(batch=32768, nstacks=1, log_n=12, nblocks=2, inc=True, cplx=False, base4=False, bw=True,
+                      cpu_batch=1024, module="separate",
+                      metric="Butterfly(4096,4096,bias) module fwd+bwd GB/s, bias as separate PyTorch ops",
+                      workload="cfg5 (module level, unfused): the same layer computed as butterfly_multiply followed "
+                               "by a PyTorch `+ bias`, autograd backward; for comparison with cfg5m"),
 }
 
 
@@ -156,7 +167,7 @@ def main():
     c = CONFIGS[args.config]
 
     import torch
-    import butterfly_amd  # noqa: F401
+    import butterfly_amd
     ops = torch.ops.torch_butterfly
     assert torch.cuda.is_available(), "bench.py needs a HIP device"
     torch.manual_seed(0)
@@ -164,7 +175,24 @@ def main():
     tws, x, grad = make_operands(c, torch, dev)
     inc = c["inc"]
 
-    if c["base4"]:
+    if c.get("module"):
+        # module level: the layer's forward, then autograd for all three gradients
+        layer = butterfly_amd.Butterfly(1 << c["log_n"], 1 << c["log_n"], bias=True, init="ortho",
+                                        nblocks=c["nblocks"]).to(dev)
+        xm = x.reshape(c["batch"], -1).requires_grad_()
+        gm = grad.reshape(c["batch"], -1)
+        state = {}
+        if c["module"] == "fused":
+            def fw_call():
+                state["y"] = layer(xm)
+        else:
+            from butterfly_amd.multiply import butterfly_multiply
+
+            def fw_call():
+                z = butterfly_multiply(layer.twiddle, layer.pre_process(xm), layer.increasing_stride, layer.out_size)
+                state["y"] = z.reshape(c["batch"], -1) + layer.bias
+        bw_call = lambda: torch.autograd.grad(state["y"], (xm, layer.twiddle, layer.bias), gm)
+    elif c["base4"]:
         fw_call = lambda: ops.butterfly_multiply_base4_fw(tws[0], tws[1], x, inc, None)
         bw_call = lambda: ops.butterfly_multiply_base4_bw(tws[0], tws[1], x, grad, inc)
     else:

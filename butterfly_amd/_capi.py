@@ -17,6 +17,8 @@ SYMBOLS = [
     "bf_version", "bf_hip_version", "bf_last_error",
     "bf_butterfly_multiply_fw", "bf_butterfly_multiply_fw_workspace_bytes",
     "bf_butterfly_multiply_bw_workspace_bytes", "bf_butterfly_multiply_bw",
+    "bf_butterfly_multiply_bias_fw", "bf_butterfly_bias_grad", "bf_butterfly_bias_grad_workspace_bytes",
+    "bf_butterfly_multiply_bias_bw", "bf_butterfly_multiply_bias_bw_workspace_bytes",
     "bf_butterfly_multiply_base4_fw", "bf_butterfly_multiply_base4_fw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw",
@@ -59,6 +61,13 @@ def lib():
         L.bf_butterfly_multiply_bw_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_bw_workspace_bytes.restype = sz
         L.bf_butterfly_multiply_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_bias_fw.argtypes = [pp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_bias_grad.argtypes = [pp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_bias_grad_workspace_bytes.argtypes = [pp]
+        L.bf_butterfly_bias_grad_workspace_bytes.restype = sz
+        L.bf_butterfly_multiply_bias_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_bias_bw_workspace_bytes.argtypes = [pp]
+        L.bf_butterfly_multiply_bias_bw_workspace_bytes.restype = sz
         L.bf_butterfly_multiply_base4_fw.argtypes = [pp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_base4_fw_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_base4_fw_workspace_bytes.restype = sz
@@ -125,6 +134,58 @@ def multiply_fw(twiddle, input, increasing_stride, output_size=None):
     _check(lib().bf_butterfly_multiply_fw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(out), _ptr(ws), nbytes,
                                           _stream()))
     return out
+
+
+def multiply_bias_fw(twiddle, input, bias, increasing_stride, output_size=None):
+    """Forward with the bias (S, output_size) added by the library."""
+    assert twiddle.is_contiguous() and twiddle.is_cuda and input.is_cuda
+    nb, log_n = twiddle.shape[1], twiddle.shape[2]
+    n = 1 << log_n
+    O = n if output_size is None else output_size
+    assert bias.is_contiguous() and tuple(bias.shape) == (input.shape[1], O) and bias.dtype == input.dtype
+    p = make_problem(input, log_n, nb, increasing_stride, O)
+    out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
+    p.output_stride = _strides(out)
+    nbytes = lib().bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_bias_fw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(bias), _ptr(out),
+                                               _ptr(ws), nbytes, _stream()))
+    return out
+
+
+def bias_grad(grad):
+    """Column sums of grad (B, S, O) over the batch, (S, O)."""
+    assert grad.is_cuda and grad.dim() == 3
+    p = Problem()
+    p.dtype = _dtype_code(grad)
+    p.batch, p.nstacks, p.output_size = grad.shape
+    p.input_size = grad.shape[2]
+    p.log_n = max(1, (int(grad.shape[2]) - 1).bit_length())
+    p.nblocks = 1
+    p.output_stride = _strides(grad)
+    d_bias = torch.empty(grad.shape[1], grad.shape[2], dtype=grad.dtype, device=grad.device)
+    nbytes = lib().bf_butterfly_bias_grad_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=grad.device)
+    _check(lib().bf_butterfly_bias_grad(ctypes.byref(p), _ptr(grad), _ptr(d_bias), _ptr(ws), nbytes, _stream()))
+    return d_bias
+
+
+def multiply_bias_bw(twiddle, input, grad, increasing_stride):
+    """Backward that also returns d_bias (S, O).  Returns (d_twiddle, d_input, d_bias)."""
+    assert twiddle.is_contiguous() and twiddle.is_cuda and input.is_cuda and grad.is_cuda
+    nb, log_n = twiddle.shape[1], twiddle.shape[2]
+    p = make_problem(input, log_n, nb, increasing_stride, grad.shape[2])
+    p.output_stride = _strides(grad)
+    d_twiddle = torch.empty_like(twiddle)
+    d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
+    d_bias = torch.empty(grad.shape[1], grad.shape[2], dtype=grad.dtype, device=grad.device)
+    p.d_input_stride = _strides(d_input)
+    nbytes = lib().bf_butterfly_multiply_bias_bw_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_bias_bw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
+                                               _ptr(d_twiddle), _ptr(d_input), _ptr(d_bias), _ptr(ws), nbytes,
+                                               _stream()))
+    return d_twiddle, d_input, d_bias
 
 
 def multiply_bw(twiddle, input, grad, increasing_stride):

@@ -11,7 +11,7 @@ import torch
 from torch import nn
 
 from .complex_utils import complex_reshape, real_dtype_to_complex
-from .multiply import butterfly_multiply
+from .multiply import butterfly_multiply, butterfly_multiply_bias
 
 _INITS = ("empty", "randn", "ortho", "identity", "fft_no_br", "ifft_no_br")
 
@@ -132,23 +132,38 @@ class Butterfly(nn.Module):
             # (prod of stages)^T: transpose every 2x2 and reverse the stage and block order
             twiddle = twiddle.transpose(-1, -2).flip([1, 2])
             last_inc = self.increasing_stride != ((self.nblocks - 1) % 2 == 1)
-            x = butterfly_multiply(twiddle, x, not last_inc, output_size)
+            inc = not last_inc
         else:
-            x = butterfly_multiply(twiddle, x, self.increasing_stride, output_size)
-        return self.post_process(input, x, out_size=x.size(-1) if subtwiddle else None)
+            inc = self.increasing_stride
+        if self.bias is None:
+            x = butterfly_multiply(twiddle, x, inc, output_size)
+        else:
+            # the kernel that writes the output adds the bias: lay it out as (nstacks, columns)
+            # (post_process keeps the first out_size columns of the flattened stacks; with
+            # subtwiddle, the columns of one stack)
+            cols = output_size if output_size is not None else twiddle.shape[3] * 2
+            total = self.nstacks * cols
+            kept = cols if subtwiddle else self.out_size
+            bias = self.bias[:kept]
+            if bias.shape[0] != kept:
+                raise ValueError("bias is shorter than the output")
+            if kept < total:
+                bias = torch.nn.functional.pad(bias, (0, total - kept))
+            x = butterfly_multiply_bias(twiddle, x, bias.reshape(self.nstacks, cols), inc, output_size)
+        return self.post_process(input, x, out_size=x.size(-1) if subtwiddle else None, add_bias=False)
 
     def pre_process(self, input):
         size = input.size(-1)
         x = complex_reshape(input, -1, size)
         return x.unsqueeze(1).expand(x.shape[0], self.nstacks, size)
 
-    def post_process(self, input, output, out_size=None):
+    def post_process(self, input, output, out_size=None, add_bias=True):
         out_size = self.out_size if out_size is None else out_size
         batch = output.shape[0]
         flat = output.reshape(batch, self.nstacks * output.size(-1))
         if flat.shape[-1] != out_size:
             flat = flat[:, :out_size]
-        if self.bias is not None:
+        if self.bias is not None and add_bias:
             flat = flat + self.bias[:out_size]
         return flat.reshape(*input.shape[:-1], out_size)
 

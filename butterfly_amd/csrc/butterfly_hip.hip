@@ -18,6 +18,7 @@
 #include "high.hpp"
 #include "wide.hpp"
 #include "fast4.hpp"
+#include "bias.hpp"
 
 namespace {
 
@@ -417,10 +418,13 @@ void fill_stage_table(int *dst, int cap, const Pass &q)
 
 // Forward through the pass plan.  `scratch` holds one dense (B, S, n) activation when there
 // is more than one pass (passes run in place on it).
+// `bias` (may be NULL) is added by the last pass when that pass runs in a kernel that can do
+// it; *bias_done says whether it was.
 int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, const void *input, void *output,
                       void *scratch, const View &in_view, const View &out_view, int first, int last,
-                      hipStream_t stream)
+                      hipStream_t stream, const void *bias = nullptr, bool *bias_done = nullptr)
 {
+    if (bias_done) *bias_done = false;
     const int64_t n = (int64_t)1 << p->log_n;
     const View dense = dense_view(p->nstacks, n);
     for (int k = first; k < last; ++k) {
@@ -460,6 +464,10 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
             a.batch = p->batch;
             a.ngroups = g.ngroups;
             a.groups_per_wg = g.groups_per_wg;
+            if (k == last - 1 && bias) {
+                a.bias = bias;
+                if (bias_done) *bias_done = true;
+            }
             const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, 1);
             const dim3 block(kFastThreads);
             const bool cplx = p->dtype == BF_C64;
@@ -484,6 +492,10 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
             a.batch = p->batch;
             a.ngroups = g.ngroups;
             a.groups_per_wg = g.groups_per_wg;
+            if (k == last - 1 && bias) {
+                a.bias = bias;
+                if (bias_done) *bias_done = true;
+            }
             const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)pl.chunks);
             BF_FAST_DISPATCH(launch_fast_fw_t, q, p->dtype == BF_C64, a, grid, stream);
             BF_HIP_CHECK(hipGetLastError());
@@ -615,8 +627,30 @@ size_t forward_workspace(const bf_problem *p, bool base4)
     return align256((size_t)p->batch * p->nstacks * n * elem_bytes(p->dtype));
 }
 
+// output += bias over all rows, for schedules whose last pass could not add it itself
+template <typename T>
+int launch_bias_add(const bf_problem *p, const void *bias, void *output, const View &out_view, hipStream_t stream)
+{
+    if (p->batch <= 0 || p->nstacks <= 0 || p->output_size <= 0) return BF_OK;
+    BiasArgs a = {};
+    a.bias = bias;
+    a.out = output;
+    a.view = out_view;
+    a.batch = p->batch;
+    a.width = p->output_size;
+    const int64_t cols = (p->output_size + kBiasThreads - 1) / kBiasThreads;
+    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * 8 / (cols * p->nstacks));
+    a.nparts = std::min<int64_t>(std::min<int64_t>(want, p->batch), 65535);
+    a.rows_per_part = (p->batch + a.nparts - 1) / a.nparts;
+    a.nparts = (p->batch + a.rows_per_part - 1) / a.rows_per_part;
+    const dim3 grid((unsigned)cols, (unsigned)p->nstacks, (unsigned)a.nparts);
+    hipLaunchKernelGGL((bias_add_kernel<T>), grid, dim3(kBiasThreads), 0, stream, a);
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
+}
+
 int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, const void *input,
-            void *output, void *workspace, size_t workspace_bytes, void *stream_)
+            void *output, void *workspace, size_t workspace_bytes, void *stream_, const void *bias = nullptr)
 {
     int rc = check_problem(p, false);
     if (rc) return rc;
@@ -639,7 +673,9 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
         const size_t need = forward_workspace(p, base4);
         if (need > 0 && (!workspace || workspace_bytes < need))
             return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-        return fast4_forward(p, tw4, input, output, workspace, in_view, out_view, 0, (int)p->nblocks, stream);
+        rc = fast4_forward(p, tw4, input, output, workspace, in_view, out_view, 0, (int)p->nblocks, stream);
+        if (rc || !bias) return rc;
+        return launch_bias_add<float>(p, bias, output, out_view, stream);
     }
     const PassPlan mp = build_passes(p, base4, true);
     if (mp.ok && passes_addressable(p, mp, false)) {
@@ -648,10 +684,59 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
             return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
         if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
             return fail(BF_ERR_WORKSPACE, "workspace must be 16-byte aligned");
-        return multipass_forward(p, mp, tw2, input, output, workspace, in_view, out_view, 0, mp.npass, stream);
+        bool bias_done = false;
+        rc = multipass_forward(p, mp, tw2, input, output, workspace, in_view, out_view, 0, mp.npass, stream, bias,
+                               &bias_done);
+        if (rc || !bias || bias_done) return rc;
+        return p->dtype == BF_C64 ? launch_bias_add<float2>(p, bias, output, out_view, stream)
+                                  : launch_bias_add<float>(p, bias, output, out_view, stream);
     }
-    return launch_generic_fw(p, sc, 0, sc.per * sc.nblocks, tw2, tw4, input, in_view, output,
-                             out_view, stream);
+    rc = launch_generic_fw(p, sc, 0, sc.per * sc.nblocks, tw2, tw4, input, in_view, output, out_view, stream);
+    if (rc || !bias) return rc;
+    return p->dtype == BF_C64 ? launch_bias_add<float2>(p, bias, output, out_view, stream)
+                              : launch_bias_add<float>(p, bias, output, out_view, stream);
+}
+
+// ---- bias gradient ------------------------------------------------------------------------------
+
+struct BiasGradPlan {
+    int64_t cols, nparts, rows_per_part;
+    size_t bytes;
+};
+
+BiasGradPlan plan_bias_grad(const bf_problem *p)
+{
+    BiasGradPlan b = {};
+    if (p->batch <= 0 || p->nstacks <= 0 || p->output_size <= 0) return b;
+    b.cols = (p->output_size + kBiasThreads - 1) / kBiasThreads;
+    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * 8 / (b.cols * p->nstacks));
+    b.nparts = std::min<int64_t>(std::min<int64_t>(want, p->batch), 65535);
+    b.rows_per_part = (p->batch + b.nparts - 1) / b.nparts;
+    b.nparts = (p->batch + b.rows_per_part - 1) / b.rows_per_part;
+    b.bytes = align256((size_t)b.nparts * p->nstacks * p->output_size * elem_bytes(p->dtype));
+    return b;
+}
+
+template <typename T>
+int launch_bias_grad(const bf_problem *p, const BiasGradPlan &b, const void *grad, void *d_bias, void *workspace,
+                     hipStream_t stream)
+{
+    BiasArgs a = {};
+    a.grad = grad;
+    a.view = make_view(p->output_stride, p->output_size);
+    a.partial = workspace;
+    a.d_bias = d_bias;
+    a.batch = p->batch;
+    a.width = p->output_size;
+    a.rows_per_part = b.rows_per_part;
+    a.nparts = b.nparts;
+    const dim3 grid1((unsigned)b.cols, (unsigned)p->nstacks, (unsigned)b.nparts);
+    hipLaunchKernelGGL((bias_grad_partial_kernel<T>), grid1, dim3(kBiasThreads), 0, stream, a);
+    BF_HIP_CHECK(hipGetLastError());
+    const dim3 grid2((unsigned)b.cols, (unsigned)p->nstacks, 1);
+    hipLaunchKernelGGL((bias_grad_final_kernel<T>), grid2, dim3(kBiasThreads), 0, stream, a);
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
 }
 
 // ---- generic backward -----------------------------------------------------------------------
@@ -792,10 +877,14 @@ int launch_reduce(const bf_problem *p, const Schedule &sc, int t0, int t1, int64
     return BF_OK;
 }
 
+// bias_partial / bias_nparts: when given, and when the pass that reads `grad` runs in a kernel
+// that can do it, that kernel also leaves the per-workgroup column sums of grad there
+// (*bias_nparts slices of (S, output_size)); *bias_nparts stays 0 otherwise.
 int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, const void *input,
              const void *grad, void *d_tw2, void *d_tw4, void *d_input, void *workspace,
-             size_t workspace_bytes, void *stream_)
+             size_t workspace_bytes, void *stream_, void *bias_partial = nullptr, int64_t *bias_nparts = nullptr)
 {
+    if (bias_nparts) *bias_nparts = 0;
     int rc = check_problem(p, true);
     if (rc) return rc;
     if ((rc = ensure_attributes())) return rc;
@@ -925,6 +1014,11 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                 a.ngroups = g.ngroups;
                 a.groups_per_wg = g.groups_per_wg;
                 nparts = g.nwg;
+                if (k == P - 1 && bias_partial && bias_nparts && q.L == 10 && p->dtype == BF_F32) {
+                    a.bias_partial = bias_partial;
+                    a.bias_width = p->output_size;
+                    *bias_nparts = g.nwg;
+                }
                 const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)mp.chunks);
                 // two row groups in flight once a workgroup has enough of them to fill the pipeline
                 BF_FAST_DISPATCH(launch_fast_bw_t, q, p->dtype == BF_C64, g.groups_per_wg >= 16, a, grid, stream);
@@ -1030,6 +1124,94 @@ size_t bf_butterfly_multiply_base4_fw_workspace_bytes(const bf_problem *p)
 {
     if (check_problem(p, false)) return 0;
     return forward_workspace(p, true);
+}
+
+int bf_butterfly_multiply_bias_fw(const bf_problem *p, const void *twiddle, const void *input, const void *bias,
+                                  void *output, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return forward(p, false, twiddle, nullptr, input, output, workspace, workspace_bytes, stream, bias);
+}
+
+size_t bf_butterfly_bias_grad_workspace_bytes(const bf_problem *p)
+{
+    if (check_problem(p, false)) return 0;
+    return plan_bias_grad(p).bytes;
+}
+
+int bf_butterfly_bias_grad(const bf_problem *p, const void *grad, void *d_bias, void *workspace,
+                           size_t workspace_bytes, void *stream)
+{
+    int rc = check_problem(p, false);
+    if (rc) return rc;
+    if (p->nstacks <= 0 || p->output_size <= 0) return BF_OK;
+    if (!d_bias) return fail(BF_ERR_INVALID, "d_bias is NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (p->batch <= 0) {
+        // an empty batch sums to zero: the final kernel over zero partitions writes exactly that
+        BiasArgs a = {};
+        a.d_bias = d_bias;
+        a.width = p->output_size;
+        const dim3 grid((unsigned)((p->output_size + kBiasThreads - 1) / kBiasThreads), (unsigned)p->nstacks, 1);
+        if (p->dtype == BF_C64) hipLaunchKernelGGL((bias_grad_final_kernel<float2>), grid, dim3(kBiasThreads), 0, s, a);
+        else hipLaunchKernelGGL((bias_grad_final_kernel<float>), grid, dim3(kBiasThreads), 0, s, a);
+        BF_HIP_CHECK(hipGetLastError());
+        return BF_OK;
+    }
+    if (!grad) return fail(BF_ERR_INVALID, "grad is NULL");
+    const BiasGradPlan b = plan_bias_grad(p);
+    if (!workspace || workspace_bytes < b.bytes)
+        return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", b.bytes, workspace_bytes);
+    return p->dtype == BF_C64 ? launch_bias_grad<float2>(p, b, grad, d_bias, workspace, s)
+                              : launch_bias_grad<float>(p, b, grad, d_bias, workspace, s);
+}
+
+// Bias area behind the backward workspace: room for either the per-workgroup column sums the
+// backward kernel leaves (at most one slice per compute unit) or the partitions of the
+// stand-alone column sum.
+static size_t bias_area_bytes(const bf_problem *p)
+{
+    const size_t fused = align256((size_t)kNumCU * std::max<int64_t>(p->nstacks, 1) *
+                                  std::max<int64_t>(p->output_size, 0) * elem_bytes(p->dtype));
+    return std::max(fused, plan_bias_grad(p).bytes);
+}
+
+size_t bf_butterfly_multiply_bias_bw_workspace_bytes(const bf_problem *p)
+{
+    if (check_problem(p, true)) return 0;
+    return align256(plan_bw(p, false).total) + bias_area_bytes(p);
+}
+
+int bf_butterfly_multiply_bias_bw(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
+                                  void *d_twiddle, void *d_input, void *d_bias, void *workspace,
+                                  size_t workspace_bytes, void *stream)
+{
+    int rc = check_problem(p, true);
+    if (rc) return rc;
+    const size_t main_bytes = align256(plan_bw(p, false).total);
+    const size_t need = main_bytes + bias_area_bytes(p);
+    if (!workspace || workspace_bytes < need)
+        return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    if (!d_bias && p->nstacks > 0 && p->output_size > 0) return fail(BF_ERR_INVALID, "d_bias is NULL");
+    char *area = static_cast<char *>(workspace) + main_bytes;
+    int64_t nparts = 0;
+    rc = backward(p, false, twiddle, nullptr, input, grad, d_twiddle, nullptr, d_input, workspace, main_bytes, stream,
+                  area, &nparts);
+    if (rc) return rc;
+    if (p->nstacks <= 0 || p->output_size <= 0) return BF_OK;
+    if (nparts > 0) {
+        // the backward kernel left one slice of column sums per workgroup: add them up in order
+        BiasArgs a = {};
+        a.partial = area;
+        a.d_bias = d_bias;
+        a.width = p->output_size;
+        a.nparts = nparts;
+        const dim3 grid((unsigned)((p->output_size + kBiasThreads - 1) / kBiasThreads), (unsigned)p->nstacks, 1);
+        hipLaunchKernelGGL((bias_grad_final_kernel<float>), grid, dim3(kBiasThreads), 0,
+                           static_cast<hipStream_t>(stream), a);
+        BF_HIP_CHECK(hipGetLastError());
+        return BF_OK;
+    }
+    return bf_butterfly_bias_grad(p, grad, d_bias, area, bias_area_bytes(p), stream);
 }
 
 int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4, const void *twiddle2,

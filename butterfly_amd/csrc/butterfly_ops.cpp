@@ -79,8 +79,9 @@ bf_problem make_problem(const Shapes &s, const Tensor &input, bool increasing_st
 
 // ---- base-2 -----------------------------------------------------------------------------
 
-Tensor butterfly_multiply_fw(const Tensor twiddle, const Tensor input, bool increasing_stride,
-                             c10::optional<int64_t> output_size)
+// Shared body of butterfly_multiply_fw and butterfly_multiply_bias_fw (`bias` undefined = none).
+Tensor multiply_fw_impl(const Tensor &twiddle, const Tensor &input, const Tensor &bias, bool increasing_stride,
+                        c10::optional<int64_t> output_size, const char *who)
 {
     CHECK_DEVICE(twiddle); CHECK_DEVICE(input); CHECK_SAME_DEVICE(twiddle, input);
     CHECK_DIM(twiddle, 6); CHECK_DIM(input, 3);
@@ -90,33 +91,83 @@ Tensor butterfly_multiply_fw(const Tensor twiddle, const Tensor input, bool incr
     s.input_size = input.size(2);
     s.nblocks = twiddle.size(1);
     s.log_n = twiddle.size(2);
-    TORCH_CHECK(s.log_n <= 30, "butterfly_multiply_fw: n must be a power of 2");
+    TORCH_CHECK(s.log_n <= 30, who, ": n must be a power of 2");
     s.n = (int64_t)1 << s.log_n;
     CHECK_SHAPE(twiddle, s.nstacks, s.nblocks, s.log_n, s.n / 2, 2, 2);
     const int64_t output_size_val = output_size.has_value() ? output_size.value() : s.n;
-    TORCH_CHECK(output_size_val <= s.n, "butterfly_multiply_fw: output_size must be <= n");
-    TORCH_CHECK(output_size_val >= 0, "butterfly_multiply_fw: output_size must be >= 0");
-    require_device(input, "butterfly_multiply_fw");
-    TORCH_CHECK(twiddle.scalar_type() == input.scalar_type(),
-                "butterfly_multiply_fw: twiddle and input must have the same dtype");
+    TORCH_CHECK(output_size_val <= s.n, who, ": output_size must be <= n");
+    TORCH_CHECK(output_size_val >= 0, who, ": output_size must be >= 0");
+    require_device(input, who);
+    TORCH_CHECK(twiddle.scalar_type() == input.scalar_type(), who, ": twiddle and input must have the same dtype");
+    Tensor b;
+    if (bias.defined()) {
+        CHECK_DEVICE(bias); CHECK_SAME_DEVICE(bias, input);
+        CHECK_DIM(bias, 2);
+        CHECK_SHAPE(bias, s.nstacks, output_size_val);
+        TORCH_CHECK(bias.scalar_type() == input.scalar_type(), who, ": bias and input must have the same dtype");
+        b = dense(bias);
+    }
 
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const Tensor tw = dense(twiddle);
     const Tensor x = input.resolve_conj();
     Tensor output = at::empty({s.batch, s.nstacks, s.n}, x.options());
     if (output_size_val < s.n) output = output.slice(2, 0, output_size_val);
-    bf_problem p = make_problem(s, x, increasing_stride, output_size_val, "butterfly_multiply_fw");
+    bf_problem p = make_problem(s, x, increasing_stride, output_size_val, who);
     set_strides(p.output_stride, output);
     const size_t ws_bytes = bf_butterfly_multiply_fw_workspace_bytes(&p);
     Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
-    check_rc(bf_butterfly_multiply_fw(&p, tw.data_ptr(), x.data_ptr(), output.data_ptr(), ws.data_ptr(), ws_bytes,
-                                      current_stream()),
-             "butterfly_multiply_fw");
+    check_rc(bf_butterfly_multiply_bias_fw(&p, tw.data_ptr(), x.data_ptr(), b.defined() ? b.data_ptr() : nullptr,
+                                           output.data_ptr(), ws.data_ptr(), ws_bytes, current_stream()),
+             who);
     return output;
 }
 
-std::tuple<Tensor, Tensor> butterfly_multiply_bw(const Tensor twiddle, const Tensor input,
-                                                 const Tensor grad, bool increasing_stride)
+Tensor butterfly_multiply_fw(const Tensor twiddle, const Tensor input, bool increasing_stride,
+                             c10::optional<int64_t> output_size)
+{
+    return multiply_fw_impl(twiddle, input, Tensor(), increasing_stride, output_size, "butterfly_multiply_fw");
+}
+
+// New operators (no counterpart in the reference's op set): the layer bias folded into the
+// multiply, where Butterfly.post_process runs a separate elementwise pass
+// (torch_butterfly/butterfly.py:152-169).  bias: (nstacks, output_size).
+Tensor butterfly_multiply_bias_fw(const Tensor twiddle, const Tensor input, const Tensor bias,
+                                  bool increasing_stride, c10::optional<int64_t> output_size)
+{
+    TORCH_CHECK(bias.defined(), "butterfly_multiply_bias_fw: bias is undefined");
+    return multiply_fw_impl(twiddle, input, bias, increasing_stride, output_size, "butterfly_multiply_bias_fw");
+}
+
+// d_bias (nstacks, output_size) = sum of grad (batch, nstacks, output_size) over the batch.
+Tensor butterfly_bias_grad(const Tensor grad)
+{
+    CHECK_DEVICE(grad);
+    CHECK_DIM(grad, 3);
+    require_device(grad, "butterfly_bias_grad");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
+    const Tensor g = grad.resolve_conj();
+    bf_problem p = {};
+    p.dtype = dtype_code(g, "butterfly_bias_grad");
+    p.batch = g.size(0);
+    p.nstacks = g.size(1);
+    p.output_size = g.size(2);
+    p.input_size = g.size(2);
+    p.nblocks = 1;
+    p.log_n = 1;
+    while (((int64_t)1 << p.log_n) < p.output_size) ++p.log_n;
+    set_strides(p.output_stride, g);
+    Tensor d_bias = at::empty({p.nstacks, p.output_size}, g.options());
+    const size_t ws_bytes = bf_butterfly_bias_grad_workspace_bytes(&p);
+    Tensor ws = at::empty({(int64_t)ws_bytes}, g.options().dtype(at::kByte));
+    check_rc(bf_butterfly_bias_grad(&p, g.data_ptr(), d_bias.data_ptr(), ws.data_ptr(), ws_bytes, current_stream()),
+             "butterfly_bias_grad");
+    return d_bias;
+}
+
+// Shared body of butterfly_multiply_bw and butterfly_multiply_bias_bw.
+std::tuple<Tensor, Tensor, Tensor> multiply_bw_impl(const Tensor &twiddle, const Tensor &input, const Tensor &grad,
+                                                    bool increasing_stride, bool with_bias, const char *who)
 {
     CHECK_DEVICE(twiddle); CHECK_DEVICE(input); CHECK_DEVICE(grad);
     CHECK_SAME_DEVICE(twiddle, input); CHECK_SAME_DEVICE(input, grad);
@@ -127,15 +178,15 @@ std::tuple<Tensor, Tensor> butterfly_multiply_bw(const Tensor twiddle, const Ten
     s.input_size = input.size(2);
     s.nblocks = twiddle.size(1);
     s.log_n = twiddle.size(2);
-    TORCH_CHECK(s.log_n <= 30, "butterfly_multiply_bw: n must be a power of 2");
+    TORCH_CHECK(s.log_n <= 30, who, ": n must be a power of 2");
     s.n = (int64_t)1 << s.log_n;
     const int64_t output_size = grad.size(2);
     CHECK_SHAPE(twiddle, s.nstacks, s.nblocks, s.log_n, s.n / 2, 2, 2);
     CHECK_SHAPE(grad, s.batch, s.nstacks, output_size);
-    TORCH_CHECK(output_size <= s.n, "butterfly_multiply_bw: grad must have at most n columns");
-    require_device(input, "butterfly_multiply_bw");
-    TORCH_CHECK(twiddle.scalar_type() == input.scalar_type() && grad.scalar_type() == input.scalar_type(),
-                "butterfly_multiply_bw: twiddle, input and grad must have the same dtype");
+    TORCH_CHECK(output_size <= s.n, who, ": grad must have at most n columns");
+    require_device(input, who);
+    TORCH_CHECK(twiddle.scalar_type() == input.scalar_type() && grad.scalar_type() == input.scalar_type(), who,
+                ": twiddle, input and grad must have the same dtype");
 
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const Tensor tw = dense(twiddle);
@@ -144,16 +195,40 @@ std::tuple<Tensor, Tensor> butterfly_multiply_bw(const Tensor twiddle, const Ten
     Tensor d_twiddle = at::empty(tw.sizes(), tw.options());
     Tensor d_input = at::empty({s.batch, s.nstacks, std::max(s.input_size, s.n)}, x.options());
     if (s.input_size < s.n) d_input = d_input.slice(2, 0, s.input_size);
-    bf_problem p = make_problem(s, x, increasing_stride, output_size, "butterfly_multiply_bw");
+    bf_problem p = make_problem(s, x, increasing_stride, output_size, who);
     set_strides(p.output_stride, g);
     set_strides(p.d_input_stride, d_input);
-    const size_t ws_bytes = bf_butterfly_multiply_bw_workspace_bytes(&p);
-    Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
-    check_rc(bf_butterfly_multiply_bw(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), d_twiddle.data_ptr(),
-                                      d_input.data_ptr(), ws.data_ptr(), ws_bytes,
-                                      current_stream()),
-             "butterfly_multiply_bw");
-    return std::make_tuple(d_twiddle, d_input);
+    Tensor d_bias;
+    if (with_bias) {
+        d_bias = at::empty({s.nstacks, output_size}, g.options());
+        const size_t ws_bytes = bf_butterfly_multiply_bias_bw_workspace_bytes(&p);
+        Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+        check_rc(bf_butterfly_multiply_bias_bw(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), d_twiddle.data_ptr(),
+                                               d_input.data_ptr(), d_bias.data_ptr(), ws.data_ptr(), ws_bytes,
+                                               current_stream()),
+                 who);
+    } else {
+        const size_t ws_bytes = bf_butterfly_multiply_bw_workspace_bytes(&p);
+        Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+        check_rc(bf_butterfly_multiply_bw(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), d_twiddle.data_ptr(),
+                                          d_input.data_ptr(), ws.data_ptr(), ws_bytes, current_stream()),
+                 who);
+    }
+    return std::make_tuple(d_twiddle, d_input, d_bias);
+}
+
+std::tuple<Tensor, Tensor> butterfly_multiply_bw(const Tensor twiddle, const Tensor input,
+                                                 const Tensor grad, bool increasing_stride)
+{
+    auto r = multiply_bw_impl(twiddle, input, grad, increasing_stride, false, "butterfly_multiply_bw");
+    return std::make_tuple(std::get<0>(r), std::get<1>(r));
+}
+
+// (d_twiddle, d_input, d_bias): the backward of butterfly_multiply_bias_fw
+std::tuple<Tensor, Tensor, Tensor> butterfly_multiply_bias_bw(const Tensor twiddle, const Tensor input,
+                                                              const Tensor grad, bool increasing_stride)
+{
+    return multiply_bw_impl(twiddle, input, grad, increasing_stride, true, "butterfly_multiply_bias_bw");
 }
 
 using torch::autograd::AutogradContext;
@@ -182,6 +257,31 @@ Tensor butterfly_multiply(Tensor twiddle, Tensor input, bool increasing_stride,
                           c10::optional<int64_t> output_size)
 {
     return ButterflyMultiply::apply(twiddle, input, increasing_stride, output_size);
+}
+
+class ButterflyMultiplyBias : public torch::autograd::Function<ButterflyMultiplyBias> {
+public:
+    static Tensor forward(AutogradContext *ctx, Tensor twiddle, Tensor input, Tensor bias, bool increasing_stride,
+                          c10::optional<int64_t> output_size)
+    {
+        ctx->saved_data["increasing_stride"] = increasing_stride;
+        ctx->save_for_backward({twiddle, input});
+        return butterfly_multiply_bias_fw(twiddle, input, bias, increasing_stride, output_size);
+    }
+
+    static variable_list backward(AutogradContext *ctx, variable_list grad_output)
+    {
+        const auto saved = ctx->get_saved_variables();
+        const bool increasing_stride = ctx->saved_data["increasing_stride"].toBool();
+        auto result = butterfly_multiply_bias_bw(saved[0], saved[1], grad_output[0], increasing_stride);
+        return {std::get<0>(result), std::get<1>(result), std::get<2>(result), Tensor(), Tensor()};
+    }
+};
+
+Tensor butterfly_multiply_bias(Tensor twiddle, Tensor input, Tensor bias, bool increasing_stride,
+                               c10::optional<int64_t> output_size)
+{
+    return ButterflyMultiplyBias::apply(twiddle, input, bias, increasing_stride, output_size);
 }
 
 // ---- base-4 -----------------------------------------------------------------------------
@@ -295,6 +395,10 @@ TORCH_LIBRARY(torch_butterfly, m)
     m.def("butterfly_multiply_fw", butterfly_multiply_fw);
     m.def("butterfly_multiply_bw", butterfly_multiply_bw);
     m.def("butterfly_multiply", butterfly_multiply);
+    m.def("butterfly_multiply_bias_fw", butterfly_multiply_bias_fw);
+    m.def("butterfly_bias_grad", butterfly_bias_grad);
+    m.def("butterfly_multiply_bias_bw", butterfly_multiply_bias_bw);
+    m.def("butterfly_multiply_bias", butterfly_multiply_bias);
     m.def("butterfly_multiply_base4_fw", butterfly_multiply_base4_fw);
     m.def("butterfly_multiply_base4_bw", butterfly_multiply_base4_bw);
     m.def("butterfly_multiply_base4", butterfly_multiply_base4);

@@ -321,6 +321,7 @@ struct FastFwArgs {
     int64_t batch;
     int64_t ngroups;           // ceil(batch / SLOTS)
     int64_t groups_per_wg;
+    const void *bias;          // NULL, or (S, out_view.width) dense: added to every output row
 };
 
 // Loads the factor entries each thread needs for every stage: its row (ta, tb) and, for the
@@ -419,6 +420,9 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     // thread-constant part of the offsets; the row group adds a wave-uniform part
     const int in_thr = col < a.in_view.width ? c.slot * in_row + (int)(col * a.in_view.se * EB) : kOob;
     const int out_thr = col < a.out_view.width ? c.slot * out_row + (int)(col * a.out_view.se * EB) : kOob;
+    const T bias = (a.bias && col < a.out_view.width)
+                       ? reinterpret_cast<const T *>(a.bias)[stack * a.out_view.width + col]
+                       : zero_of(T());
 
     auto load_rows = [&](int grel, T (&v)[R]) {
 #pragma unroll
@@ -497,7 +501,7 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
-            buf_store(out_rs, ok ? out_thr : kOob, (grel + r) * SLOTS * out_row, v[r]);
+            buf_store(out_rs, ok ? out_thr : kOob, (grel + r) * SLOTS * out_row, add(v[r], bias));
         }
     }
     if constexpr (DIRECT) wait_rows_in_lds<0>();  // requests past the last group (they fetch nothing)
@@ -519,6 +523,10 @@ struct FastBwArgs {
     int64_t batch;
     int64_t ngroups;
     int64_t groups_per_wg;
+    // float kernels on 1024-element rows or chunks only: when set, the column sums of g_out over
+    // this workgroup's rows (a layer's bias gradient) go to (gridDim.x, S, bias_width)
+    void *bias_partial;
+    int64_t bias_width;
 };
 
 // Backward kernel, software-pipelined over rows: iteration i runs the forward replay of
@@ -651,6 +659,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     __shared__ T lds_ta[NTA > 0 ? NTA * kFastThreads : 1];
     // row slots: 4 sets of R for x, then 4 sets of R for the output gradient
     __shared__ float lds_rows[DIRECT ? 8 * R * kFastRowWords : 1];
+    __shared__ float lds_bias[(DIRECT && SLOTS == 1) ? kFastThreads : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
@@ -714,6 +723,12 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // iterations before they are read: one is enough when the wait for them sits late in the
     // iteration (behind two or more barriers), otherwise two.
     constexpr int AHEAD = Q::K >= 2 ? 1 : 2;
+    // Column sum of the output gradient (see FastBwArgs::bias_partial): the thread adds the
+    // element it reads at the top of every reverse sweep, into a private LDS word (a register
+    // held across the row loop is one too many for the two-block schedules).
+    constexpr bool BIAS_SUM = DIRECT && SLOTS == 1;
+    const bool bias_on = BIAS_SUM && a.bias_partial != nullptr;
+    if constexpr (BIAS_SUM) lds_bias[t] = 0.0f;
     auto fetch_x = [&](int j) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -755,6 +770,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 const float gr = lds_rows[((4 + (it & 3)) * R + r) * kFastRowWords + (Q::SB ? c.fB : c.fA)];
                 vF[r] = xv;
                 gv[r] = gr;
+                if constexpr (BIAS_SUM) {
+                    if (bias_on) lds_bias[t] += gr;
+                }
             }
         }
         static_for<0, Q::K + 1>([&](auto KK) {
@@ -875,6 +893,14 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     int t2 = t;
     asm volatile("" : "+v"(t2));
     const FastCoords c2 = fast_coords<L>(t2);
+    if constexpr (BIAS_SUM) {
+        if (bias_on) {
+            const int64_t bcol = ((int64_t)chunk << L) + (Q::SB ? c2.eB : c2.eA);
+            if (bcol < a.bias_width)
+                reinterpret_cast<float *>(a.bias_partial)[((int64_t)blockIdx.x * gridDim.y + stack) * a.bias_width +
+                                                          bcol] = lds_bias[t2];
+        }
+    }
     // One partial slice per workgroup.  When the workgroup holds several rows at once
     // (n < 1024) the per-row-slot sums are first added through LDS in ascending slot order.
     T *part = reinterpret_cast<T *>(a.partial) + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * a.partial_slot +

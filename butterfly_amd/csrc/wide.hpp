@@ -110,9 +110,13 @@ __global__ __launch_bounds__(kFastThreads) void wide_fw_kernel(FastFwArgs a)
         make_rsrc(reinterpret_cast<T *>(a.out) + r0 * a.out_view.sb + stack * a.out_view.ss);
     const int in_row = (int)(a.in_view.sb * EB), out_row = (int)(a.out_view.sb * EB);
     int in_thr[Q], out_thr[Q], in_dma[Q];
+    T bias[Q];
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
         const int col = (q << 10) | c.eA;
+        bias[q] = (a.bias && col < a.out_view.width)
+                      ? reinterpret_cast<const T *>(a.bias)[stack * a.out_view.width + col]
+                      : zero_of(T());
         in_thr[q] = col < a.in_view.width ? (int)(col * a.in_view.se * EB) : kOob;
         out_thr[q] = col < a.out_view.width ? (int)(col * a.out_view.se * EB) : kOob;
         const int col_d = (q << 10) | t;
@@ -189,7 +193,7 @@ __global__ __launch_bounds__(kFastThreads) void wide_fw_kernel(FastFwArgs a)
             transpose_rows<T, Q, DIRECT, 2 * Q>(buf, c.fB, c.fA, v);
         }
 #pragma unroll
-        for (int q = 0; q < Q; ++q) buf_store(out_rs, row < nr ? out_thr[q] : kOob, row * out_row, v[q]);
+        for (int q = 0; q < Q; ++q) buf_store(out_rs, row < nr ? out_thr[q] : kOob, row * out_row, add(v[q], bias[q]));
     }
     if constexpr (DIRECT) wait_rows_in_lds<0>();  // requests past the last row (they fetch nothing)
 }

@@ -30,6 +30,15 @@ def butterfly_multiply(twiddle: torch.Tensor, input: torch.Tensor, increasing_st
                                                         output_size)
 
 
+def butterfly_multiply_bias(twiddle: torch.Tensor, input: torch.Tensor, bias: torch.Tensor,
+                            increasing_stride: bool, output_size: Optional[int] = None) -> torch.Tensor:
+    """butterfly_multiply(...) + bias with the addition done by the kernel that writes the
+    output; bias (nstacks, output_size or n).  Differentiable in all three tensors.  The
+    reference adds the bias as a separate pass (torch_butterfly/butterfly.py:152-169)."""
+    return torch.ops.torch_butterfly.butterfly_multiply_bias(twiddle, input, bias, increasing_stride,
+                                                             output_size)
+
+
 def fit_last_dim(x: torch.Tensor, n: int) -> torch.Tensor:
     """Zero-pad or trim the last dimension to exactly ``n``."""
     size = x.shape[-1]

@@ -83,6 +83,37 @@ int bf_butterfly_multiply_bw(const bf_problem *p, const void *twiddle, const voi
                              const void *grad, void *d_twiddle, void *d_input,
                              void *workspace, size_t workspace_bytes, void *stream);
 
+/* Forward multiply with the layer bias folded into the last pass:
+ * output[b][s][c] = multiply(...)[b][s][c] + bias[s][c], bias (S, O) dense (NULL = no bias).
+ * Stands where Butterfly.post_process adds the bias as a separate elementwise pass over
+ * the output (torch_butterfly/butterfly.py:152-169).  Workspace as for
+ * bf_butterfly_multiply_fw.                                                            */
+int bf_butterfly_multiply_bias_fw(const bf_problem *p, const void *twiddle, const void *input,
+                                  const void *bias, void *output, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
+/* Bias gradient of such a layer: d_bias[s][c] = sum over b of grad[b][s][c], d_bias (S, O)
+ * dense, fully overwritten; what autograd derives for the `+ bias` of
+ * torch_butterfly/butterfly.py:167-168.  Only batch, nstacks, output_size, dtype and
+ * output_stride (the strides of grad) of the problem are used.  Fixed summation order:
+ * bitwise reproducible.                                                                */
+int bf_butterfly_bias_grad(const bf_problem *p, const void *grad, void *d_bias, void *workspace,
+                           size_t workspace_bytes, void *stream);
+
+size_t bf_butterfly_bias_grad_workspace_bytes(const bf_problem *p);
+
+/* Backward multiply that also returns the bias gradient of the layer: as
+ * bf_butterfly_multiply_bw, plus d_bias (S, O) = sum over b of grad[b][s][c].  Where the
+ * kernel that reads grad can do it (float, rows or chunks of 1024) it forms the column sums
+ * on the way, so grad is not read a second time; otherwise this is
+ * bf_butterfly_multiply_bw followed by bf_butterfly_bias_grad.  No counterpart in the
+ * reference's op set (autograd's sum for torch_butterfly/butterfly.py:167-168).          */
+int bf_butterfly_multiply_bias_bw(const bf_problem *p, const void *twiddle, const void *input,
+                                  const void *grad, void *d_twiddle, void *d_input, void *d_bias,
+                                  void *workspace, size_t workspace_bytes, void *stream);
+
+size_t bf_butterfly_multiply_bias_bw_workspace_bytes(const bf_problem *p);
+
 /* Base-4 forward: per block log_n/2 radix-4 stages from twiddle4
  * (S, nb, log_n/2, n/4, 4, 4), then one 2x2 stage from twiddle2 (S, nb, 1, n/2, 2, 2)
  * when log_n is odd (twiddle2 may be NULL when log_n is even).

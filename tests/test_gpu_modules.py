@@ -47,6 +47,29 @@ def test_butterfly_shapes_and_matrix_flags():
     assert close(b(eye, transpose=True, conjugate=True).t(), M.t().conj(), atol=1e-4)
 
 
+def test_module_bias_matches_separate_addition():
+    """Butterfly folds its bias into the multiply; values and all gradients must equal the
+    reference formulation (multiply, flatten, slice, + bias; torch_butterfly/butterfly.py:152-169)."""
+    import butterfly_amd as bfa
+    from butterfly_amd.multiply import butterfly_multiply
+    torch.manual_seed(3)
+    for in_size, out_size, complex_, nblocks in [(100, 300, False, 2), (64, 40, True, 1), (4096, 4096, False, 2)]:
+        say("module bias", in_size, out_size, complex_, nblocks)
+        b = bfa.Butterfly(in_size, out_size, True, complex_, True, "randn", nblocks).cuda()
+        dtype = torch.complex64 if complex_ else torch.float32
+        x = torch.randn(9, in_size, dtype=dtype, device="cuda", requires_grad=True)
+        g = torch.randn(9, out_size, dtype=dtype, device="cuda")
+        y = b(x)
+        grads = torch.autograd.grad(y, (x, b.twiddle, b.bias), g)
+        out_cols = b.out_size if b.nstacks == 1 else None
+        z = butterfly_multiply(b.twiddle, b.pre_process(x), b.increasing_stride, out_cols)
+        z = z.reshape(9, -1)[:, :out_size] + b.bias
+        ref = torch.autograd.grad(z, (x, b.twiddle, b.bias), g)
+        assert close(y, z, atol=1e-4)
+        for a, r in zip(grads, ref):
+            assert close(a, r, rtol=1e-3, atol=1e-4 * max(1.0, r.abs().max().item()))
+
+
 def test_autograd_through_module_reduces_loss():
     import butterfly_amd as bfa
     torch.manual_seed(0)

@@ -348,3 +348,76 @@ def test_headline_size_properties():
     dtw_ref, _ = oracle.butterfly_bw(tw, x[:1024], g[:1024], False)
     dtw_small, _ = _capi.multiply_bw(twd, xd[:1024], gd[:1024], False)
     assert rel_err(dtw_small.cpu().numpy(), dtw_ref) < BW_TOL
+
+
+BIAS_CASES = [
+    # dtype, B, S, L, nb, I, O, inc -- every kind of last pass: fast (fused), wide (fused),
+    # high-bit and generic (separate add), several stacks, trimmed outputs
+    (np.float32, 37, 2, 5, 2, 20, 27, True),
+    (np.float32, 300, 1, 10, 2, None, None, False),
+    (np.float32, 41, 3, 7, 1, None, 100, True),
+    (np.float32, 19, 1, 11, 2, None, 2000, False),
+    (np.float32, 23, 2, 12, 1, None, None, True),
+    (np.complex64, 29, 2, 6, 3, None, 50, False),
+    (np.complex64, 17, 1, 11, 1, None, None, True),
+    (np.complex64, 9, 1, 12, 1, None, 4000, True),
+    (np.float32, 11, 1, 13, 1, None, 8000, True),
+    (np.float32, 5000, 1, 10, 1, None, 1000, True),
+    (np.float32, 2100, 1, 12, 2, None, 4090, True),
+]
+
+
+@pytest.mark.parametrize("case", BIAS_CASES, ids=lambda c: f"{np.dtype(c[0]).name}-B{c[1]}-S{c[2]}-L{c[3]}-nb{c[4]}-I{c[5]}-O{c[6]}-inc{int(c[7])}")
+def test_bias_folded_into_forward_and_bias_gradient(case):
+    """output = multiply + bias (one rounding of the sum, like the oracle's) and
+    d_bias = column sums of grad, through the C ABI."""
+    from butterfly_amd import _capi
+    dtype, B, S, L, nb, I, O, inc = case
+    say("bias case", case)
+    rng = np.random.default_rng(1700 + L * 19 + nb)
+    tw, x, g = make_case(rng, dtype, B, S, L, nb, I, O)
+    cols = (1 << L) if O is None else O
+    bias = randn(rng, (S, cols), dtype)
+    y_ref = oracle.butterfly_fw(tw, x, inc, O) + bias[None]
+    y = _capi.multiply_bias_fw(dev(tw), dev(x), dev(bias), inc, O)
+    db = _capi.bias_grad(dev(g))
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    db_ref = g.astype(np.complex128 if np.iscomplexobj(g) else np.float64).sum(axis=0)
+    assert rel_err(db.cpu().numpy(), db_ref) < BW_TOL
+    # non-contiguous gradient, run-to-run bitwise equality
+    gt = dev(np.ascontiguousarray(g.transpose(1, 0, 2))).transpose(0, 1)
+    db2 = _capi.bias_grad(gt)
+    db3 = _capi.bias_grad(gt)
+    torch.cuda.synchronize()
+    assert torch.equal(db2, db3) and torch.equal(db2, db)
+    # the backward call that forms d_bias on the way
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+    dtw, dx, db4 = _capi.multiply_bias_bw(dev(tw), dev(x), dev(g), inc)
+    torch.cuda.synchronize()
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+    assert rel_err(db4.cpu().numpy(), db_ref) < BW_TOL
+
+
+def test_bias_operator_autograd():
+    """The autograd operator returns the three gradients the separate formulation gives."""
+    import butterfly_amd  # noqa: F401
+    ops = torch.ops.torch_butterfly
+    torch.manual_seed(5)
+    for dtype, S, L, nb, O in [(torch.float32, 2, 6, 2, 50), (torch.complex64, 1, 5, 1, None),
+                               (torch.float32, 1, 12, 2, None)]:
+        n = 1 << L
+        cols = n if O is None else O
+        tw = (torch.randn(S, nb, L, n // 2, 2, 2, dtype=dtype) / 2 ** 0.5).cuda().requires_grad_()
+        x = torch.randn(21, S, n, dtype=dtype).cuda().requires_grad_()
+        bias = torch.randn(S, cols, dtype=dtype).cuda().requires_grad_()
+        g = torch.randn(21, S, cols, dtype=dtype).cuda()
+        y = ops.butterfly_multiply_bias(tw, x, bias, True, O)
+        d_tw, d_x, d_b = torch.autograd.grad(y, (tw, x, bias), g)
+        y2 = ops.butterfly_multiply(tw, x, True, O) + bias
+        e_tw, e_x, e_b = torch.autograd.grad(y2, (tw, x, bias), g)
+        for a, b in [(y, y2), (d_tw, e_tw), (d_x, e_x), (d_b, e_b)]:
+            assert (a - b).abs().max().item() <= 1e-4 * max(1.0, b.abs().max().item())
+    with pytest.raises(RuntimeError, match="bias must have shape"):
+        ops.butterfly_multiply_bias_fw(tw.detach(), x.detach(), bias.detach()[:, :-1], True, None)
