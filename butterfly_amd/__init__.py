@@ -28,13 +28,15 @@ _load_native()
 
 from .multiply import butterfly_multiply  # noqa: E402
 from .multiply_base4 import butterfly_multiply_base4  # noqa: E402
-from .butterfly import Butterfly  # noqa: E402
+from .butterfly import Butterfly, ButterflyBmm, ButterflyUnitary  # noqa: E402
 from .butterfly_base4 import ButterflyBase4  # noqa: E402
 from . import combine, complex_utils, diagonal, multiply, multiply_base4, permutation, special  # noqa: E402,F401
 
 __all__ = [
     "Butterfly",
     "ButterflyBase4",
+    "ButterflyBmm",
+    "ButterflyUnitary",
     "butterfly_multiply",
     "butterfly_multiply_base4",
     "__version__",

@@ -115,7 +115,7 @@ class Butterfly(nn.Module):
         transpose / conjugate apply the transposed / conjugated matrix; subtwiddle uses only
         the leading part of the parameters for a shorter input (output is then
         nstacks * n' wide, n' the input size rounded up to a power of 2)."""
-        twiddle = self.twiddle
+        twiddle = self.effective_twiddle()
         x = self.pre_process(input)
         output_size = self.out_size if self.nstacks == 1 else None
         if subtwiddle:
@@ -138,19 +138,27 @@ class Butterfly(nn.Module):
         if self.bias is None:
             x = butterfly_multiply(twiddle, x, inc, output_size)
         else:
-            # the kernel that writes the output adds the bias: lay it out as (nstacks, columns)
-            # (post_process keeps the first out_size columns of the flattened stacks; with
-            # subtwiddle, the columns of one stack)
+            # the kernel that writes the output adds the bias, laid out as (stacks, columns)
             cols = output_size if output_size is not None else twiddle.shape[3] * 2
-            total = self.nstacks * cols
-            kept = cols if subtwiddle else self.out_size
-            bias = self.bias[:kept]
-            if bias.shape[0] != kept:
-                raise ValueError("bias is shorter than the output")
-            if kept < total:
-                bias = torch.nn.functional.pad(bias, (0, total - kept))
-            x = butterfly_multiply_bias(twiddle, x, bias.reshape(self.nstacks, cols), inc, output_size)
+            x = butterfly_multiply_bias(twiddle, x, self.bias_rows(cols, subtwiddle), inc, output_size)
         return self.post_process(input, x, out_size=x.size(-1) if subtwiddle else None, add_bias=False)
+
+    def effective_twiddle(self):
+        """(stacks, nblocks, log_n, n/2, 2, 2) factors the multiply runs with."""
+        return self.twiddle
+
+    def bias_rows(self, cols, subtwiddle=False):
+        """The bias as the (stacks, cols) tensor that lines up with the multiply's output:
+        post_process keeps the first out_size columns of the flattened stacks (with subtwiddle,
+        the columns of one stack); the rest is padding."""
+        total = self.nstacks * cols
+        kept = cols if subtwiddle else self.out_size
+        bias = self.bias[:kept]
+        if bias.shape[0] != kept:
+            raise ValueError("bias is shorter than the output")
+        if kept < total:
+            bias = torch.nn.functional.pad(bias, (0, total - kept))
+        return bias.reshape(self.nstacks, cols)
 
     def pre_process(self, input):
         size = input.size(-1)
@@ -195,3 +203,138 @@ class Butterfly(nn.Module):
         return (f"in_size={self.in_size}, out_size={self.out_size}, bias={self.bias is not None}, "
                 f"complex={self.complex}, increasing_stride={self.increasing_stride}, "
                 f"init={self.init}, nblocks={self.nblocks}")
+
+
+class ButterflyUnitary(Butterfly):
+    """Butterfly layer constrained to be unitary: every 2x2 factor is a U(2) element
+    [[e^{i(a+p)} cos f, e^{i(a+x)} sin f], [-e^{i(a-x)} sin f, e^{i(a-p)} cos f]] built from the
+    four real angles (f, a, p, x) stored in ``twiddle[..., 4]``.  Complex; same forward flags as
+    ``Butterfly`` (reference: torch_butterfly/butterfly.py:210-305)."""
+
+    def __init__(self, in_size, out_size, bias=True, increasing_stride=True, nblocks=1):
+        nn.Module.__init__(self)
+        if nblocks < 1:
+            raise ValueError("nblocks must be >= 1")
+        self.in_size = in_size
+        self.out_size = out_size
+        self.log_n = int(math.ceil(math.log2(in_size)))
+        self.n = 1 << self.log_n
+        self.nstacks = -(-out_size // self.n)
+        self.complex = True
+        self.increasing_stride = increasing_stride
+        self.nblocks = nblocks
+        self.init = "ortho"
+        self.twiddle = nn.Parameter(torch.empty(self.nstacks, nblocks, self.log_n, self.n // 2, 4))
+        if bias:
+            self.bias = nn.Parameter(torch.empty(out_size, dtype=real_dtype_to_complex[torch.get_default_dtype()]))
+        else:
+            self.register_parameter("bias", None)
+        self.twiddle._is_structured = True
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        # Haar measure on U(2): sin^2(f) uniform, the three phases uniform
+        core = self.twiddle.shape[:-1]
+        phi = torch.rand(core).sqrt().asin()
+        phases = torch.rand((3,) + tuple(core)) * (2 * math.pi)
+        with torch.no_grad():
+            self.twiddle.copy_(torch.stack((phi, phases[0], phases[1], phases[2]), -1))
+        if self.bias is not None:
+            bound = 1 / math.sqrt(self.in_size)
+            nn.init.uniform_(self.bias, -bound, bound)
+
+    def effective_twiddle(self):
+        phi, alpha, psi, chi = self.twiddle.unbind(-1)
+        c, s = phi.cos(), phi.sin()
+
+        def polar(r, angle):
+            return torch.complex(r * angle.cos(), r * angle.sin())
+
+        top = torch.stack((polar(c, alpha + psi), polar(s, alpha + chi)), -1)
+        bot = torch.stack((polar(-s, alpha - chi), polar(c, alpha - psi)), -1)
+        return torch.stack((top, bot), -2)
+
+    __imul__ = None
+    to_base4 = None
+    diagonal_multiply_ = None
+
+    def extra_repr(self):
+        return (f"in_size={self.in_size}, out_size={self.out_size}, bias={self.bias is not None}, "
+                f"increasing_stride={self.increasing_stride}, nblocks={self.nblocks}")
+
+
+class ButterflyBmm(Butterfly):
+    """``matrix_batch`` independent Butterfly layers applied to the matching slices of the
+    input: (batch, *, matrix_batch, in_size) -> (batch, *, matrix_batch, out_size).  The
+    matrices ride on the stack dimension of one multiply (reference:
+    torch_butterfly/butterfly.py:308-397)."""
+
+    def __init__(self, in_size, out_size, matrix_batch=1, bias=True, complex=False, increasing_stride=True,
+                 init="randn", nblocks=1):
+        nn.Module.__init__(self)
+        if nblocks < 1:
+            raise ValueError("nblocks must be >= 1")
+        self.in_size = in_size
+        self.out_size = out_size
+        self.matrix_batch = matrix_batch
+        self.log_n = int(math.ceil(math.log2(in_size)))
+        self.n = 1 << self.log_n
+        self.nstacks = -(-out_size // self.n)
+        self.complex = complex
+        self.increasing_stride = increasing_stride
+        self.nblocks = nblocks
+        dtype = torch.get_default_dtype()
+        if complex:
+            dtype = real_dtype_to_complex[dtype]
+        shape = (matrix_batch * self.nstacks, nblocks, self.log_n, self.n // 2, 2, 2)
+        if isinstance(init, torch.Tensor):
+            if tuple(init.shape) != shape or init.dtype != dtype:
+                raise ValueError(f"init tensor must have shape {shape} and dtype {dtype}")
+            self.init = None
+            self.twiddle = nn.Parameter(init.clone())
+        else:
+            if init not in _INITS:
+                raise ValueError(f"init must be a tensor or one of {_INITS}")
+            self.init = init
+            self.twiddle = nn.Parameter(torch.empty(shape, dtype=dtype))
+        if bias:
+            self.bias = nn.Parameter(torch.empty(matrix_batch, out_size, dtype=dtype))
+        else:
+            self.register_parameter("bias", None)
+        self.twiddle._is_structured = True
+        self.reset_parameters()
+
+    def forward(self, input, transpose=False, conjugate=False):
+        return super().forward(input, transpose, conjugate, subtwiddle=False)
+
+    def bias_rows(self, cols, subtwiddle=False):
+        total = self.nstacks * cols
+        bias = self.bias[:, :self.out_size]
+        if self.out_size < total:
+            bias = torch.nn.functional.pad(bias, (0, total - self.out_size))
+        return bias.reshape(self.matrix_batch * self.nstacks, cols)
+
+    def pre_process(self, input):
+        size = input.size(-1)
+        if input.size(-2) != self.matrix_batch:
+            raise ValueError("the second to last dimension of the input must be matrix_batch")
+        x = complex_reshape(input, -1, self.matrix_batch, size)
+        x = x.unsqueeze(2).expand(x.shape[0], self.matrix_batch, self.nstacks, size)
+        return x.reshape(x.shape[0], self.matrix_batch * self.nstacks, size)
+
+    def post_process(self, input, output, out_size=None, add_bias=True):
+        out_size = self.out_size if out_size is None else out_size
+        batch = output.shape[0]
+        flat = output.reshape(batch, self.matrix_batch, self.nstacks * output.size(-1))
+        if flat.shape[-1] != out_size:
+            flat = flat[:, :, :out_size]
+        if self.bias is not None and add_bias:
+            flat = flat + self.bias[:, :out_size]
+        return flat.reshape(*input.shape[:-2], self.matrix_batch, out_size)
+
+    to_base4 = None
+
+    def extra_repr(self):
+        return (f"in_size={self.in_size}, out_size={self.out_size}, matrix_batch={self.matrix_batch}, "
+                f"bias={self.bias is not None}, complex={self.complex}, "
+                f"increasing_stride={self.increasing_stride}, init={self.init}, nblocks={self.nblocks}")

@@ -164,3 +164,71 @@ def test_base4_module_equals_base2_module():
             (dx2,) = torch.autograd.grad(y2, x, g)
             (dx4,) = torch.autograd.grad(y4, x, g)
             assert close(dx4, dx2, atol=1e-4)
+
+
+def test_butterfly_unitary_shapes_unitarity_and_gradients():
+    """Model: the reference's tests/test_butterfly.py:212-237 (shapes, B B^H = I), plus the
+    angle gradients against autograd through a dense matrix built from the same factors."""
+    import butterfly_amd as bfa
+    torch.manual_seed(11)
+    for in_size, out_size in [(7, 15), (15, 7)]:
+        for inc in (True, False):
+            for nblocks in (1, 2, 3):
+                say("unitary", in_size, out_size, inc, nblocks)
+                b = bfa.ButterflyUnitary(in_size, out_size, True, inc, nblocks=nblocks).cuda()
+                x = torch.randn(10, in_size, dtype=torch.complex64, device="cuda")
+                assert b(x).shape == (10, out_size)
+    size = 32
+    eye = torch.eye(size, dtype=torch.complex64, device="cuda")
+    for inc in (True, False):
+        for nblocks in (1, 2, 3):
+            b = bfa.ButterflyUnitary(size, size, False, inc, nblocks=nblocks).cuda()
+            M = b(eye).t()
+            assert close(M @ M.conj().t(), eye, atol=1e-4)
+            # transpose and conjugate flags give the inverse of a unitary matrix
+            assert close(b(b(eye), transpose=True, conjugate=True), eye, atol=1e-4)
+    # gradient w.r.t. the angles: compare with the dense product of the same 2x2 factors
+    from butterfly_amd.multiply import butterfly_multiply_torch
+    b = bfa.ButterflyUnitary(16, 16, False, True, nblocks=2).cuda()
+    x = torch.randn(6, 16, dtype=torch.complex64, device="cuda")
+    g = torch.randn(6, 16, dtype=torch.complex64, device="cuda")
+    (ga,) = torch.autograd.grad(b(x), b.twiddle, g)
+    y_ref = butterfly_multiply_torch(b.effective_twiddle(), x.unsqueeze(1), True).squeeze(1)
+    (gr,) = torch.autograd.grad(y_ref, b.twiddle, g)
+    assert close(ga, gr, rtol=1e-3, atol=1e-4)
+
+
+def test_butterfly_bmm_equals_loop_over_layers():
+    """Model: tests/test_butterfly.py:239-266."""
+    import butterfly_amd as bfa
+    torch.manual_seed(12)
+    mb = 3
+    for in_size, out_size in [(7, 15), (15, 7)]:
+        for complex_ in (False, True):
+            for inc in (True, False):
+                for nblocks in (1, 2, 3):
+                    say("bmm", in_size, out_size, complex_, inc, nblocks)
+                    bmm = bfa.ButterflyBmm(in_size, out_size, mb, True, complex_, inc, nblocks=nblocks).cuda()
+                    dtype = torch.complex64 if complex_ else torch.float32
+                    x = torch.randn(10, mb, in_size, dtype=dtype, device="cuda", requires_grad=True)
+                    y = bmm(x)
+                    assert y.shape == (10, mb, out_size)
+                    outs = []
+                    layers = []
+                    for i in range(mb):
+                        tw = bmm.twiddle[i * bmm.nstacks:(i + 1) * bmm.nstacks].detach()
+                        layer = bfa.Butterfly(in_size, out_size, True, complex_, inc, init=tw, nblocks=nblocks).cuda()
+                        with torch.no_grad():
+                            layer.bias.copy_(bmm.bias[i])
+                        layers.append(layer)
+                        outs.append(layer(x[:, i]))
+                    y_loop = torch.stack(outs, 1)
+                    assert close(y, y_loop, atol=1e-5)
+                    g = torch.randn_like(y)
+                    gx, gtw, gb = torch.autograd.grad(y, (x, bmm.twiddle, bmm.bias), g)
+                    hx = torch.autograd.grad(y_loop, x, g)[0]
+                    assert close(gx, hx, atol=1e-4)
+                    for i, layer in enumerate(layers):
+                        ht, hb = torch.autograd.grad(layer(x[:, i]), (layer.twiddle, layer.bias), g[:, i])
+                        assert close(gtw[i * bmm.nstacks:(i + 1) * bmm.nstacks], ht, atol=1e-4)
+                        assert close(gb[i], hb, atol=1e-4)
