@@ -1,11 +1,13 @@
-"""Twiddle algebra: fold a diagonal into a Butterfly, concatenate two Butterflies
-(reference: torch_butterfly/combine.py:11-80)."""
+"""Twiddle algebra: fold a diagonal into a Butterfly, concatenate two Butterflies, tensor and
+Kronecker products, change of stride direction (reference: torch_butterfly/combine.py)."""
 import copy
 
 import torch
+from torch import nn
 from torch.nn import functional as F
 
 from .butterfly import Butterfly
+from .permutation import FixedPermutation, bitreversal_permutation
 
 
 def diagonal_butterfly(butterfly: Butterfly, diagonal: torch.Tensor, diag_first: bool,
@@ -59,3 +61,72 @@ def butterfly_product(butterfly1: Butterfly, butterfly2: Butterfly) -> Butterfly
     out.in_size = butterfly1.in_size
     out.out_size = butterfly2.out_size
     return out
+
+
+class TensorProduct(nn.Module):
+    """map1 along the last dimension, then map2 along the one before it: (*, n2, n1) -> (*, m2, m1)
+    (reference: torch_butterfly/combine.py:80-98)."""
+
+    def __init__(self, map1, map2) -> None:
+        super().__init__()
+        self.map1 = map1
+        self.map2 = map2
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        rows_done = self.map1(input)
+        return self.map2(rows_done.transpose(-1, -2)).transpose(-1, -2)
+
+
+def butterfly_kronecker(butterfly1: Butterfly, butterfly2: Butterfly) -> Butterfly:
+    """The Butterfly of size n1 * n2 equal to butterfly2 (x) butterfly1 on inputs flattened
+    from (n2, n1): element index = i2 * n1 + i1, so butterfly1 owns the low log2(n1) index bits
+    and butterfly2 the high ones.  A stage of butterfly1 then sees every pair index modulo
+    n1 / 2 (its factors tiled n2 times), a stage of butterfly2 sees the pair index divided by n1
+    (each factor repeated n1 times); with increasing stride butterfly1's stages come first.
+    Both must have the same stride direction, one stack, one block and no bias
+    (reference: torch_butterfly/combine.py:101-130)."""
+    if butterfly1.increasing_stride != butterfly2.increasing_stride:
+        raise ValueError("the factors must have the same stride direction")
+    if butterfly1.complex != butterfly2.complex:
+        raise ValueError("the factors must both be real or both be complex")
+    for b in (butterfly1, butterfly2):
+        if b.bias is not None or b.nstacks != 1 or b.nblocks != 1:
+            raise ValueError("butterfly_kronecker needs nstacks == 1, nblocks == 1 and no bias")
+    n1, n2 = 1 << butterfly1.log_n, 1 << butterfly2.log_n
+    low = butterfly1.twiddle.detach().repeat(1, 1, 1, n2, 1, 1)
+    high = butterfly2.twiddle.detach().repeat_interleave(n1, dim=3)
+    stages = (low, high) if butterfly1.increasing_stride else (high, low)
+    out = Butterfly(n1 * n2, n1 * n2, bias=False, complex=butterfly1.complex,
+                    increasing_stride=butterfly1.increasing_stride, init=torch.cat(stages, dim=2))
+    out.in_size = butterfly1.in_size * butterfly2.in_size
+    out.out_size = butterfly1.out_size * butterfly2.out_size
+    return out
+
+
+def permutation_kronecker(perm1: FixedPermutation, perm2: FixedPermutation) -> FixedPermutation:
+    """The permutation of n1 * n2 flattened (n2, n1) elements that applies perm1 within rows and
+    perm2 across rows (reference: torch_butterfly/combine.py:133-139)."""
+    p1, p2 = perm1.permutation, perm2.permutation
+    n1 = p1.shape[-1]
+    return FixedPermutation((p2.unsqueeze(1) * n1 + p1.unsqueeze(0)).reshape(-1))
+
+
+def flip_increasing_stride(butterfly: Butterfly) -> nn.Module:
+    """The same matrix with the opposite stride direction, between two bit reversals.
+
+    Conjugating with the bit reversal P of the element index sends the stage pairing bit l to
+    one pairing bit log_n - 1 - l and keeps its position in the block; the pair index of a
+    stage is the element index with the paired bit removed, so it gets bit-reversed as a
+    (log_n - 1)-bit number.  Hence B = P B' P with B'.twiddle[..., i] = B.twiddle[..., br(i)]
+    (reference: torch_butterfly/combine.py:142-160)."""
+    n = 1 << butterfly.log_n
+    if butterfly.bias is not None or butterfly.in_size != n or butterfly.out_size != n:
+        raise ValueError("flip_increasing_stride needs a square power-of-2 Butterfly without bias")
+    flipped = copy.deepcopy(butterfly)
+    flipped.increasing_stride = not butterfly.increasing_stride
+    if n > 2:
+        pairs = bitreversal_permutation(n // 2, pytorch_format=True).to(butterfly.twiddle.device)
+        with torch.no_grad():
+            flipped.twiddle.copy_(butterfly.twiddle.detach()[:, :, :, pairs])
+    br = bitreversal_permutation(n, pytorch_format=True).to(butterfly.twiddle.device)
+    return nn.Sequential(FixedPermutation(br), flipped, FixedPermutation(br.clone()))

@@ -39,3 +39,158 @@ class FixedPermutation(nn.Module):
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         return index_last_dim(input, self.permutation)
+
+
+def wavelet_permutation(n, pytorch_format=False):
+    """Order of the in-place multilevel Haar transform's outputs: position 0 (the coarsest
+    average), then the positions whose lowest set bit is log2(n) - 1, log2(n) - 2, ..., 0, each
+    group ascending -- [0, 4, 2, 6, 1, 3, 5, 7] for n = 8
+    (reference: torch_butterfly/permutation.py:33-52)."""
+    log_n = int(n).bit_length() - 1
+    if n != 1 << log_n:
+        raise ValueError("n must be a power of 2")
+    groups = [np.zeros(1, dtype=np.int64)]
+    for bit in range(log_n - 1, -1, -1):
+        groups.append(np.arange(1 << bit, n, 2 << bit, dtype=np.int64))
+    perm = np.concatenate(groups)
+    return torch.from_numpy(perm) if pytorch_format else perm
+
+
+def perm_vec_to_mat(p, left=False):
+    """0/1 matrix of the permutation vector p: (M x)[i] = x[p[i]] (left=False), i.e.
+    M[i, p[i]] = 1; left=True gives the transpose (x M convention)."""
+    p = np.asarray(p)
+    m = np.zeros((p.size, p.size), dtype=np.int64)
+    m[np.arange(p.size), p] = 1
+    return m.T if left else m
+
+
+def perm_mat_to_vec(m, left=False):
+    """Inverse of perm_vec_to_mat."""
+    m = np.asarray(m)
+    return np.argmax(m.T if left else m, axis=1)
+
+
+def is_2x2_block_diag(mat):
+    """True when mat is block diagonal with 2x2 blocks."""
+    mat = np.asarray(mat)
+    n = mat.shape[0]
+    if mat.shape != (n, n) or n % 2:
+        return False
+    mask = np.kron(np.eye(n // 2, dtype=bool), np.ones((2, 2), dtype=bool))
+    return not np.any(mat[~mask])
+
+
+def is_butterfly_factor(mat, k):
+    """True when mat is a butterfly factor of block size k: block diagonal with k x k blocks, each
+    of which only couples i with i + k/2 (four diagonal k/2 x k/2 sub-blocks)."""
+    mat = np.asarray(mat)
+    n = mat.shape[0]
+    if mat.shape != (n, n) or n % k or k % 2:
+        return False
+    i, j = np.indices((n, n))
+    allowed = (i // k == j // k) & ((i - j) % (k // 2) == 0)
+    return not np.any(mat[~allowed])
+
+
+def matrix_to_butterfly_factor(mat, log_k, pytorch_format=False, check_input=False):
+    """The (n/2, 2, 2) twiddle of the butterfly factor ``mat`` of block size k = 2^log_k: pair
+    index i couples positions pos and pos + k/2 with pos = 2 (i - i mod k/2) + i mod k/2."""
+    mat = np.asarray(mat)
+    n = mat.shape[0]
+    k = 1 << log_k
+    if check_input and not is_butterfly_factor(mat, k):
+        raise ValueError("not a butterfly factor of this block size")
+    half = k // 2
+    i = np.arange(n // 2)
+    low = i % half
+    pos = 2 * (i - low) + low
+    rows = np.stack((pos, pos + half), -1)                       # (n/2, 2)
+    tw = mat[rows[:, :, None], rows[:, None, :]]                 # tw[i, r, c] = mat[rows[i, r], rows[i, c]]
+    return torch.from_numpy(np.ascontiguousarray(tw)) if pytorch_format else tw
+
+
+def _benes_switches(perm, log_n, increasing_stride):
+    """Routes ``perm`` (out[d] = in[perm[d]]) through the 2 log_n stages of a two-block
+    butterfly whose factors are straight / crossed 2x2 switches (a Benes network: stage j of
+    the first block and stage log_n - 1 - j of the second both pair bit b_j = j for increasing
+    stride, log_n - 1 - j for decreasing).  Looping algorithm, one level per pass: signals
+    sharing an input pair or an output pair of the level's bit take different halves, which
+    2-colours every loop; the colours set the two outer switch columns and leave a permutation
+    inside each half for the next level.  Returns cross[2][log_n][n/2] booleans."""
+    n = 1 << log_n
+    cross = np.zeros((2, log_n, n // 2), dtype=bool)
+    cur = np.asarray(perm, dtype=np.int64).copy()
+    for depth in range(log_n):
+        b = depth if increasing_stride else log_n - 1 - depth
+        bit = 1 << b
+        lowmask = bit - 1
+
+        def pair_index(e):
+            return ((e >> (b + 1)) << b) | (e & lowmask)
+
+        if depth == log_n - 1:
+            # two positions per sub-network left: one switch does it, the other stays straight
+            lo = np.flatnonzero((np.arange(n) & bit) == 0)
+            swapped = cur[lo] != lo
+            cross[0, depth, pair_index(lo)] = swapped
+            break
+        inv = np.empty(n, dtype=np.int64)
+        inv[cur] = np.arange(n)
+        colour = np.full(n, -1, dtype=np.int64)
+        for start in range(n):
+            if colour[start] >= 0:
+                continue
+            d = start
+            while colour[d] < 0:
+                colour[d] = 0
+                partner = d ^ bit               # shares the output pair: other half
+                colour[partner] = 1
+                d = inv[cur[partner] ^ bit]     # shares the input pair with that one: first half again
+        src = cur                                # signal d comes from src[d]
+        # input switch of the pair of s: crossed when the signal entering at the low position leaves for half 1
+        lo_src = np.flatnonzero((src & bit) == 0)            # signals (by destination) whose source has the bit clear
+        cross[0, depth, pair_index(src[lo_src])] = colour[lo_src] == 1
+        # output switch: crossed when the signal bound for the low position travels in half 1
+        lo_dst = np.flatnonzero((np.arange(n) & bit) == 0)
+        cross[1, log_n - 1 - depth, pair_index(lo_dst)] = colour[lo_dst] == 1
+        # inside the halves: signal d now sits at src with the bit set to its colour and must
+        # reach d with the bit set to its colour
+        d_all = np.arange(n)
+        inner_dst = (d_all & ~bit) | (colour * bit)
+        inner_src = (src & ~bit) | (colour * bit)
+        nxt = np.empty(n, dtype=np.int64)
+        nxt[inner_dst] = inner_src
+        cur = nxt
+    return cross
+
+
+def perm2butterfly(v, complex=False, increasing_stride=False):
+    """A two-block Butterfly whose matrix is the permutation v: ``b(x) == x[..., v]``.
+    v is padded with fixed points to the next power of 2
+    (reference: torch_butterfly/permutation.py:395-433)."""
+    from .butterfly import Butterfly  # (butterfly.py does not import this module)
+    if isinstance(v, torch.Tensor):
+        v = v.detach().cpu().numpy()
+    v = np.asarray(v, dtype=np.int64)
+    size = v.size
+    if size < 2:
+        raise ValueError("the permutation must have at least 2 elements")
+    if not np.array_equal(np.sort(v), np.arange(size)):
+        raise ValueError("v is not a permutation")
+    log_n = int(size - 1).bit_length()
+    n = 1 << log_n
+    full = np.concatenate((v, np.arange(size, n, dtype=np.int64)))
+    cross = _benes_switches(full, log_n, increasing_stride)
+    dtype = torch.get_default_dtype()
+    if complex:
+        from .complex_utils import real_dtype_to_complex
+        dtype = real_dtype_to_complex[dtype]
+    straight = torch.eye(2, dtype=dtype)
+    crossed = torch.tensor([[0.0, 1.0], [1.0, 0.0]], dtype=dtype)
+    pick = torch.from_numpy(cross).reshape(1, 2, log_n, n // 2, 1, 1)
+    twiddle = torch.where(pick, crossed, straight)
+    b = Butterfly(n, n, bias=False, complex=complex, increasing_stride=increasing_stride, init=twiddle, nblocks=2)
+    b.in_size = size
+    b.out_size = size
+    return b

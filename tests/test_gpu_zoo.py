@@ -1,0 +1,216 @@
+"""The closed-form transforms, combinators and permutation tools built on the native multiply,
+each against a library routine or a direct computation (the reference's tests/test_special.py,
+test_combine.py and test_permutation.py are the model for what is compared)."""
+import math
+import sys
+
+import numpy as np
+import pytest
+import scipy.fft
+import scipy.linalg
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def close(a, b, rtol=1e-4, atol=1e-4):
+    return torch.allclose(a, b, rtol=rtol, atol=atol)
+
+
+def crand(*shape):
+    return torch.randn(*shape, dtype=torch.complex64, device="cuda")
+
+
+def test_unitary_fourier_transforms():
+    from butterfly_amd import special
+    torch.manual_seed(0)
+    for n in (2, 16, 64):
+        x = crand(5, n)
+        for br_first in (True, False):
+            say("fft_unitary", n, br_first)
+            assert close(special.fft_unitary(n, br_first).cuda()(x), torch.fft.fft(x, norm="ortho"))
+            assert close(special.ifft_unitary(n, br_first).cuda()(x), torch.fft.ifft(x, norm="ortho"))
+
+
+def test_dct_and_dst_against_scipy():
+    from butterfly_amd import special
+    torch.manual_seed(1)
+    for n in (2, 8, 64, 256):
+        x = torch.randn(7, n)
+        for normalized in (False, True):
+            norm = "ortho" if normalized else None
+            for t in (2, 3, 4):
+                say("dct", n, t, normalized)
+                ref = torch.from_numpy(scipy.fft.dct(x.numpy(), type=t, norm=norm))
+                out = special.dct(n, type=t, normalized=normalized).cuda()(x.cuda()).cpu()
+                assert close(out, ref, rtol=1e-4, atol=1e-4 * max(1.0, ref.abs().max().item()))
+            for t in (2, 4):
+                say("dst", n, t, normalized)
+                ref = torch.from_numpy(scipy.fft.dst(x.numpy(), type=t, norm=norm))
+                out = special.dst(n, type=t, normalized=normalized).cuda()(x.cuda()).cpu()
+                assert close(out, ref, rtol=1e-4, atol=1e-4 * max(1.0, ref.abs().max().item()))
+
+
+def test_hadamard_diagonal_and_fastfood():
+    from butterfly_amd import special
+    torch.manual_seed(2)
+    n, k = 32, 3
+    H = torch.from_numpy(scipy.linalg.hadamard(n)).float()
+    x = torch.randn(6, n)
+    diags = torch.randn(k, n)
+    for normalized in (False, True):
+        Hn = H / math.sqrt(n) if normalized else H
+        ref = x
+        for d in diags:
+            ref = (ref * d) @ Hn.t()
+        for inc in (True, False):
+            for sep in (True, False):
+                say("hadamard_diagonal", normalized, inc, sep)
+                m = special.hadamard_diagonal(diags, normalized, inc, sep).cuda()
+                assert close(m(x.cuda()).cpu(), ref, atol=1e-3 * ref.abs().max().item())
+    d1, d2, d3 = torch.randn(3, n)
+    perm = torch.randperm(n)
+    for normalized in (False, True):
+        Hn = H / math.sqrt(n) if normalized else H
+        ref = ((((x * d1) @ Hn.t())[:, perm] * d2) @ Hn.t()) * d3
+        for inc in (True, False):
+            for sep in (True, False):
+                m = special.fastfood(d1, d2, d3, perm, normalized, inc, sep).cuda()
+                assert close(m(x.cuda()).cpu(), ref, atol=1e-3 * ref.abs().max().item())
+
+
+def test_acdc():
+    from butterfly_amd import special
+    torch.manual_seed(3)
+    n = 64
+    x = torch.randn(5, n)
+    d1, d2 = torch.randn(2, n)
+    C = lambda v: torch.from_numpy(scipy.fft.dct(v.numpy(), type=2, norm="ortho"))
+    Ci = lambda v: torch.from_numpy(scipy.fft.idct(v.numpy(), type=2, norm="ortho"))
+    for dct_first in (True, False):
+        ref = Ci(C(x) * d1) * d2 if dct_first else C(Ci(x) * d1) * d2
+        for sep in (True, False):
+            say("acdc", dct_first, sep)
+            m = special.acdc(d1, d2, dct_first, sep).cuda()
+            assert close(m(x.cuda()).cpu(), ref, atol=1e-4 * max(1.0, ref.abs().max().item()))
+
+
+def test_circular_convolutions():
+    from butterfly_amd import special
+    torch.manual_seed(4)
+    for n in (13, 16):
+        for k in (1, 3, 5):
+            for cplx in (False, True):
+                dtype = torch.complex64 if cplx else torch.float32
+                say("conv1d", n, k, cplx)
+                w = torch.randn(1, 1, k, dtype=dtype)
+                x = torch.randn(4, 1, n, dtype=dtype)
+                ref = torch.nn.functional.conv1d(torch.nn.functional.pad(x, (k // 2, k // 2), mode="circular"), w)
+                for sep in (True, False):
+                    m = special.conv1d_circular_singlechannel(n, w, sep).cuda()
+                    assert close(m(x.cuda()).cpu(), ref)
+                w = torch.randn(3, 2, k, dtype=dtype)
+                x = torch.randn(4, 2, n, dtype=dtype)
+                ref = torch.nn.functional.conv1d(torch.nn.functional.pad(x, (k // 2, k // 2), mode="circular"), w)
+                m = special.conv1d_circular_multichannel(n, w).cuda()
+                assert close(m(x.cuda()).cpu(), ref)
+    for (n1, n2, flatten) in [(8, 16, False), (8, 16, True), (6, 9, False)]:
+        for (k1, k2) in [(3, 3), (5, 1)]:
+            say("conv2d", n1, n2, k1, k2, flatten)
+            w = torch.randn(3, 2, k2, k1)
+            x = torch.randn(4, 2, n2, n1)
+            xp = torch.nn.functional.pad(x, (k1 // 2, k1 // 2, k2 // 2, k2 // 2), mode="circular")
+            ref = torch.nn.functional.conv2d(xp, w)
+            m = special.conv2d_circular_multichannel(n1, n2, w, flatten=flatten).cuda()
+            assert close(m(x.cuda()).cpu(), ref, atol=1e-3)
+
+
+def test_fourier_2d():
+    from butterfly_amd import special
+    torch.manual_seed(5)
+    n1, n2 = 16, 8
+    x = crand(3, n2, n1)
+    for normalized in (False, True):
+        norm = "ortho" if normalized else None
+        for br_first in (True, False):
+            for flatten in (False, True):
+                say("fft2d", normalized, br_first, flatten)
+                f = special.fft2d(n1, n2, normalized, br_first, flatten=flatten).cuda()
+                assert close(f(x), torch.fft.fftn(x, dim=(-2, -1), norm=norm), atol=1e-3)
+                f = special.ifft2d(n1, n2, normalized, br_first, flatten=flatten).cuda()
+                assert close(f(x), torch.fft.ifftn(x, dim=(-2, -1), norm=norm), atol=1e-3)
+    for br_first in (True, False):
+        assert close(special.fft2d_unitary(n1, n2, br_first).cuda()(x), torch.fft.fftn(x, dim=(-2, -1), norm="ortho"))
+        assert close(special.ifft2d_unitary(n1, n2, br_first).cuda()(x), torch.fft.ifftn(x, dim=(-2, -1), norm="ortho"))
+
+
+def haar_direct(x):
+    """Multilevel orthonormal Haar transform, coarsest first (what pywt.wavedec(x, 'haar')
+    returns, concatenated)."""
+    out = []
+    a = x
+    while a.shape[-1] > 1:
+        even, odd = a[..., 0::2], a[..., 1::2]
+        out.append((even - odd) / math.sqrt(2))
+        a = (even + odd) / math.sqrt(2)
+    return np.concatenate([a] + out[::-1], axis=-1)
+
+
+def test_wavelet_haar():
+    from butterfly_amd import special
+    rng = np.random.default_rng(6)
+    for n in (2, 8, 32):
+        x = rng.standard_normal((4, n)).astype(np.float32)
+        out = special.wavelet_haar(n).cuda()(torch.from_numpy(x).cuda()).detach().cpu().numpy()
+        assert np.allclose(out, haar_direct(x), atol=1e-5)
+
+
+def test_kronecker_and_flip():
+    import butterfly_amd as bfa
+    from butterfly_amd import combine
+    torch.manual_seed(7)
+    for cplx in (False, True):
+        dtype = torch.complex64 if cplx else torch.float32
+        for inc in (True, False):
+            say("kronecker", cplx, inc)
+            b1 = bfa.Butterfly(8, 8, bias=False, complex=cplx, increasing_stride=inc).cuda()
+            b2 = bfa.Butterfly(16, 16, bias=False, complex=cplx, increasing_stride=inc).cuda()
+            x = torch.randn(3, 16, 8, dtype=dtype, device="cuda")
+            ref = combine.TensorProduct(b1, b2)(x)
+            bk = combine.butterfly_kronecker(b1, b2).cuda()
+            assert close(bk(x.reshape(3, -1)).reshape(3, 16, 8), ref)
+            for nblocks in (1, 2, 3):
+                b = bfa.Butterfly(32, 32, bias=False, complex=cplx, increasing_stride=inc, nblocks=nblocks).cuda()
+                y = torch.randn(5, 32, dtype=dtype, device="cuda")
+                assert close(combine.flip_increasing_stride(b).cuda()(y), b(y))
+    p1 = bfa.permutation.FixedPermutation(torch.randperm(8))
+    p2 = bfa.permutation.FixedPermutation(torch.randperm(4))
+    z = torch.randn(2, 4, 8)
+    assert torch.equal(combine.permutation_kronecker(p1, p2)(z.reshape(2, -1)).reshape(2, 4, 8),
+                       combine.TensorProduct(p1, p2)(z))
+
+
+def test_perm2butterfly():
+    from butterfly_amd import permutation
+    rng = np.random.default_rng(8)
+    for n in (2, 3, 13, 64, 200):
+        for inc in (False, True):
+            for cplx in (False, True):
+                v = rng.permutation(n)
+                say("perm2butterfly", n, inc, cplx)
+                b = permutation.perm2butterfly(v, complex=cplx, increasing_stride=inc).cuda()
+                dtype = torch.complex64 if cplx else torch.float32
+                x = torch.randn(4, n, dtype=dtype, device="cuda")
+                assert torch.equal(b(x), x[:, torch.from_numpy(v).cuda()])
+    m = permutation.perm_vec_to_mat(np.array([2, 0, 1]))
+    assert np.array_equal(permutation.perm_mat_to_vec(m), [2, 0, 1])
+    f = np.kron(np.eye(2), np.array([[1, 0, 2, 0], [0, 3, 0, 4], [5, 0, 6, 0], [0, 7, 0, 8]]))
+    assert permutation.is_butterfly_factor(f, 4) and not permutation.is_butterfly_factor(f, 2)
+    tw = permutation.matrix_to_butterfly_factor(f, 2, check_input=True)
+    assert tw.shape == (4, 2, 2) and np.array_equal(tw[0], [[1, 2], [5, 6]]) and np.array_equal(tw[1], [[3, 4], [7, 8]])
+    assert np.array_equal(permutation.wavelet_permutation(8), [0, 4, 2, 6, 1, 3, 5, 7])

@@ -198,3 +198,51 @@ def test_module_bookkeeping():
     assert torch.allclose(b.twiddle, before * 2.0 ** (1 / 6))
     with pytest.raises(ValueError):
         bfa.Butterfly(8, 8, init=torch.zeros(3))
+
+
+def _apply_switches(cross, log_n, inc, x):
+    """Two-block butterfly of straight / crossed switches applied with numpy."""
+    n = 1 << log_n
+    y = x.copy()
+    for block in range(2):
+        block_inc = inc != (block == 1)
+        for idx in range(log_n):
+            b = idx if block_inc else log_n - 1 - idx
+            bit = 1 << b
+            e = np.flatnonzero((np.arange(n) & bit) == 0)
+            pair = ((e >> (b + 1)) << b) | (e & (bit - 1))
+            swap = cross[block, idx, pair]
+            out = y.copy()
+            out[e[swap]], out[e[swap] ^ bit] = y[e[swap] ^ bit], y[e[swap]]
+            y = out
+    return y
+
+
+def test_permutation_routing_and_helpers_on_the_host():
+    """The Benes routing behind perm2butterfly realises every permutation (exhaustive for n = 4,
+    random up to n = 256), in both stride orders; the small permutation helpers."""
+    import itertools
+    from butterfly_amd import permutation
+    for inc in (False, True):
+        for p in itertools.permutations(range(4)):
+            cross = permutation._benes_switches(np.array(p), 2, inc)
+            assert np.array_equal(_apply_switches(cross, 2, inc, np.arange(4)), np.array(p))
+    rng = np.random.default_rng(0)
+    for log_n in range(1, 9):
+        for inc in (False, True):
+            for _ in range(5):
+                p = rng.permutation(1 << log_n)
+                cross = permutation._benes_switches(p, log_n, inc)
+                assert np.array_equal(_apply_switches(cross, log_n, inc, np.arange(1 << log_n)), p)
+    assert np.array_equal(permutation.wavelet_permutation(8), [0, 4, 2, 6, 1, 3, 5, 7])
+    assert np.array_equal(permutation.wavelet_permutation(2), [0, 1])
+    m = permutation.perm_vec_to_mat(np.array([2, 0, 3, 1]))
+    x = np.arange(4) * 10
+    assert np.array_equal(m @ x, x[[2, 0, 3, 1]])
+    assert np.array_equal(permutation.perm_mat_to_vec(m), [2, 0, 3, 1])
+    assert np.array_equal(permutation.perm_mat_to_vec(permutation.perm_vec_to_mat([2, 0, 3, 1], left=True), left=True),
+                          [2, 0, 3, 1])
+    assert permutation.is_2x2_block_diag(np.kron(np.eye(3), np.ones((2, 2))))
+    assert not permutation.is_2x2_block_diag(np.ones((4, 4)))
+    with pytest.raises(ValueError):
+        permutation.perm2butterfly(np.array([0, 0, 1]))
