@@ -56,3 +56,15 @@ class _IndexLastDim(torch.autograd.Function):
 
 
 index_last_dim = _IndexLastDim.apply
+
+
+def complex_mul(x, y):
+    """Elementwise product (reference: torch_butterfly/complex_utils.py:complex_mul)."""
+    return x * y
+
+
+def complex_matmul(x, y):
+    """Batched matrix product of real or complex tensors.  The reference routes complex
+    operands through cupy or four real products (torch_butterfly/complex_utils.py:41-95) because
+    its PyTorch had no complex matmul on the device; here the library product does it."""
+    return x @ y

@@ -214,3 +214,25 @@ def test_perm2butterfly():
     tw = permutation.matrix_to_butterfly_factor(f, 2, check_input=True)
     assert tw.shape == (4, 2, 2) and np.array_equal(tw[0], [[1, 2], [5, 6]]) and np.array_equal(tw[1], [[3, 4], [7, 8]])
     assert np.array_equal(permutation.wavelet_permutation(8), [0, 4, 2, 6, 1, 3, 5, 7])
+
+
+def test_kop2d_fft_init_is_a_circular_convolution():
+    """Model: convolution/models/test_kops.py of the reference."""
+    from butterfly_amd.kops import KOP2d
+    torch.manual_seed(9)
+    in_ch, out_ch = 3, 6
+    for in_size in [(32, 32), (16, 16), (32, 16), (16, 32)]:
+        for nblocks in (1, 2, 3):
+            for base in (2, 4):
+                say("kop2d", in_size, nblocks, base)
+                kop = KOP2d(in_size, in_ch, out_ch, 5, init="fft", nblocks=nblocks, base=base).cuda()
+                x = torch.randn(10, in_ch, *in_size, device="cuda")
+                conv = torch.nn.Conv2d(in_ch, out_ch, 5, padding=2, padding_mode="circular", bias=False).cuda()
+                with torch.no_grad():
+                    conv.weight.copy_(kop.weight.flip([-1, -2]))
+                assert close(kop(x), conv(x), rtol=1e-4, atol=1e-4)
+    # gradients reach the kernel and the factors
+    kop = KOP2d(16, 2, 3, 3, init="ortho").cuda()
+    y = kop(torch.randn(4, 2, 16, 16, device="cuda"))
+    y.square().mean().backward()
+    assert kop.weight.grad is not None and all(p.grad is not None for p in kop.parameters())
