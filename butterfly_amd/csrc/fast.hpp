@@ -390,13 +390,13 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     using P = FastPlan<L, NB, INC>;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
-    // float rows are fetched straight into LDS, one iteration (R row groups) ahead, and the
+    // float rows are fetched straight into LDS, two iterations (2 R row groups) ahead, and the
     // walk starts in the layout of its first stage; complex64 rows arrive in registers, layout A
     constexpr bool DIRECT = sizeof(T) == 4;
     constexpr int SF = DIRECT ? P::layout(0) : 0;
     constexpr int TT = P::fw_transposes_total(SF);  // barriers per iteration
     __shared__ __align__(16) T lds[TT > 0 ? 2 * R * kFastRowWords : 1];
-    __shared__ float lds_rows[DIRECT ? 2 * R * kFastRowWords : 1];
+    __shared__ float lds_rows[DIRECT ? 4 * R * kFastRowWords : 1];  // four sets of R row slots
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
@@ -437,18 +437,37 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     const int slot_d = t >> L, col_d = (chunk << L) + (t & (n - 1));
     const int in_dma = col_d < a.in_view.width ? slot_d * in_row + (int)(col_d * a.in_view.se * EB) : kOob;
     const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
-    auto fetch_rows = [&](int grel, int set) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const bool ok = (grel + r) * SLOTS + slot_d < rows_valid;
-            load_row_to_lds(in_desc, rows_addr + (set * R + r) * kFastRowWords * 4, ok ? in_dma : kOob,
-                            (grel + r) * SLOTS * in_row);
-        }
+    auto fetch_row = [&](int grel, int set, int r) {
+        const bool ok = (grel + r) * SLOTS + slot_d < rows_valid;
+        load_row_to_lds(in_desc, rows_addr + (set * R + r) * kFastRowWords * 4, ok ? in_dma : kOob,
+                        (grel + r) * SLOTS * in_row);
     };
+    // The requests of an iteration are spread over its TT + 1 phases (row r goes out at the
+    // start of phase r mod (TT + 1)): sixteen wavefronts asking for R rows each at the same
+    // moment, right behind the previous iteration's stores, queue up at the memory pipeline.
+    auto fetch_phase = [&](int grel, int set, auto PHASE) {
+        static_for<0, R>([&](auto RR) {
+            if constexpr (RR % (TT + 1) == decltype(PHASE)::value) fetch_row(grel, set, RR);
+        });
+    };
+    // requests of an iteration that go out before its last barrier (all of them when there is none)
+    constexpr int EARLY = [] {
+        int c = 0;
+        for (int r = 0; r < R; ++r) c += (TT == 0 || r % (TT + 1) < TT) ? 1 : 0;
+        return c;
+    }();
+    // Before the last barrier of an iteration each wavefront waits for the rows of the next
+    // iteration, requested during the previous one.  Younger than those: the previous
+    // iteration's R stores and this iteration's EARLY requests.
+    constexpr int YOUNGER = R + EARLY;
 
     T nxt[R];
     if constexpr (DIRECT) {
-        fetch_rows(0, 0);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            fetch_row(0, 0, r);
+            fetch_row(R, 1, r);
+        }
         wait_rows_in_lds<0>();
         __syncthreads();
     } else {
@@ -464,8 +483,8 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     for (int grel = 0; grel < ng; grel += R) {
         T v[R];
         if constexpr (DIRECT) {
-            const int set = (grel / R) & 1;
-            fetch_rows(grel + R, set ^ 1);
+            const int set = (grel / R) & 3;
+            fetch_phase(grel + 2 * R, (set + 2) & 3, std::integral_constant<int, 0>{});
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const float x = lds_rows[(set * R + r) * kFastRowWords + (SF ? c.fB : c.fA)];
@@ -477,8 +496,6 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
             load_rows(grel + R, nxt);
         }
 
-        // The rows requested above must be in LDS, for every wavefront, when the next
-        // iteration starts: each wavefront waits for its own just before the last barrier.
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
             constexpr int K = P::kind(s);
@@ -487,7 +504,9 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
                 constexpr int to_b = P::layout(s);
                 T *buf = lds + (nth & 1) * R * kFastRowWords;
                 const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
-                transpose_rows<T, R, DIRECT && nth + 1 == TT>(buf, wr, rd, v);
+                transpose_rows<T, R, DIRECT && nth + 1 == TT, YOUNGER>(buf, wr, rd, v);
+                if constexpr (DIRECT)
+                    fetch_phase(grel + 2 * R, (((grel / R) & 3) + 2) & 3, std::integral_constant<int, nth + 1>{});
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) v[r] = fw_product<K>(v[r], ta[s], tb[s], c.bperm_addr);
@@ -495,9 +514,11 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
         if constexpr (P::layout(NS - 1) != 0) {
             constexpr int nth = P::fw_transposes_before(NS, SF);
             T *buf = lds + (nth & 1) * R * kFastRowWords;
-            transpose_rows<T, R, DIRECT>(buf, c.fB, c.fA, v);
+            transpose_rows<T, R, DIRECT, YOUNGER>(buf, c.fB, c.fA, v);
+            if constexpr (DIRECT)
+                fetch_phase(grel + 2 * R, (((grel / R) & 3) + 2) & 3, std::integral_constant<int, nth + 1>{});
         }
-        if constexpr (DIRECT && TT == 0) wait_rows_in_lds<0>();
+        if constexpr (DIRECT && TT == 0) wait_rows_in_lds<YOUNGER>();
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
