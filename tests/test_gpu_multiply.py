@@ -421,3 +421,40 @@ def test_bias_operator_autograd():
             assert (a - b).abs().max().item() <= 1e-4 * max(1.0, b.abs().max().item())
     with pytest.raises(RuntimeError, match="bias must have shape"):
         ops.butterfly_multiply_bias_fw(tw.detach(), x.detach(), bias.detach()[:, :-1], True, None)
+
+
+@pytest.mark.parametrize("shape", [(600, 1, 10, 2, False), (300, 1, 12, 2, True), (100, 2, 11, 1, False)],
+                         ids=lambda s: f"B{s[0]}-S{s[1]}-L{s[2]}-nb{s[3]}")
+def test_library_calls_replay_from_a_captured_graph(shape):
+    """The library neither allocates nor synchronises, so its calls can be recorded in a HIP
+    graph; every replay (with eager work and synchronisation in between) must reproduce what
+    the eager calls give for the operands then in place."""
+    from butterfly_amd import _capi
+    B, S, L, nb, inc = shape
+    n = 1 << L
+    say("graph case", shape)
+    torch.manual_seed(21)
+    tw = (torch.randn(S, nb, L, n // 2, 2, 2) / 2 ** 0.5).cuda()
+    x = torch.randn(B, S, n).cuda()
+    g = torch.randn(B, S, n).cuda()
+    bias = torch.randn(S, n).cuda()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):     # warm-up outside the capture, as graphs require
+        _capi.multiply_bias_fw(tw, x, bias, inc)
+        _capi.multiply_bias_bw(tw, x, g, inc)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = _capi.multiply_bias_fw(tw, x, bias, inc)
+        dtw, dx, db = _capi.multiply_bias_bw(tw, x, g, inc)
+    for rep in range(3):
+        x.copy_(torch.randn(B, S, n).cuda())
+        g.copy_(torch.randn(B, S, n).cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        y_e = _capi.multiply_bias_fw(tw, x, bias, inc)
+        dtw_e, dx_e, db_e = _capi.multiply_bias_bw(tw, x, g, inc)
+        torch.cuda.synchronize()
+        assert torch.equal(y, y_e) and torch.equal(dx, dx_e) and torch.equal(dtw, dtw_e) and torch.equal(db, db_e), rep
