@@ -67,6 +67,17 @@ CONFIGS = {
                       metric="Butterfly(4096,4096,bias) module fwd+bwd GB/s, bias as separate PyTorch ops",
                       workload="cfg5 (module level, unfused): the same layer computed as butterfly_multiply followed "
                                "by a PyTorch `+ bias`, autograd backward; for comparison with cfg5m"),
+    "cfg3m": dict(batch=8192, nstacks=1, log_n=12, nblocks=1, inc=True, cplx=True, base4=False, bw=True,
+                  cpu_batch=256, module="fft-fused",
+                  metric="special.fft(4096) module fwd+bwd GB/s, complex64, batch 8192, bit reversal folded in",
+                  workload="cfg3 (module level): special.fft(4096, normalized=True) = bit reversal + Butterfly, "
+                           "forward + autograd backward (d_input, d_twiddle), input (8192,4096) complex64; the "
+                           "bit reversal is applied by the multiply's own first read / last write"),
+    "cfg3m-sep": dict(batch=8192, nstacks=1, log_n=12, nblocks=1, inc=True, cplx=True, base4=False, bw=True,
+                      cpu_batch=256, module="fft-sep",
+                      metric="special.fft(4096) module fwd+bwd GB/s, bit reversal as a separate gather",
+                      workload="cfg3 (module level, unfused): the same two modules run one after the other "
+                               "(PyTorch gather, then butterfly_multiply); for comparison with cfg3m"),
 }
 
 
@@ -138,7 +149,7 @@ def make_operands(c, torch, dev):
         tw4 = (torch.randn(S, nb, L // 2, n // 4, 4, 4, dtype=dtype) / 2).to(dev)
         tw2 = (torch.randn(S, nb, L % 2, n // 2, 2, 2, dtype=dtype) / 2 ** 0.5).to(dev)
         tws = (tw4, tw2)
-    elif c["cplx"]:
+    elif c["cplx"] and S == 1 and nb == 1:
         from butterfly_amd import special
         tws = (special.fft(n, normalized=True, with_br_perm=False).twiddle.detach().to(dev),)
     elif nb == 2 and L == 12:
@@ -157,6 +168,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="cfg2", choices=sorted(CONFIGS))
+    ap.add_argument("--shape", default=None, metavar="B,S,LOG_N,NBLOCKS,f32|c64[,inc|dec]",
+                    help="forward + backward at an arbitrary shape instead of a named configuration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of the input (a kernel of known traffic, for scaling "
@@ -165,6 +178,18 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU; --gpus must be 1 (rows shard trivially, see DESIGN.md)")
     c = CONFIGS[args.config]
+    if args.shape:
+        f = args.shape.split(",")
+        B, S, L, nb = (int(v) for v in f[:4])
+        cplx = f[4] == "c64"
+        inc = len(f) < 6 or f[5] == "inc"
+        args.config = "shape"
+        c = dict(batch=B, nstacks=S, log_n=L, nblocks=nb, inc=inc, cplx=cplx, base4=False, bw=True,
+                 cpu_batch=max(1, min(B, (1 << 21) // (S << L))),
+                 metric=f"butterfly_multiply fwd+bwd GB/s, batch {B} nstacks {S} n={1 << L} nblocks {nb} "
+                        f"{'complex64' if cplx else 'fp32'}",
+                 workload=f"shape: butterfly_multiply fw+bw, input ({B},{S},{1 << L}) {'complex64' if cplx else 'fp32'} "
+                          f"N(0,1), twiddle ({S},{nb},{L},{(1 << L) // 2},2,2) N(0,1/2), increasing_stride={inc}")
 
     import torch
     import butterfly_amd
@@ -175,7 +200,20 @@ def main():
     tws, x, grad = make_operands(c, torch, dev)
     inc = c["inc"]
 
-    if c.get("module"):
+    if c.get("module", "").startswith("fft"):
+        # module level: bit reversal + butterfly, then autograd for both gradients
+        from butterfly_amd import special
+        layer = special.fft(1 << c["log_n"], normalized=True).to(dev)
+        if c["module"] == "fft-sep":
+            layer = torch.nn.Sequential(*layer)
+        xm = x.reshape(c["batch"], -1).requires_grad_()
+        gm = grad.reshape(c["batch"], -1)
+        state = {}
+
+        def fw_call():
+            state["y"] = layer(xm)
+        bw_call = lambda: torch.autograd.grad(state["y"], (xm, layer[1].twiddle), gm)
+    elif c.get("module"):
         # module level: the layer's forward, then autograd for all three gradients
         layer = butterfly_amd.Butterfly(1 << c["log_n"], 1 << c["log_n"], bias=True, init="ortho",
                                         nblocks=c["nblocks"]).to(dev)

@@ -19,6 +19,7 @@ SYMBOLS = [
     "bf_butterfly_multiply_bw_workspace_bytes", "bf_butterfly_multiply_bw",
     "bf_butterfly_multiply_bias_fw", "bf_butterfly_bias_grad", "bf_butterfly_bias_grad_workspace_bytes",
     "bf_butterfly_multiply_bias_bw", "bf_butterfly_multiply_bias_bw_workspace_bytes",
+    "bf_butterfly_multiply_perm_fw", "bf_butterfly_multiply_perm_bw",
     "bf_butterfly_multiply_base4_fw", "bf_butterfly_multiply_base4_fw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw",
@@ -68,6 +69,8 @@ def lib():
         L.bf_butterfly_multiply_bias_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_bias_bw_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_bias_bw_workspace_bytes.restype = sz
+        L.bf_butterfly_multiply_perm_fw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_perm_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_base4_fw.argtypes = [pp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_base4_fw_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_base4_fw_workspace_bytes.restype = sz
@@ -185,6 +188,53 @@ def multiply_bias_bw(twiddle, input, grad, increasing_stride):
     _check(lib().bf_butterfly_multiply_bias_bw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
                                                _ptr(d_twiddle), _ptr(d_input), _ptr(d_bias), _ptr(ws), nbytes,
                                                _stream()))
+    return d_twiddle, d_input, d_bias
+
+
+def _table(t, n):
+    if t is None:
+        return None
+    assert t.is_cuda and t.dtype == torch.int32 and t.is_contiguous() and tuple(t.shape) == (n,)
+    return _ptr(t)
+
+
+def multiply_perm_fw(twiddle, input, in_perm, out_index, bias, increasing_stride, output_size=None):
+    """Forward between two column permutations (int32 tables of n entries or None):
+    u[c] = input[in_perm[c]], output[out_index[c]] = multiply(u)[c] + bias[c]."""
+    assert twiddle.is_contiguous() and twiddle.is_cuda and input.is_cuda
+    nb, log_n = twiddle.shape[1], twiddle.shape[2]
+    n = 1 << log_n
+    O = n if output_size is None else output_size
+    p = make_problem(input, log_n, nb, increasing_stride, O)
+    out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
+    p.output_stride = _strides(out)
+    nbytes = lib().bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_perm_fw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _table(in_perm, n),
+                                               _table(out_index, n), None if bias is None else _ptr(bias),
+                                               _ptr(out), _ptr(ws), nbytes, _stream()))
+    return out
+
+
+def multiply_perm_bw(twiddle, input, grad, in_perm, out_index, increasing_stride, with_bias=False):
+    """Backward of multiply_perm_fw.  Returns (d_twiddle, d_input, d_bias or None)."""
+    assert twiddle.is_contiguous() and twiddle.is_cuda and input.is_cuda and grad.is_cuda
+    nb, log_n = twiddle.shape[1], twiddle.shape[2]
+    n = 1 << log_n
+    p = make_problem(input, log_n, nb, increasing_stride, grad.shape[2])
+    p.output_stride = _strides(grad)
+    d_twiddle = torch.empty_like(twiddle)
+    d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
+    d_bias = torch.empty(grad.shape[1], grad.shape[2], dtype=grad.dtype, device=grad.device) if with_bias else None
+    p.d_input_stride = _strides(d_input)
+    size_fn = lib().bf_butterfly_multiply_bias_bw_workspace_bytes if with_bias \
+        else lib().bf_butterfly_multiply_bw_workspace_bytes
+    nbytes = size_fn(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_perm_bw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
+                                               _table(in_perm, n), _table(out_index, n), _ptr(d_twiddle),
+                                               _ptr(d_input), None if d_bias is None else _ptr(d_bias), _ptr(ws),
+                                               nbytes, _stream()))
     return d_twiddle, d_input, d_bias
 
 

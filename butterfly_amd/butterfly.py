@@ -11,7 +11,7 @@ import torch
 from torch import nn
 
 from .complex_utils import complex_reshape, real_dtype_to_complex
-from .multiply import butterfly_multiply, butterfly_multiply_bias
+from .multiply import butterfly_multiply, butterfly_multiply_bias, butterfly_multiply_perm
 
 _INITS = ("empty", "randn", "ortho", "identity", "fft_no_br", "ifft_no_br")
 
@@ -109,12 +109,23 @@ class Butterfly(nn.Module):
                 if self.nblocks > 1:
                     tw[:, 1:] = torch.eye(2, dtype=tw.dtype)
 
-    def forward(self, input, transpose=False, conjugate=False, subtwiddle=False):
+    def forward(self, input, transpose=False, conjugate=False, subtwiddle=False, in_perm=None, out_index=None):
         """input (batch, *, in_size) -> (batch, *, out_size).
 
         transpose / conjugate apply the transposed / conjugated matrix; subtwiddle uses only
         the leading part of the parameters for a shorter input (output is then
-        nstacks * n' wide, n' the input size rounded up to a power of 2)."""
+        nstacks * n' wide, n' the input size rounded up to a power of 2).
+
+        in_perm / out_index (int32 tables of n entries, see FixedPermutation.column_table): a
+        fixed permutation in front of / behind the layer, applied by the layer's own kernels;
+        they describe the untransposed layer (transpose swaps their roles)."""
+        if in_perm is not None or out_index is not None:
+            if subtwiddle:
+                raise ValueError("column tables cannot be combined with subtwiddle")
+            if out_index is not None and self.nstacks != 1:
+                raise ValueError("a permutation behind the layer needs nstacks == 1")
+            if transpose:
+                in_perm, out_index = out_index, in_perm
         twiddle = self.effective_twiddle()
         x = self.pre_process(input)
         output_size = self.out_size if self.nstacks == 1 else None
@@ -135,7 +146,11 @@ class Butterfly(nn.Module):
             inc = not last_inc
         else:
             inc = self.increasing_stride
-        if self.bias is None:
+        if in_perm is not None or out_index is not None:
+            cols = output_size if output_size is not None else twiddle.shape[3] * 2
+            bias = None if self.bias is None else self.bias_rows(cols, subtwiddle)
+            x = butterfly_multiply_perm(twiddle, x, in_perm, out_index, bias, inc, output_size)
+        elif self.bias is None:
             x = butterfly_multiply(twiddle, x, inc, output_size)
         else:
             # the kernel that writes the output adds the bias, laid out as (stacks, columns)

@@ -7,7 +7,7 @@ from torch import nn
 from torch.nn import functional as F
 
 from .butterfly import Butterfly
-from .permutation import FixedPermutation, bitreversal_permutation
+from .permutation import FixedPermutation, FusedSequential, bitreversal_permutation
 
 
 def diagonal_butterfly(butterfly: Butterfly, diagonal: torch.Tensor, diag_first: bool,
@@ -129,4 +129,4 @@ def flip_increasing_stride(butterfly: Butterfly) -> nn.Module:
         with torch.no_grad():
             flipped.twiddle.copy_(butterfly.twiddle.detach()[:, :, :, pairs])
     br = bitreversal_permutation(n, pytorch_format=True).to(butterfly.twiddle.device)
-    return nn.Sequential(FixedPermutation(br), flipped, FixedPermutation(br.clone()))
+    return FusedSequential(FixedPermutation(br), flipped, FixedPermutation(br.clone()))

@@ -33,8 +33,10 @@ __global__ __launch_bounds__(kBiasThreads) void bias_add_kernel(BiasArgs a)
     const int64_t col = (int64_t)blockIdx.x * kBiasThreads + threadIdx.x;
     const int stack = blockIdx.y;
     if (col >= a.width) return;
+    const int64_t vc = view_col(a.view, col);
+    if (vc < 0) return;
     const T b = reinterpret_cast<const T *>(a.bias)[stack * a.width + col];
-    T *out = reinterpret_cast<T *>(a.out) + stack * a.view.ss + col * a.view.se;
+    T *out = reinterpret_cast<T *>(a.out) + stack * a.view.ss + vc * a.view.se;
     const int64_t r0 = (int64_t)blockIdx.z * a.rows_per_part;
     const int64_t r1 = r0 + a.rows_per_part < a.batch ? r0 + a.rows_per_part : a.batch;
     for (int64_t r = r0; r < r1; ++r) out[r * a.view.sb] = add(out[r * a.view.sb], b);
@@ -46,9 +48,10 @@ __global__ __launch_bounds__(kBiasThreads) void bias_grad_partial_kernel(BiasArg
     const int64_t col = (int64_t)blockIdx.x * kBiasThreads + threadIdx.x;
     const int stack = blockIdx.y;
     if (col >= a.width) return;
-    const T *g = reinterpret_cast<const T *>(a.grad) + stack * a.view.ss + col * a.view.se;
+    const int64_t vc = view_col(a.view, col);
+    const T *g = reinterpret_cast<const T *>(a.grad) + stack * a.view.ss + (vc < 0 ? 0 : vc) * a.view.se;
     const int64_t r0 = (int64_t)blockIdx.z * a.rows_per_part;
-    const int64_t r1 = r0 + a.rows_per_part < a.batch ? r0 + a.rows_per_part : a.batch;
+    const int64_t r1 = vc < 0 ? r0 : (r0 + a.rows_per_part < a.batch ? r0 + a.rows_per_part : a.batch);
     // four running sums keep four loads in flight; they are combined in a fixed order
     T s0 = zero_of(T()), s1 = s0, s2 = s0, s3 = s0;
     int64_t r = r0;

@@ -94,13 +94,14 @@ Schedule make_schedule(const bf_problem *p, bool base4)
     return sc;
 }
 
-View make_view(const int64_t stride[3], int64_t width)
+View make_view(const int64_t stride[3], int64_t width, const int *perm = nullptr)
 {
     View v;
     v.sb = stride[0];
     v.ss = stride[1];
     v.se = stride[2];
     v.width = width;
+    v.perm = perm;
     return v;
 }
 
@@ -111,6 +112,7 @@ View dense_view(int64_t nstacks, int64_t n)
     v.ss = n;
     v.se = 1;
     v.width = n;
+    v.perm = nullptr;
     return v;
 }
 
@@ -649,11 +651,24 @@ int launch_bias_add(const bf_problem *p, const void *bias, void *output, const V
     return BF_OK;
 }
 
+// Column tables are only defined over the n columns of the transform and need a stage to ride on.
+int check_perms(const bf_problem *p, bool base4, const int *in_perm, const int *out_index)
+{
+    if (!in_perm && !out_index) return BF_OK;
+    const int64_t n = (int64_t)1 << p->log_n;
+    if (p->input_size > n) return fail(BF_ERR_INVALID, "column tables need input_size <= n");
+    if (make_schedule(p, base4).per * p->nblocks == 0)
+        return fail(BF_ERR_UNSUPPORTED, "column tables need at least one stage");
+    return BF_OK;
+}
+
 int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, const void *input,
-            void *output, void *workspace, size_t workspace_bytes, void *stream_, const void *bias = nullptr)
+            void *output, void *workspace, size_t workspace_bytes, void *stream_, const void *bias = nullptr,
+            const int *in_perm = nullptr, const int *out_index = nullptr)
 {
     int rc = check_problem(p, false);
     if (rc) return rc;
+    if ((rc = check_perms(p, base4, in_perm, out_index))) return rc;
     if ((rc = ensure_attributes())) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const Schedule sc = make_schedule(p, base4);
@@ -667,8 +682,8 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
             if (base4 && (p->log_n & 1) && !tw2) return fail(BF_ERR_INVALID, "twiddle2 is NULL");
         }
     }
-    const View in_view = make_view(p->input_stride, std::min(p->input_size, n));
-    const View out_view = make_view(p->output_stride, p->output_size);
+    const View in_view = make_view(p->input_stride, std::min(p->input_size, n), in_perm);
+    const View out_view = make_view(p->output_stride, p->output_size, out_index);
     if (fast4_ok(p, base4, false)) {
         const size_t need = forward_workspace(p, base4);
         if (need > 0 && (!workspace || workspace_bytes < need))
@@ -719,11 +734,11 @@ BiasGradPlan plan_bias_grad(const bf_problem *p)
 
 template <typename T>
 int launch_bias_grad(const bf_problem *p, const BiasGradPlan &b, const void *grad, void *d_bias, void *workspace,
-                     hipStream_t stream)
+                     hipStream_t stream, const int *out_index)
 {
     BiasArgs a = {};
     a.grad = grad;
-    a.view = make_view(p->output_stride, p->output_size);
+    a.view = make_view(p->output_stride, p->output_size, out_index);
     a.partial = workspace;
     a.d_bias = d_bias;
     a.batch = p->batch;
@@ -882,11 +897,13 @@ int launch_reduce(const bf_problem *p, const Schedule &sc, int t0, int t1, int64
 // (*bias_nparts slices of (S, output_size)); *bias_nparts stays 0 otherwise.
 int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, const void *input,
              const void *grad, void *d_tw2, void *d_tw4, void *d_input, void *workspace,
-             size_t workspace_bytes, void *stream_, void *bias_partial = nullptr, int64_t *bias_nparts = nullptr)
+             size_t workspace_bytes, void *stream_, void *bias_partial = nullptr, int64_t *bias_nparts = nullptr,
+             const int *in_perm = nullptr, const int *out_index = nullptr)
 {
     if (bias_nparts) *bias_nparts = 0;
     int rc = check_problem(p, true);
     if (rc) return rc;
+    if ((rc = check_perms(p, base4, in_perm, out_index))) return rc;
     if ((rc = ensure_attributes())) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const Schedule sc = make_schedule(p, base4);
@@ -899,9 +916,9 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
         return fail(BF_ERR_WORKSPACE, "workspace must be 16-byte aligned");
 
-    const View x_view = make_view(p->input_stride, std::min(p->input_size, n));
-    const View g_view = make_view(p->output_stride, std::min(p->output_size, n));
-    const View di_view = make_view(p->d_input_stride, p->input_size);
+    const View x_view = make_view(p->input_stride, std::min(p->input_size, n), in_perm);
+    const View g_view = make_view(p->output_stride, std::min(p->output_size, n), out_index);
+    const View di_view = make_view(p->d_input_stride, p->input_size, in_perm);
     const View dense = dense_view(p->nstacks, n);
     char *ws = static_cast<char *>(workspace);
     const size_t e_bytes = elem_bytes(p->dtype);
@@ -918,7 +935,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                                k == 0 ? x_view : dense, dense, k, k + 1, stream);
             if (rc) return rc;
         }
-        const View dn_view = make_view(p->d_input_stride, std::min(p->input_size, n));
+        const View dn_view = make_view(p->d_input_stride, std::min(p->input_size, n), in_perm);
         const FastGrid g = fast_grid(p->batch, L, p->nstacks, 1, 1);
         for (int k = P - 1; k >= 0; --k) {
             Fast4Args a = {};
@@ -963,7 +980,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                                    k == 0 ? x_view : dense, dense, k, k + 1, stream);
             if (rc) return rc;
         }
-        const View dn_view = make_view(p->d_input_stride, std::min(p->input_size, n));
+        const View dn_view = make_view(p->d_input_stride, std::min(p->input_size, n), in_perm);
         for (int k = P - 1; k >= 0; --k) {
             const Pass &q = mp.pass[k];
             const void *xin = k == 0 ? input : boundary(k);
@@ -1138,8 +1155,9 @@ size_t bf_butterfly_bias_grad_workspace_bytes(const bf_problem *p)
     return plan_bias_grad(p).bytes;
 }
 
-int bf_butterfly_bias_grad(const bf_problem *p, const void *grad, void *d_bias, void *workspace,
-                           size_t workspace_bytes, void *stream)
+// d_bias[s][c] = sum over the batch of grad[b][s][out_index[c]] (out_index NULL: column c)
+static int bias_grad(const bf_problem *p, const void *grad, void *d_bias, void *workspace, size_t workspace_bytes,
+                     void *stream, const int *out_index)
 {
     int rc = check_problem(p, false);
     if (rc) return rc;
@@ -1161,8 +1179,14 @@ int bf_butterfly_bias_grad(const bf_problem *p, const void *grad, void *d_bias, 
     const BiasGradPlan b = plan_bias_grad(p);
     if (!workspace || workspace_bytes < b.bytes)
         return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", b.bytes, workspace_bytes);
-    return p->dtype == BF_C64 ? launch_bias_grad<float2>(p, b, grad, d_bias, workspace, s)
-                              : launch_bias_grad<float>(p, b, grad, d_bias, workspace, s);
+    return p->dtype == BF_C64 ? launch_bias_grad<float2>(p, b, grad, d_bias, workspace, s, out_index)
+                              : launch_bias_grad<float>(p, b, grad, d_bias, workspace, s, out_index);
+}
+
+int bf_butterfly_bias_grad(const bf_problem *p, const void *grad, void *d_bias, void *workspace,
+                           size_t workspace_bytes, void *stream)
+{
+    return bias_grad(p, grad, d_bias, workspace, workspace_bytes, stream, nullptr);
 }
 
 // Bias area behind the backward workspace: room for either the per-workgroup column sums the
@@ -1181,9 +1205,9 @@ size_t bf_butterfly_multiply_bias_bw_workspace_bytes(const bf_problem *p)
     return align256(plan_bw(p, false).total) + bias_area_bytes(p);
 }
 
-int bf_butterfly_multiply_bias_bw(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
-                                  void *d_twiddle, void *d_input, void *d_bias, void *workspace,
-                                  size_t workspace_bytes, void *stream)
+static int bias_backward(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
+                         void *d_twiddle, void *d_input, void *d_bias, void *workspace, size_t workspace_bytes,
+                         void *stream, const int *in_perm, const int *out_index)
 {
     int rc = check_problem(p, true);
     if (rc) return rc;
@@ -1195,7 +1219,7 @@ int bf_butterfly_multiply_bias_bw(const bf_problem *p, const void *twiddle, cons
     char *area = static_cast<char *>(workspace) + main_bytes;
     int64_t nparts = 0;
     rc = backward(p, false, twiddle, nullptr, input, grad, d_twiddle, nullptr, d_input, workspace, main_bytes, stream,
-                  area, &nparts);
+                  area, &nparts, in_perm, out_index);
     if (rc) return rc;
     if (p->nstacks <= 0 || p->output_size <= 0) return BF_OK;
     if (nparts > 0) {
@@ -1211,7 +1235,34 @@ int bf_butterfly_multiply_bias_bw(const bf_problem *p, const void *twiddle, cons
         BF_HIP_CHECK(hipGetLastError());
         return BF_OK;
     }
-    return bf_butterfly_bias_grad(p, grad, d_bias, area, bias_area_bytes(p), stream);
+    return bias_grad(p, grad, d_bias, area, bias_area_bytes(p), stream, out_index);
+}
+
+int bf_butterfly_multiply_bias_bw(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
+                                  void *d_twiddle, void *d_input, void *d_bias, void *workspace,
+                                  size_t workspace_bytes, void *stream)
+{
+    return bias_backward(p, twiddle, input, grad, d_twiddle, d_input, d_bias, workspace, workspace_bytes, stream,
+                         nullptr, nullptr);
+}
+
+int bf_butterfly_multiply_perm_fw(const bf_problem *p, const void *twiddle, const void *input, const int32_t *in_perm,
+                                  const int32_t *out_index, const void *bias, void *output, void *workspace,
+                                  size_t workspace_bytes, void *stream)
+{
+    return forward(p, false, twiddle, nullptr, input, output, workspace, workspace_bytes, stream, bias, in_perm,
+                   out_index);
+}
+
+int bf_butterfly_multiply_perm_bw(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
+                                  const int32_t *in_perm, const int32_t *out_index, void *d_twiddle, void *d_input,
+                                  void *d_bias, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (d_bias)
+        return bias_backward(p, twiddle, input, grad, d_twiddle, d_input, d_bias, workspace, workspace_bytes, stream,
+                             in_perm, out_index);
+    return backward(p, false, twiddle, nullptr, input, grad, d_twiddle, nullptr, d_input, workspace, workspace_bytes,
+                    stream, nullptr, nullptr, in_perm, out_index);
 }
 
 int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4, const void *twiddle2,

@@ -79,9 +79,23 @@ bf_problem make_problem(const Shapes &s, const Tensor &input, bool increasing_st
 
 // ---- base-2 -----------------------------------------------------------------------------
 
-// Shared body of butterfly_multiply_fw and butterfly_multiply_bias_fw (`bias` undefined = none).
+// A column table of the *_perm operators: int32, n entries, dense, on the device of `like`.
+// Its entries are the caller's responsibility (each table a permutation of 0..n-1).
+const int32_t *table_ptr(const Tensor &t, Tensor &keep, const Tensor &like, int64_t n, const char *name,
+                         const char *who)
+{
+    if (!t.defined()) return nullptr;
+    TORCH_CHECK(t.device() == like.device(), who, ": ", name, " must be on the device of input");
+    TORCH_CHECK(t.scalar_type() == at::kInt, who, ": ", name, " must be int32");
+    TORCH_CHECK(t.dim() == 1 && t.size(0) == n, who, ": ", name, " must have n entries");
+    keep = t.contiguous();
+    return keep.data_ptr<int32_t>();
+}
+
+// Shared body of the forward operators (`bias`, `in_perm`, `out_index` undefined = none).
 Tensor multiply_fw_impl(const Tensor &twiddle, const Tensor &input, const Tensor &bias, bool increasing_stride,
-                        c10::optional<int64_t> output_size, const char *who)
+                        c10::optional<int64_t> output_size, const char *who, const Tensor &in_perm = Tensor(),
+                        const Tensor &out_index = Tensor())
 {
     CHECK_DEVICE(twiddle); CHECK_DEVICE(input); CHECK_SAME_DEVICE(twiddle, input);
     CHECK_DIM(twiddle, 6); CHECK_DIM(input, 3);
@@ -117,6 +131,17 @@ Tensor multiply_fw_impl(const Tensor &twiddle, const Tensor &input, const Tensor
     set_strides(p.output_stride, output);
     const size_t ws_bytes = bf_butterfly_multiply_fw_workspace_bytes(&p);
     Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+    Tensor keep_in, keep_out;
+    const int32_t *ip = table_ptr(in_perm, keep_in, x, s.n, "in_perm", who);
+    const int32_t *oi = table_ptr(out_index, keep_out, x, s.n, "out_index", who);
+    if (ip || oi) {
+        TORCH_CHECK(s.input_size <= s.n, who, ": column tables need input_size <= n");
+        check_rc(bf_butterfly_multiply_perm_fw(&p, tw.data_ptr(), x.data_ptr(), ip, oi,
+                                               b.defined() ? b.data_ptr() : nullptr, output.data_ptr(),
+                                               ws.data_ptr(), ws_bytes, current_stream()),
+                 who);
+        return output;
+    }
     check_rc(bf_butterfly_multiply_bias_fw(&p, tw.data_ptr(), x.data_ptr(), b.defined() ? b.data_ptr() : nullptr,
                                            output.data_ptr(), ws.data_ptr(), ws_bytes, current_stream()),
              who);
@@ -165,9 +190,11 @@ Tensor butterfly_bias_grad(const Tensor grad)
     return d_bias;
 }
 
-// Shared body of butterfly_multiply_bw and butterfly_multiply_bias_bw.
+// Shared body of the backward operators.
 std::tuple<Tensor, Tensor, Tensor> multiply_bw_impl(const Tensor &twiddle, const Tensor &input, const Tensor &grad,
-                                                    bool increasing_stride, bool with_bias, const char *who)
+                                                    bool increasing_stride, bool with_bias, const char *who,
+                                                    const Tensor &in_perm = Tensor(),
+                                                    const Tensor &out_index = Tensor())
 {
     CHECK_DEVICE(twiddle); CHECK_DEVICE(input); CHECK_DEVICE(grad);
     CHECK_SAME_DEVICE(twiddle, input); CHECK_SAME_DEVICE(input, grad);
@@ -199,7 +226,21 @@ std::tuple<Tensor, Tensor, Tensor> multiply_bw_impl(const Tensor &twiddle, const
     set_strides(p.output_stride, g);
     set_strides(p.d_input_stride, d_input);
     Tensor d_bias;
-    if (with_bias) {
+    Tensor keep_in, keep_out;
+    const int32_t *ip = table_ptr(in_perm, keep_in, x, s.n, "in_perm", who);
+    const int32_t *oi = table_ptr(out_index, keep_out, x, s.n, "out_index", who);
+    if (ip || oi) {
+        TORCH_CHECK(s.input_size <= s.n, who, ": column tables need input_size <= n");
+        if (with_bias) d_bias = at::empty({s.nstacks, output_size}, g.options());
+        const size_t ws_bytes = with_bias ? bf_butterfly_multiply_bias_bw_workspace_bytes(&p)
+                                          : bf_butterfly_multiply_bw_workspace_bytes(&p);
+        Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+        check_rc(bf_butterfly_multiply_perm_bw(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), ip, oi,
+                                               d_twiddle.data_ptr(), d_input.data_ptr(),
+                                               with_bias ? d_bias.data_ptr() : nullptr, ws.data_ptr(), ws_bytes,
+                                               current_stream()),
+                 who);
+    } else if (with_bias) {
         d_bias = at::empty({s.nstacks, output_size}, g.options());
         const size_t ws_bytes = bf_butterfly_multiply_bias_bw_workspace_bytes(&p);
         Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
@@ -282,6 +323,74 @@ Tensor butterfly_multiply_bias(Tensor twiddle, Tensor input, Tensor bias, bool i
                                c10::optional<int64_t> output_size)
 {
     return ButterflyMultiplyBias::apply(twiddle, input, bias, increasing_stride, output_size);
+}
+
+// New operators: the multiply between two fixed column permutations, folded into the first
+// read and the last write (in front: u[c] = input[in_perm[c]]; behind: output[out_index[c]] =
+// y[c]; bias (nstacks, output_size) indexed by c).  Where the reference chains FixedPermutation
+// and Butterfly modules (torch_butterfly/special.py:17-66), each permutation costs a pass of
+// its own over the activations.  Tables: int32 (n,), undefined = identity.
+Tensor opt(const c10::optional<Tensor> &t) { return t.has_value() ? t.value() : Tensor(); }
+
+Tensor butterfly_multiply_perm_fw(const Tensor twiddle, const Tensor input, c10::optional<Tensor> in_perm,
+                                  c10::optional<Tensor> out_index, c10::optional<Tensor> bias,
+                                  bool increasing_stride, c10::optional<int64_t> output_size)
+{
+    return multiply_fw_impl(twiddle, input, opt(bias), increasing_stride, output_size, "butterfly_multiply_perm_fw",
+                            opt(in_perm), opt(out_index));
+}
+
+// (d_twiddle, d_input, d_bias); d_bias is undefined unless with_bias
+std::tuple<Tensor, Tensor, Tensor> butterfly_multiply_perm_bw(const Tensor twiddle, const Tensor input,
+                                                              const Tensor grad, c10::optional<Tensor> in_perm,
+                                                              c10::optional<Tensor> out_index, bool with_bias,
+                                                              bool increasing_stride)
+{
+    auto r = multiply_bw_impl(twiddle, input, grad, increasing_stride, with_bias, "butterfly_multiply_perm_bw",
+                              opt(in_perm), opt(out_index));
+    if (!with_bias) std::get<2>(r) = at::empty({0}, grad.options());  // the schema has no optional results
+    return r;
+}
+
+class ButterflyMultiplyPerm : public torch::autograd::Function<ButterflyMultiplyPerm> {
+public:
+    static Tensor forward(AutogradContext *ctx, Tensor twiddle, Tensor input, c10::optional<Tensor> in_perm,
+                          c10::optional<Tensor> out_index, c10::optional<Tensor> bias, bool increasing_stride,
+                          c10::optional<int64_t> output_size)
+    {
+        ctx->saved_data["increasing_stride"] = increasing_stride;
+        ctx->saved_data["with_bias"] = bias.has_value();
+        ctx->saved_data["has_in"] = in_perm.has_value();
+        ctx->saved_data["has_out"] = out_index.has_value();
+        variable_list saved = {twiddle, input};
+        if (in_perm.has_value()) saved.push_back(in_perm.value());
+        if (out_index.has_value()) saved.push_back(out_index.value());
+        ctx->save_for_backward(saved);
+        return butterfly_multiply_perm_fw(twiddle, input, in_perm, out_index, bias, increasing_stride, output_size);
+    }
+
+    static variable_list backward(AutogradContext *ctx, variable_list grad_output)
+    {
+        const auto saved = ctx->get_saved_variables();
+        const bool has_in = ctx->saved_data["has_in"].toBool(), has_out = ctx->saved_data["has_out"].toBool();
+        c10::optional<Tensor> in_perm, out_index;
+        size_t next = 2;
+        if (has_in) in_perm = saved[next++];
+        if (has_out) out_index = saved[next++];
+        auto r = butterfly_multiply_perm_bw(saved[0], saved[1], grad_output[0], in_perm, out_index,
+                                            ctx->saved_data["with_bias"].toBool(),
+                                            ctx->saved_data["increasing_stride"].toBool());
+        const bool with_bias = ctx->saved_data["with_bias"].toBool();
+        return {std::get<0>(r), std::get<1>(r), Tensor(), Tensor(), with_bias ? std::get<2>(r) : Tensor(), Tensor(),
+                Tensor()};
+    }
+};
+
+Tensor butterfly_multiply_perm(Tensor twiddle, Tensor input, c10::optional<Tensor> in_perm,
+                               c10::optional<Tensor> out_index, c10::optional<Tensor> bias, bool increasing_stride,
+                               c10::optional<int64_t> output_size)
+{
+    return ButterflyMultiplyPerm::apply(twiddle, input, in_perm, out_index, bias, increasing_stride, output_size);
 }
 
 // ---- base-4 -----------------------------------------------------------------------------
@@ -399,6 +508,9 @@ TORCH_LIBRARY(torch_butterfly, m)
     m.def("butterfly_bias_grad", butterfly_bias_grad);
     m.def("butterfly_multiply_bias_bw", butterfly_multiply_bias_bw);
     m.def("butterfly_multiply_bias", butterfly_multiply_bias);
+    m.def("butterfly_multiply_perm_fw", butterfly_multiply_perm_fw);
+    m.def("butterfly_multiply_perm_bw", butterfly_multiply_perm_bw);
+    m.def("butterfly_multiply_perm", butterfly_multiply_perm);
     m.def("butterfly_multiply_base4_fw", butterfly_multiply_base4_fw);
     m.def("butterfly_multiply_base4_bw", butterfly_multiply_base4_bw);
     m.def("butterfly_multiply_base4", butterfly_multiply_base4);

@@ -97,6 +97,16 @@ __host__ __device__ __forceinline__ StageInfo stage_info(const Schedule &sc, int
 struct View {
     int64_t sb, ss, se;
     int64_t width;
+    const int *perm;  // NULL, or n entries: column c of the row as the kernels see it lives in tensor column perm[c]
 };
+
+// Tensor column behind column `col` (< n) of a row as the kernels see it, or -1 when that
+// column does not exist in the tensor (reads give zero, writes are dropped).  The table is a
+// fixed permutation in front of or behind the multiply, folded into the access.
+__device__ __forceinline__ int64_t view_col(const View &v, int64_t col)
+{
+    if (v.perm) col = v.perm[col];
+    return col < v.width ? col : -1;
+}
 
 }  // namespace bf

@@ -418,8 +418,9 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
         make_rsrc(reinterpret_cast<T *>(a.out) + g0 * SLOTS * a.out_view.sb + stack * a.out_view.ss);
     const int in_row = (int)(a.in_view.sb * EB), out_row = (int)(a.out_view.sb * EB);
     // thread-constant part of the offsets; the row group adds a wave-uniform part
-    const int in_thr = col < a.in_view.width ? c.slot * in_row + (int)(col * a.in_view.se * EB) : kOob;
-    const int out_thr = col < a.out_view.width ? c.slot * out_row + (int)(col * a.out_view.se * EB) : kOob;
+    const int64_t in_col = view_col(a.in_view, col), out_col = view_col(a.out_view, col);
+    const int in_thr = in_col >= 0 ? c.slot * in_row + (int)(in_col * a.in_view.se * EB) : kOob;
+    const int out_thr = out_col >= 0 ? c.slot * out_row + (int)(out_col * a.out_view.se * EB) : kOob;
     const T bias = (a.bias && col < a.out_view.width)
                        ? reinterpret_cast<const T *>(a.bias)[stack * a.out_view.width + col]
                        : zero_of(T());
@@ -435,7 +436,8 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     // at the padded word 65 w + l of the group's slot; `set` alternates between iterations
     const BufDesc in_desc = make_desc(in_base);
     const int slot_d = t >> L, col_d = (chunk << L) + (t & (n - 1));
-    const int in_dma = col_d < a.in_view.width ? slot_d * in_row + (int)(col_d * a.in_view.se * EB) : kOob;
+    const int64_t in_col_d = view_col(a.in_view, col_d);
+    const int in_dma = in_col_d >= 0 ? slot_d * in_row + (int)(in_col_d * a.in_view.se * EB) : kOob;
     const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
     auto fetch_row = [&](int grel, int set, int r) {
         const bool ok = (grel + r) * SLOTS + slot_d < rows_valid;
@@ -715,7 +717,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const __amdgpu_buffer_rsrc_t gi_rs =
         make_rsrc(reinterpret_cast<T *>(a.g_in) + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
     const int x_row = (int)(a.x_view.sb * EB), g_row = (int)(a.g_view.sb * EB), gi_row = (int)(a.gi_view.sb * EB);
-    const int gi_thr = col < a.gi_view.width ? c.slot * gi_row + (int)(col * a.gi_view.se * EB) : kOob;
+    const int64_t gi_col = view_col(a.gi_view, col);
+    const int gi_thr = gi_col >= 0 ? c.slot * gi_row + (int)(gi_col * a.gi_view.se * EB) : kOob;
     auto group_ok = [&](int grp) { return grp >= 0 && grp * SLOTS + c.slot < rows_valid; };
     auto store_grad = [&](int grp, T gval) {
         buf_store(gi_rs, group_ok(grp) ? gi_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * gi_row, gval);
@@ -723,8 +726,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 
     // --- operand fetch, register flavour: thread t holds its layout-A element
     const __amdgpu_buffer_rsrc_t x_rs = make_rsrc(x_base), g_rs = make_rsrc(g_base);
-    const int x_thr = col < a.x_view.width ? c.slot * x_row + (int)(col * a.x_view.se * EB) : kOob;
-    const int g_thr = col < a.g_view.width ? c.slot * g_row + (int)(col * a.g_view.se * EB) : kOob;
+    const int64_t x_col = view_col(a.x_view, col), g_col = view_col(a.g_view, col);
+    const int x_thr = x_col >= 0 ? c.slot * x_row + (int)(x_col * a.x_view.se * EB) : kOob;
+    const int g_thr = g_col >= 0 ? c.slot * g_row + (int)(g_col * a.g_view.se * EB) : kOob;
     auto load_x = [&](int grp) {
         return buf_load<T>(x_rs, group_ok(grp) ? x_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row);
     };
@@ -735,8 +739,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // group, which lands at the padded word 65 w + l of the slot
     const BufDesc x_desc = make_desc(x_base), g_desc = make_desc(g_base);
     const int slot_d = t >> L, col_d = (chunk << L) + (t & (n - 1));
-    const int x_dma = col_d < a.x_view.width ? slot_d * x_row + (int)(col_d * a.x_view.se * EB) : kOob;
-    const int g_dma = col_d < a.g_view.width ? slot_d * g_row + (int)(col_d * a.g_view.se * EB) : kOob;
+    const int64_t x_col_d = view_col(a.x_view, col_d), g_col_d = view_col(a.g_view, col_d);
+    const int x_dma = x_col_d >= 0 ? slot_d * x_row + (int)(x_col_d * a.x_view.se * EB) : kOob;
+    const int g_dma = g_col_d >= 0 ? slot_d * g_row + (int)(g_col_d * a.g_view.se * EB) : kOob;
     const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
     auto group_ok_d = [&](int grp) { return grp >= 0 && grp * SLOTS + slot_d < rows_valid; };
     // Iteration j replays the R groups R j .. R j + R - 1 (they sit in x set j & 3) and sweeps

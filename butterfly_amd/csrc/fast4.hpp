@@ -131,8 +131,9 @@ __global__ __launch_bounds__(kFastThreads) void fast4_fw_kernel(Fast4Args a)
     const __amdgpu_buffer_rsrc_t in_rs = make_rsrc(a.x_in + g0 * SLOTS * a.x_view.sb + stack * a.x_view.ss);
     const __amdgpu_buffer_rsrc_t out_rs = make_rsrc(a.x_out + g0 * SLOTS * a.xo_view.sb + stack * a.xo_view.ss);
     const int in_row = (int)(a.x_view.sb * 4), out_row = (int)(a.xo_view.sb * 4);
-    const int in_thr = c.eA < a.x_view.width ? c.slot * in_row + (int)(c.eA * a.x_view.se * 4) : kOob;
-    const int out_thr = c.eA < a.xo_view.width ? c.slot * out_row + (int)(c.eA * a.xo_view.se * 4) : kOob;
+    const int64_t in_col = view_col(a.x_view, c.eA), out_col = view_col(a.xo_view, c.eA);
+    const int in_thr = in_col >= 0 ? c.slot * in_row + (int)(in_col * a.x_view.se * 4) : kOob;
+    const int out_thr = out_col >= 0 ? c.slot * out_row + (int)(out_col * a.xo_view.se * 4) : kOob;
 
     auto load_rows = [&](int grel, float (&v)[R]) {
 #pragma unroll
@@ -208,9 +209,10 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
     const __amdgpu_buffer_rsrc_t g_rs = make_rsrc(a.g_out + g0 * SLOTS * a.g_view.sb + stack * a.g_view.ss);
     const __amdgpu_buffer_rsrc_t gi_rs = make_rsrc(a.g_in + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
     const int x_row = (int)(a.x_view.sb * 4), g_row = (int)(a.g_view.sb * 4), gi_row = (int)(a.gi_view.sb * 4);
-    const int x_thr = c.eA < a.x_view.width ? c.slot * x_row + (int)(c.eA * a.x_view.se * 4) : kOob;
-    const int g_thr = c.eA < a.g_view.width ? c.slot * g_row + (int)(c.eA * a.g_view.se * 4) : kOob;
-    const int gi_thr = c.eA < a.gi_view.width ? c.slot * gi_row + (int)(c.eA * a.gi_view.se * 4) : kOob;
+    const int64_t x_col = view_col(a.x_view, c.eA), g_col = view_col(a.g_view, c.eA), gi_col = view_col(a.gi_view, c.eA);
+    const int x_thr = x_col >= 0 ? c.slot * x_row + (int)(x_col * a.x_view.se * 4) : kOob;
+    const int g_thr = g_col >= 0 ? c.slot * g_row + (int)(g_col * a.g_view.se * 4) : kOob;
+    const int gi_thr = gi_col >= 0 ? c.slot * gi_row + (int)(gi_col * a.gi_view.se * 4) : kOob;
 
     auto transpose = [&](float v, int to_b) -> float {
         const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;

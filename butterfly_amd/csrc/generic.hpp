@@ -90,7 +90,8 @@ __global__ __launch_bounds__(kGenericThreads) void generic_fw_kernel(GenericFwAr
     for (int it = tid; it < (rows << log_n); it += kGenericThreads) {
         const int r = it >> log_n, j = it & (n - 1);
         T v = zero_of(T());
-        if (j < a.in_view.width) v = in[(b0 + r) * a.in_view.sb + s * a.in_view.ss + j * a.in_view.se];
+        const int64_t jc = view_col(a.in_view, j);
+        if (jc >= 0) v = in[(b0 + r) * a.in_view.sb + s * a.in_view.ss + jc * a.in_view.se];
         buf[it] = v;
     }
     for (int t = a.t0; t < a.t1; ++t) {
@@ -108,8 +109,8 @@ __global__ __launch_bounds__(kGenericThreads) void generic_fw_kernel(GenericFwAr
     T *out = reinterpret_cast<T *>(a.out);
     for (int it = tid; it < (rows << log_n); it += kGenericThreads) {
         const int r = it >> log_n, j = it & (n - 1);
-        if (j < a.out_view.width)
-            out[(b0 + r) * a.out_view.sb + s * a.out_view.ss + j * a.out_view.se] = buf[it];
+        const int64_t jc = view_col(a.out_view, j);
+        if (jc >= 0) out[(b0 + r) * a.out_view.sb + s * a.out_view.ss + jc * a.out_view.se] = buf[it];
     }
 }
 
@@ -153,8 +154,9 @@ __global__ __launch_bounds__(kGenericThreads) void generic_bw_kernel(GenericBwAr
     for (int64_t b = blockIdx.x; b < a.batch; b += gridDim.x) {
         for (int j = tid; j < n; j += kGenericThreads) {
             T v = zero_of(T()), gv = zero_of(T());
-            if (j < a.x_view.width) v = x_in[b * a.x_view.sb + s * a.x_view.ss + j * a.x_view.se];
-            if (j < a.g_view.width) gv = g_out[b * a.g_view.sb + s * a.g_view.ss + j * a.g_view.se];
+            const int64_t xc = view_col(a.x_view, j), gc = view_col(a.g_view, j);
+            if (xc >= 0) v = x_in[b * a.x_view.sb + s * a.x_view.ss + xc * a.x_view.se];
+            if (gc >= 0) gv = g_out[b * a.g_view.sb + s * a.g_view.ss + gc * a.g_view.se];
             xs[j] = v;
             g[j] = gv;
         }
@@ -241,9 +243,10 @@ __global__ __launch_bounds__(kGenericThreads) void generic_bw_kernel(GenericBwAr
             }
         }
         __syncthreads();
-        for (int64_t j = tid; j < a.gi_view.width; j += kGenericThreads) {
-            const T v = j < n ? g[j] : zero_of(T());
-            g_in[b * a.gi_view.sb + s * a.gi_view.ss + j * a.gi_view.se] = v;
+        const int64_t jend = a.gi_view.width > n ? a.gi_view.width : n;
+        for (int64_t j = tid; j < jend; j += kGenericThreads) {
+            const int64_t jc = j < n ? view_col(a.gi_view, j) : j;
+            if (jc >= 0) g_in[b * a.gi_view.sb + s * a.gi_view.ss + jc * a.gi_view.se] = j < n ? g[j] : zero_of(T());
         }
         __syncthreads();
         first_row = false;

@@ -87,11 +87,17 @@ __global__ __launch_bounds__(kHighThreads) void high_fw_kernel(HighArgs a)
     const T *in = reinterpret_cast<const T *>(a.x_in) + stack * a.x_view.ss;
     T *out = reinterpret_cast<T *>(a.x_out) + stack * a.xo_view.ss;
 
+    int x_col[E], xo_col[E];  // tensor columns of the thread's elements (-1: none)
+#pragma unroll
+    for (int j = 0; j < E; ++j) {
+        const int col = (j << kHighLowBits) | p;
+        x_col[j] = (int)view_col(a.x_view, col);
+        xo_col[j] = (int)view_col(a.xo_view, col);
+    }
     auto load_row = [&](int64_t row, T (&v)[E]) {
 #pragma unroll
         for (int j = 0; j < E; ++j) {
-            const int col = (j << kHighLowBits) | p;
-            v[j] = (row < r1 && col < a.x_view.width) ? in[row * a.x_view.sb + col * a.x_view.se] : zero_of(T());
+            v[j] = (row < r1 && x_col[j] >= 0) ? in[row * a.x_view.sb + x_col[j] * a.x_view.se] : zero_of(T());
         }
     };
     T nxt[E];
@@ -114,8 +120,7 @@ __global__ __launch_bounds__(kHighThreads) void high_fw_kernel(HighArgs a)
         });
 #pragma unroll
         for (int j = 0; j < E; ++j) {
-            const int col = (j << kHighLowBits) | p;
-            if (col < a.xo_view.width) out[row * a.xo_view.sb + col * a.xo_view.se] = v[j];
+            if (xo_col[j] >= 0) out[row * a.xo_view.sb + xo_col[j] * a.xo_view.se] = v[j];
         }
     }
 }
@@ -170,9 +175,10 @@ __global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
 #pragma unroll
     for (int j = 0; j < E; ++j) {
         const int col = (j << kHighLowBits) | p;
-        x_off[j] = col < a.x_view.width ? (int)(col * a.x_view.se * EB) : kOob;
-        g_off[j] = col < a.g_view.width ? (int)(col * a.g_view.se * EB) : kOob;
-        gi_off[j] = col < a.gi_view.width ? (int)(col * a.gi_view.se * EB) : kOob;
+        const int64_t xc = view_col(a.x_view, col), gc = view_col(a.g_view, col), gic = view_col(a.gi_view, col);
+        x_off[j] = xc >= 0 ? (int)(xc * a.x_view.se * EB) : kOob;
+        g_off[j] = gc >= 0 ? (int)(gc * a.g_view.se * EB) : kOob;
+        gi_off[j] = gic >= 0 ? (int)(gic * a.gi_view.se * EB) : kOob;
     }
     // slot layout, in dwords: [x | g][element j][plane][thread]; a wavefront's 64 lanes are contiguous
     const unsigned wave_addr =

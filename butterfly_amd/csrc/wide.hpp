@@ -117,10 +117,11 @@ __global__ __launch_bounds__(kFastThreads) void wide_fw_kernel(FastFwArgs a)
         bias[q] = (a.bias && col < a.out_view.width)
                       ? reinterpret_cast<const T *>(a.bias)[stack * a.out_view.width + col]
                       : zero_of(T());
-        in_thr[q] = col < a.in_view.width ? (int)(col * a.in_view.se * EB) : kOob;
-        out_thr[q] = col < a.out_view.width ? (int)(col * a.out_view.se * EB) : kOob;
-        const int col_d = (q << 10) | t;
-        in_dma[q] = col_d < a.in_view.width ? (int)(col_d * a.in_view.se * EB) : kOob;
+        const int64_t in_col = view_col(a.in_view, col), out_col = view_col(a.out_view, col);
+        in_thr[q] = in_col >= 0 ? (int)(in_col * a.in_view.se * EB) : kOob;
+        out_thr[q] = out_col >= 0 ? (int)(out_col * a.out_view.se * EB) : kOob;
+        const int64_t in_col_d = view_col(a.in_view, (q << 10) | t);
+        in_dma[q] = in_col_d >= 0 ? (int)(in_col_d * a.in_view.se * EB) : kOob;
     }
     const BufDesc in_desc = make_desc(in_base);
     const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;

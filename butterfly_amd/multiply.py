@@ -39,6 +39,19 @@ def butterfly_multiply_bias(twiddle: torch.Tensor, input: torch.Tensor, bias: to
                                                              output_size)
 
 
+def butterfly_multiply_perm(twiddle: torch.Tensor, input: torch.Tensor, in_perm: Optional[torch.Tensor],
+                            out_index: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+                            increasing_stride: bool, output_size: Optional[int] = None) -> torch.Tensor:
+    """The multiply between two fixed column permutations that the kernels fold into their
+    first read and last write: u[..., c] = input[..., in_perm[c]], y = multiply(u) + bias,
+    output[..., out_index[c]] = y[..., c].  Tables are int32 of n entries (None = identity); a
+    FixedPermutation(q) behind the layer is out_index = inverse of q.  Differentiable in
+    twiddle, input and bias.  The reference runs each permutation as a separate gather
+    (torch_butterfly/permutation.py:55-78)."""
+    return torch.ops.torch_butterfly.butterfly_multiply_perm(twiddle, input, in_perm, out_index, bias,
+                                                             increasing_stride, output_size)
+
+
 def fit_last_dim(x: torch.Tensor, n: int) -> torch.Tensor:
     """Zero-pad or trim the last dimension to exactly ``n``."""
     size = x.shape[-1]

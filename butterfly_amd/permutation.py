@@ -1,5 +1,6 @@
-"""Fixed permutations on the multiply path: the FFT bit reversal and a module that applies a
-stored permutation (reference: torch_butterfly/permutation.py:14-30,55-78)."""
+"""Fixed permutations on the multiply path: the FFT bit reversal, a module that applies a
+stored permutation (reference: torch_butterfly/permutation.py:14-30,55-78) and a Sequential
+that folds such modules into the neighbouring Butterfly's kernels."""
 import numpy as np
 import torch
 from torch import nn
@@ -36,9 +37,66 @@ class FixedPermutation(nn.Module):
     def __init__(self, permutation: torch.Tensor) -> None:
         super().__init__()
         self.register_buffer("permutation", permutation)
+        self._tables = {}
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         return index_last_dim(input, self.permutation)
+
+    def column_table(self, n: int, scatter: bool) -> torch.Tensor:
+        """The permutation as the int32 table of n entries that the multiply operators fold
+        into their first read (scatter False: entry c = permutation[c]) or their last write
+        (scatter True: the inverse, entry permutation[i] = i); entries past the permutation's
+        length are fixed points.  Cached until the buffer changes."""
+        p = self.permutation
+        key = (n, scatter, p.device, p.data_ptr(), p._version)
+        table = self._tables.get(key)
+        if table is None:
+            if p.dim() != 1 or p.numel() > n:
+                raise ValueError("the permutation must be a vector of at most n entries")
+            full = torch.arange(n, dtype=torch.int64, device=p.device)
+            full[:p.numel()] = p
+            table = (invert(full) if scatter else full).to(torch.int32)
+            if len(self._tables) >= 4:
+                self._tables.clear()
+            self._tables[key] = table
+        return table
+
+
+class FusedSequential(nn.Sequential):
+    """nn.Sequential (same children, indexing and state) whose forward folds a
+    FixedPermutation standing directly in front of or behind a Butterfly into that layer's
+    kernels, so it costs no pass of its own over the activations.  Any other sequence of
+    children runs one after the other as usual."""
+
+    def forward(self, input):
+        from .butterfly import Butterfly, ButterflyBmm  # (butterfly.py does not import this module)
+        mods = list(self)
+
+        def is_layer(m):
+            return isinstance(m, Butterfly) and not isinstance(m, ButterflyBmm)
+
+        i = 0
+        while i < len(mods):
+            m = mods[i]
+            front = None
+            if (isinstance(m, FixedPermutation) and i + 1 < len(mods) and is_layer(mods[i + 1])
+                    and m.permutation.dim() == 1 and m.permutation.numel() == mods[i + 1].in_size
+                    and input.is_cuda):
+                front, m = m, mods[i + 1]
+                i += 1
+            if is_layer(m) and input.is_cuda:
+                back = None
+                if (i + 1 < len(mods) and isinstance(mods[i + 1], FixedPermutation) and m.nstacks == 1
+                        and mods[i + 1].permutation.dim() == 1 and mods[i + 1].permutation.numel() == m.out_size):
+                    back = mods[i + 1]
+                    i += 1
+                n = 1 << m.log_n
+                input = m(input, in_perm=None if front is None else front.column_table(n, False),
+                          out_index=None if back is None else back.column_table(n, True))
+            else:
+                input = m(input)
+            i += 1
+        return input
 
 
 def wavelet_permutation(n, pytorch_format=False):

@@ -16,7 +16,7 @@ from .combine import (TensorProduct, butterfly_kronecker, butterfly_product, dia
                       permutation_kronecker)
 from .complex_utils import Complex2Real, Real2Complex, index_last_dim, real2complex
 from .diagonal import Diagonal
-from .permutation import FixedPermutation, bitreversal_permutation, invert, wavelet_permutation
+from .permutation import FixedPermutation, FusedSequential, bitreversal_permutation, invert, wavelet_permutation
 
 
 def _log2_exact(n):
@@ -50,7 +50,7 @@ def _fourier(n, sign, scale, br_first, with_br_perm):
     if not with_br_perm:
         return b
     perm = FixedPermutation(bitreversal_permutation(n, pytorch_format=True))
-    return nn.Sequential(perm, b) if br_first else nn.Sequential(b, perm)
+    return FusedSequential(perm, b) if br_first else FusedSequential(b, perm)
 
 
 def fft(n, normalized=False, br_first=True, with_br_perm=True) -> nn.Module:
@@ -104,13 +104,13 @@ def circulant(col, transposed=False, separate_diagonal=True) -> nn.Module:
     diag = index_last_dim(eig, br)
     if separate_diagonal:
         core = [b_fft, Diagonal(diagonal_init=diag), b_ifft]
-        return nn.Sequential(*core) if was_complex else nn.Sequential(Real2Complex(), *core, Complex2Real())
+        return FusedSequential(*core) if was_complex else FusedSequential(Real2Complex(), *core, Complex2Real())
     with torch.no_grad():
         b_fft = diagonal_butterfly(b_fft, diag, diag_first=False, inplace=True)
     b = butterfly_product(b_fft, b_ifft)
     b.in_size = n
     b.out_size = n
-    return b if was_complex else nn.Sequential(Real2Complex(), b, Complex2Real())
+    return b if was_complex else FusedSequential(Real2Complex(), b, Complex2Real())
 
 
 def toeplitz(col, row=None, separate_diagonal=True) -> nn.Module:
@@ -163,7 +163,7 @@ def _fourier_unitary(n, sign, br_first, with_br_perm):
     if not with_br_perm:
         return b
     perm = FixedPermutation(bitreversal_permutation(n, pytorch_format=True))
-    return nn.Sequential(perm, b) if br_first else nn.Sequential(b, perm)
+    return FusedSequential(perm, b) if br_first else FusedSequential(b, perm)
 
 
 def fft_unitary(n, br_first=True, with_br_perm=True) -> nn.Module:
@@ -215,7 +215,7 @@ def _trig_type24(n, sine, shift, normalized):
     if sine or shift != 0:
         b = diagonal_butterfly(b, pre[br], diag_first=True)
     b = diagonal_butterfly(b, post, diag_first=False)
-    return nn.Sequential(FixedPermutation(perm[br]), Real2Complex(), b, Complex2Real())
+    return FusedSequential(FixedPermutation(perm[br]), Real2Complex(), b, Complex2Real())
 
 
 def dct(n: int, type: int = 2, normalized: bool = False) -> nn.Module:
@@ -242,7 +242,7 @@ def dct(n: int, type: int = 2, normalized: bool = False) -> nn.Module:
     # the decreasing-stride butterfly leaves v bit-reversed; y = v[inverse of the even/odd order]
     br = bitreversal_permutation(n, pytorch_format=True)
     gather = br[invert(_even_then_reversed_odd(n))]
-    return nn.Sequential(Real2Complex(), b, Complex2Real(), FixedPermutation(gather))
+    return FusedSequential(Real2Complex(), b, Complex2Real(), FixedPermutation(gather))
 
 
 def dst(n: int, type: int = 2, normalized: bool = False) -> nn.Module:
@@ -271,7 +271,7 @@ def hadamard_diagonal(diagonals: torch.Tensor, normalized: bool = False, increas
             parts += [Diagonal(diagonal_init=d), h]
         else:
             parts.append(diagonal_butterfly(h, d, diag_first=True))
-    return nn.Sequential(*parts) if separate_diagonal else reduce(butterfly_product, parts)
+    return FusedSequential(*parts) if separate_diagonal else reduce(butterfly_product, parts)
 
 
 def fastfood(diag1: torch.Tensor, diag2: torch.Tensor, diag3: torch.Tensor, permutation: torch.Tensor,
@@ -285,11 +285,11 @@ def fastfood(diag1: torch.Tensor, diag2: torch.Tensor, diag3: torch.Tensor, perm
     h1 = hadamard(n, normalized, increasing_stride).to(diag1.device)
     h2 = hadamard(n, normalized, not increasing_stride).to(diag1.device)
     if separate_diagonal:
-        return nn.Sequential(Diagonal(diagonal_init=diag1), h1, FixedPermutation(permutation),
+        return FusedSequential(Diagonal(diagonal_init=diag1), h1, FixedPermutation(permutation),
                              Diagonal(diagonal_init=diag2), h2, Diagonal(diagonal_init=diag3))
     h1 = diagonal_butterfly(h1, diag1, diag_first=True)
     h2 = diagonal_butterfly(diagonal_butterfly(h2, diag2, diag_first=True), diag3, diag_first=False)
-    return nn.Sequential(h1, FixedPermutation(permutation), h2)
+    return FusedSequential(h1, FixedPermutation(permutation), h2)
 
 
 def acdc(diag1: torch.Tensor, diag2: torch.Tensor, dct_first: bool = True,
@@ -305,7 +305,7 @@ def acdc(diag1: torch.Tensor, diag2: torch.Tensor, dct_first: bool = True,
     first = dct(n, type=2 if dct_first else 3, normalized=True).to(diag1.device)
     second = dct(n, type=3 if dct_first else 2, normalized=True).to(diag1.device)
     if separate_diagonal:
-        return nn.Sequential(*first, Diagonal(diagonal_init=diag1), *second, Diagonal(diagonal_init=diag2))
+        return FusedSequential(*first, Diagonal(diagonal_init=diag1), *second, Diagonal(diagonal_init=diag2))
     if dct_first:
         # type II ends [.., butterfly, Complex2Real]; type III ends [.., Complex2Real, permutation]:
         # D1 scales the rows of the first butterfly; D2, moved in front of the closing gather
@@ -315,13 +315,13 @@ def acdc(diag1: torch.Tensor, diag2: torch.Tensor, dct_first: bool = True,
         b1 = diagonal_butterfly(b1, diag1.to(b1.twiddle.dtype), diag_first=False)
         moved = diag2[invert(gather.permutation)]
         b2 = diagonal_butterfly(b2, moved.to(b2.twiddle.dtype), diag_first=False)
-        return nn.Sequential(perm, r2c, b1, c2r, r2c2, b2, c2r2, gather)
+        return FusedSequential(perm, r2c, b1, c2r, r2c2, b2, c2r2, gather)
     r2c, b1, c2r, gather = first
     perm, r2c2, b2, c2r2 = second
     moved = diag1[invert(gather.permutation)]
     b1 = diagonal_butterfly(b1, moved.to(b1.twiddle.dtype), diag_first=False)
     b2 = diagonal_butterfly(b2, diag2.to(b2.twiddle.dtype), diag_first=False)
-    return nn.Sequential(r2c, b1, c2r, gather, perm, r2c2, b2, c2r2)
+    return FusedSequential(r2c, b1, c2r, gather, perm, r2c2, b2, c2r2)
 
 
 # ---- circular convolutions ----------------------------------------------------------------------
@@ -398,7 +398,7 @@ def conv1d_circular_multichannel(n, weight) -> nn.Module:
     eig = torch.fft.fft(col, norm=None)   # eigenvalues of the circulants (unnormalised on purpose)
     eig = index_last_dim(eig, bitreversal_permutation(n_ext, pytorch_format=True).to(col.device))
     core = [b_fft, DiagonalMultiplySum(eig), b_ifft]
-    return nn.Sequential(*core) if was_complex else nn.Sequential(Real2Complex(), *core, Complex2Real())
+    return FusedSequential(*core) if was_complex else FusedSequential(Real2Complex(), *core, Complex2Real())
 
 
 # ---- two-dimensional Fourier transforms and convolutions ---------------------------------------------
@@ -416,8 +416,8 @@ def _fourier2d(make, n1, n2, br_first, with_br_perm, flatten, **kwargs):
         perm = permutation_kronecker(p1, p2) if flatten else TensorProduct(p1, p2)
         parts = [perm, b] if br_first else [b, perm]
     if flatten:
-        return nn.Sequential(nn.Flatten(start_dim=-2), *parts, nn.Unflatten(-1, (n2, n1)))
-    return parts[0] if len(parts) == 1 else nn.Sequential(*parts)
+        return FusedSequential(nn.Flatten(start_dim=-2), *parts, nn.Unflatten(-1, (n2, n1)))
+    return parts[0] if len(parts) == 1 else FusedSequential(*parts)
 
 
 def fft2d(n1: int, n2: int, normalized: bool = False, br_first: bool = True, with_br_perm: bool = True,
@@ -473,7 +473,7 @@ def conv2d_circular_multichannel(n1: int, n2: int, weight: torch.Tensor, flatten
         core = [nn.Flatten(start_dim=-2), b_fft, DiagonalMultiplySum(eig), b_ifft, nn.Unflatten(-1, (n2, n1))]
     else:
         core = [b_fft, DiagonalMultiplySum(eig), b_ifft]
-    return nn.Sequential(*core) if was_complex else nn.Sequential(Real2Complex(), *core, Complex2Real())
+    return FusedSequential(*core) if was_complex else FusedSequential(Real2Complex(), *core, Complex2Real())
 
 
 # ---- Haar wavelet ----------------------------------------------------------------------------------
@@ -494,4 +494,4 @@ def wavelet_haar(n, with_perm=True) -> nn.Module:
     b = Butterfly(n, n, bias=False, increasing_stride=True, init=torch.stack(stages).reshape(1, 1, log_n, n // 2, 2, 2))
     if not with_perm:
         return b
-    return nn.Sequential(b, FixedPermutation(wavelet_permutation(n, pytorch_format=True)))
+    return FusedSequential(b, FixedPermutation(wavelet_permutation(n, pytorch_format=True)))

@@ -114,6 +114,32 @@ int bf_butterfly_multiply_bias_bw(const bf_problem *p, const void *twiddle, cons
 
 size_t bf_butterfly_multiply_bias_bw_workspace_bytes(const bf_problem *p);
 
+/* Forward multiply between two fixed permutations of the columns, folded into the first read
+ * and the last write of the schedule instead of running as gathers of their own:
+ *   u[c]                 = pad(input)[in_perm[c]]   (in_perm NULL: u = pad(input))
+ *   y                    = multiply(u) + bias       (bias (S, O) dense, indexed by c; NULL: none)
+ *   output[out_index[c]] = y[c]                     (out_index NULL: output[c] = y[c];
+ *                                                    entries >= output_size are dropped)
+ * in_perm, out_index: device tables of n 32-bit entries, each a permutation of 0..n-1;
+ * input_size <= n.  A FixedPermutation(q) module behind the layer, out[i] = y[q[i]], is
+ * out_index = inverse of q.  Stands where FixedPermutation runs next to Butterfly as a
+ * separate pass over the activations (torch_butterfly/permutation.py:55-78, as built by
+ * torch_butterfly/special.py:17-66 for the FFT).  Workspace as for bf_butterfly_multiply_fw. */
+int bf_butterfly_multiply_perm_fw(const bf_problem *p, const void *twiddle, const void *input,
+                                  const int32_t *in_perm, const int32_t *out_index,
+                                  const void *bias, void *output, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
+/* Backward of bf_butterfly_multiply_perm_fw: grad is read through out_index, input through
+ * in_perm, and d_input[in_perm[c]] receives the gradient of u[c].  d_bias (S, O) may be NULL.
+ * Workspace: bf_butterfly_multiply_bias_bw_workspace_bytes when d_bias is given, otherwise
+ * bf_butterfly_multiply_bw_workspace_bytes.                                               */
+int bf_butterfly_multiply_perm_bw(const bf_problem *p, const void *twiddle, const void *input,
+                                  const void *grad, const int32_t *in_perm,
+                                  const int32_t *out_index, void *d_twiddle, void *d_input,
+                                  void *d_bias, void *workspace, size_t workspace_bytes,
+                                  void *stream);
+
 /* Base-4 forward: per block log_n/2 radix-4 stages from twiddle4
  * (S, nb, log_n/2, n/4, 4, 4), then one 2x2 stage from twiddle2 (S, nb, 1, n/2, 2, 2)
  * when log_n is odd (twiddle2 may be NULL when log_n is even).

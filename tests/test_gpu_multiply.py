@@ -423,6 +423,123 @@ def test_bias_operator_autograd():
         ops.butterfly_multiply_bias_fw(tw.detach(), x.detach(), bias.detach()[:, :-1], True, None)
 
 
+PERM_CASES = [
+    # dtype, B, S, L, nb, I, O, inc, tables ("io" = both, "i", "o"), bias -- every kind of first
+    # and last pass: register and LDS row fetch, wide, high-bit, generic; padded inputs,
+    # trimmed outputs, several stacks
+    (np.float32, 37, 1, 5, 2, 20, 27, True, "io", True),
+    (np.float32, 300, 1, 10, 2, None, None, False, "io", True),
+    (np.float32, 41, 3, 7, 1, 100, None, True, "i", True),
+    (np.float32, 2100, 1, 10, 1, None, 1000, True, "io", False),
+    (np.complex64, 29, 1, 6, 3, None, 50, False, "io", True),
+    (np.complex64, 530, 1, 10, 1, None, None, True, "io", False),
+    (np.complex64, 130, 2, 9, 2, None, None, False, "i", False),
+    (np.float32, 19, 1, 11, 2, None, 2000, False, "io", True),
+    (np.float32, 23, 1, 12, 1, 4000, None, True, "io", False),
+    (np.complex64, 17, 1, 11, 1, None, None, True, "io", True),
+    (np.complex64, 9, 1, 12, 1, None, 4000, True, "o", False),
+    (np.float32, 11, 1, 13, 1, None, 8000, True, "io", True),
+    (np.float32, 7, 1, 14, 2, 16000, None, False, "io", False),
+]
+
+
+@pytest.mark.parametrize("case", PERM_CASES, ids=lambda c: f"{np.dtype(c[0]).name}-B{c[1]}-S{c[2]}-L{c[3]}-nb{c[4]}-I{c[5]}-O{c[6]}-inc{int(c[7])}-{c[8]}-bias{int(c[9])}")
+def test_permutations_folded_into_first_read_and_last_write(case):
+    """multiply_perm_fw / _bw through the C ABI against the oracle applied between explicit
+    gathers: u = pad(x)[in_perm], y = B u + bias, out[out_index[c]] = y[c]."""
+    from butterfly_amd import _capi
+    dtype, B, S, L, nb, I, O, inc, which, with_bias = case
+    say("perm case", case)
+    n = 1 << L
+    rng = np.random.default_rng(2300 + L * 23 + nb)
+    tw, x, g = make_case(rng, dtype, B, S, L, nb, I, O)
+    cols = n if O is None else O
+    width = n if I is None else I
+    # in front: a permutation of the `width` input columns, fixed points on the padding;
+    # behind: a permutation of the `cols` output columns
+    in_perm = np.arange(n)
+    in_perm[:width] = rng.permutation(width)
+    q = np.arange(n)
+    q[:cols] = rng.permutation(cols)          # FixedPermutation(q): out[i] = y[q[i]]
+    out_index = np.empty(n, dtype=np.int64)
+    out_index[q] = np.arange(n)
+    use_in, use_out = "i" in which, "o" in which
+    bias = randn(rng, (S, cols), dtype) if with_bias else None
+
+    xp = np.zeros((B, S, n), dtype=dtype)
+    xp[:, :, :width] = x
+    u = xp[:, :, in_perm] if use_in else xp
+    y_ref = oracle.butterfly_fw(tw, u, inc, O)
+    if with_bias:
+        y_ref = y_ref + bias[None]
+    out_ref = y_ref[:, :, q[:cols]] if use_out else y_ref
+    gy = np.zeros((B, S, n), dtype=dtype)
+    if use_out:
+        gy[:, :, q[:cols]] = g               # y[q[i]] receives grad[i]
+    else:
+        gy[:, :, :cols] = g
+    dtw_ref, du_ref = oracle.butterfly_bw(tw, u, gy[:, :, :cols], inc)
+    dx_ref = np.zeros((B, S, n), dtype=du_ref.dtype)
+    if use_in:
+        dx_ref[:, :, in_perm] = du_ref
+    else:
+        dx_ref = du_ref
+    dx_ref = dx_ref[:, :, :width]
+    db_ref = gy[:, :, :cols].astype(np.complex128 if np.iscomplexobj(g) else np.float64).sum(axis=0)
+
+    t_in = torch.from_numpy(in_perm.astype(np.int32)).cuda() if use_in else None
+    t_out = torch.from_numpy(out_index.astype(np.int32)).cuda() if use_out else None
+    xd, gd, twd = dev(x), dev(g), dev(tw)
+    out = _capi.multiply_perm_fw(twd, xd, t_in, t_out, None if bias is None else dev(bias), inc, O)
+    dtw, dx, db = _capi.multiply_perm_bw(twd, xd, gd, t_in, t_out, inc, with_bias)
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu().numpy(), out_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+    if with_bias:
+        assert rel_err(db.cpu().numpy(), db_ref) < BW_TOL
+    # identity tables change nothing, bit for bit
+    eye = torch.arange(n, dtype=torch.int32).cuda()
+    plain = _capi.multiply_fw(twd, xd, inc, O)
+    same = _capi.multiply_perm_fw(twd, xd, eye, eye, None, inc, O)
+    torch.cuda.synchronize()
+    assert torch.equal(plain, same)
+
+
+def test_perm_operator_autograd_and_checks():
+    """The autograd operator equals gather -> multiply -> + bias -> gather under autograd."""
+    import butterfly_amd  # noqa: F401
+    ops = torch.ops.torch_butterfly
+    torch.manual_seed(9)
+    for dtype, S, L, nb, O, with_bias in [(torch.float32, 1, 6, 2, 50, True), (torch.complex64, 1, 10, 1, None, False),
+                                          (torch.float32, 1, 12, 2, None, True)]:
+        n = 1 << L
+        cols = n if O is None else O
+        tw = (torch.randn(S, nb, L, n // 2, 2, 2, dtype=dtype) / 2 ** 0.5).cuda().requires_grad_()
+        x = torch.randn(21, S, n, dtype=dtype).cuda().requires_grad_()
+        bias = torch.randn(S, cols, dtype=dtype).cuda().requires_grad_() if with_bias else None
+        g = torch.randn(21, S, cols, dtype=dtype).cuda()
+        p_in = torch.randperm(n).cuda()
+        q = torch.randperm(cols).cuda()
+        full_q = torch.cat((q, torch.arange(cols, n).cuda()))
+        out_index = torch.empty_like(full_q)
+        out_index[full_q] = torch.arange(n).cuda()
+        y = ops.butterfly_multiply_perm(tw, x, p_in.int(), out_index.int(), bias, True, O)
+        wrt = (tw, x) + ((bias,) if with_bias else ())
+        got = torch.autograd.grad(y, wrt, g)
+        y2 = ops.butterfly_multiply(tw, x[..., p_in], True, O)
+        if with_bias:
+            y2 = y2 + bias
+        y2 = y2[..., q]
+        want = torch.autograd.grad(y2, wrt, g)
+        for a, b in [(y, y2)] + list(zip(got, want)):
+            assert (a - b).abs().max().item() <= 1e-4 * max(1.0, b.abs().max().item())
+    with pytest.raises(RuntimeError, match="int32"):
+        ops.butterfly_multiply_perm_fw(tw.detach(), x.detach(), p_in, None, None, True, None)
+    with pytest.raises(RuntimeError, match="n entries"):
+        ops.butterfly_multiply_perm_fw(tw.detach(), x.detach(), p_in.int()[:-1], None, None, True, None)
+
+
 @pytest.mark.parametrize("shape", [(600, 1, 10, 2, False), (300, 1, 12, 2, True), (100, 2, 11, 1, False)],
                          ids=lambda s: f"B{s[0]}-S{s[1]}-L{s[2]}-nb{s[3]}")
 def test_library_calls_replay_from_a_captured_graph(shape):

@@ -236,3 +236,58 @@ def test_kop2d_fft_init_is_a_circular_convolution():
     y = kop(torch.randn(4, 2, 16, 16, device="cuda"))
     y.square().mean().backward()
     assert kop.weight.grad is not None and all(p.grad is not None for p in kop.parameters())
+
+
+def test_fused_sequential_equals_separate_permutations():
+    """FusedSequential (permutations applied by the Butterfly's kernels) against the same
+    children run one after the other, forward and gradients, and against torch.fft."""
+    from torch import nn
+    from butterfly_amd import Butterfly, special, combine
+    from butterfly_amd.permutation import FixedPermutation, FusedSequential
+    torch.manual_seed(3)
+
+    def compare(fused, x, with_params=True):
+        plain = nn.Sequential(*fused)
+        assert isinstance(fused, FusedSequential)
+        xa = x.clone().requires_grad_()
+        xb = x.clone().requires_grad_()
+        ya, yb = fused(xa), plain(xb)
+        assert close(ya, yb)
+        g = torch.randn_like(ya)
+        params = [p for p in fused.parameters()] if with_params else []
+        ga = torch.autograd.grad(ya, [xa] + params, g)
+        gb = torch.autograd.grad(yb, [xb] + params, g)
+        for a, b in zip(ga, gb):
+            assert close(a, b, rtol=1e-3, atol=1e-3)
+        return ya
+
+    for n in (8, 256, 1024, 2048):
+        x = crand(33, n)
+        for br_first in (True, False):
+            say("fused fft", n, br_first)
+            y = compare(special.fft(n, br_first=br_first).cuda(), x)
+            assert close(y, torch.fft.fft(x), rtol=1e-3, atol=1e-3 * math.sqrt(n))
+    say("fused wavelet")
+    compare(special.wavelet_haar(64).cuda(), torch.randn(9, 64, device="cuda"))
+    say("fused flip")
+    b = Butterfly(128, 128, bias=False, increasing_stride=True).cuda()
+    flipped = combine.flip_increasing_stride(b).cuda()
+    xr = torch.randn(12, 128, device="cuda")
+    assert close(compare(flipped, xr), b(xr))
+    say("fused, several stacks, bias, odd sizes")
+    layer = Butterfly(100, 300, bias=True).cuda()      # n = 128, 3 stacks: only the front folds
+    seq = FusedSequential(FixedPermutation(torch.randperm(100)), layer, FixedPermutation(torch.randperm(300))).cuda()
+    compare(seq, torch.randn(7, 100, device="cuda"))
+    layer = Butterfly(100, 90, bias=True, nblocks=2).cuda()   # one stack: both fold, trimmed output
+    seq = FusedSequential(FixedPermutation(torch.randperm(100)), layer, FixedPermutation(torch.randperm(90))).cuda()
+    compare(seq, torch.randn(7, 100, device="cuda"))
+    say("transpose swaps the tables")
+    p_in, q = torch.randperm(128).cuda(), torch.randperm(128).cuda()
+    sq = Butterfly(128, 128, bias=False, complex=True).cuda()
+    fp, fq = FixedPermutation(p_in), FixedPermutation(q)
+    xc = crand(5, 128)
+    # matrix M = Q B P (P, Q the gathers); M^T x = P^T B^T Q^T x
+    eye = torch.eye(128, dtype=torch.complex64, device="cuda")
+    M = fq(sq(fp(eye))).T                          # columns M e_j
+    got = sq(xc, transpose=True, in_perm=fp.column_table(128, False), out_index=fq.column_table(128, True))
+    assert close(got, xc @ M, rtol=1e-3, atol=1e-3)
