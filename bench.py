@@ -78,6 +78,12 @@ CONFIGS = {
                       metric="special.fft(4096) module fwd+bwd GB/s, bit reversal as a separate gather",
                       workload="cfg3 (module level, unfused): the same two modules run one after the other "
                                "(PyTorch gather, then butterfly_multiply); for comparison with cfg3m"),
+    "legacy": dict(batch=2048, nstacks=1, log_n=9, nblocks=1, inc=True, cplx=False, base4=False, bw=True,
+                   cpu_batch=2048, module="legacy",
+                   metric="legacy butterfly.Butterfly(512, 512, tied_weight=False) fwd+bwd GB/s, batch 2048 fp32",
+                   workload="legacy API at the shape of the reference's butterfly/benchmark.py:10-16: "
+                            "Butterfly(512, 512, bias=False, tied_weight=False) (fast-format twiddle (1,9,2,512)), "
+                            "input (2048,512) fp32, forward + autograd backward (d_input, d_twiddle)"),
 }
 
 
@@ -170,6 +176,7 @@ def main():
     ap.add_argument("--config", default="cfg2", choices=sorted(CONFIGS))
     ap.add_argument("--shape", default=None, metavar="B,S,LOG_N,NBLOCKS,f32|c64[,inc|dec]",
                     help="forward + backward at an arbitrary shape instead of a named configuration")
+    ap.add_argument("--batch", type=int, default=None, help="run the configuration at another batch size")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of the input (a kernel of known traffic, for scaling "
@@ -190,6 +197,11 @@ def main():
                         f"{'complex64' if cplx else 'fp32'}",
                  workload=f"shape: butterfly_multiply fw+bw, input ({B},{S},{1 << L}) {'complex64' if cplx else 'fp32'} "
                           f"N(0,1), twiddle ({S},{nb},{L},{(1 << L) // 2},2,2) N(0,1/2), increasing_stride={inc}")
+
+    if args.batch is not None:
+        c = dict(c, batch=args.batch, cpu_batch=min(c["cpu_batch"], args.batch),
+                 metric=c["metric"] + f" [batch overridden: {args.batch}]",
+                 workload=c["workload"] + f" [batch overridden: {args.batch}]")
 
     import torch
     import butterfly_amd
@@ -213,6 +225,16 @@ def main():
         def fw_call():
             state["y"] = layer(xm)
         bw_call = lambda: torch.autograd.grad(state["y"], (xm, layer[1].twiddle), gm)
+    elif c.get("module") == "legacy":
+        from butterfly_amd import legacy
+        layer = legacy.Butterfly(1 << c["log_n"], 1 << c["log_n"], bias=False, tied_weight=False).to(dev)
+        xm = x.reshape(c["batch"], -1).requires_grad_()
+        gm = grad.reshape(c["batch"], -1)
+        state = {}
+
+        def fw_call():
+            state["y"] = layer(xm)
+        bw_call = lambda: torch.autograd.grad(state["y"], (xm, layer.twiddle), gm)
     elif c.get("module"):
         # module level: the layer's forward, then autograd for all three gradients
         layer = butterfly_amd.Butterfly(1 << c["log_n"], 1 << c["log_n"], bias=True, init="ortho",

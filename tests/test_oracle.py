@@ -248,3 +248,175 @@ def test_base4_backward_adjoint_and_finite_differences(dtype):
                 lhs = np.sum((ye - y) * np.conj(g))
                 # d = sum g conj(dy/dt)  =>  sum dy conj(g) = conj(d)
                 assert abs(lhs - np.conj(d.reshape(-1)[j])) < 1e-8 * max(1.0, abs(lhs))
+
+
+# ---- legacy package oracle (oracle/legacy_oracle.py) ---------------------------------------------
+
+from oracle import legacy_oracle as lo  # noqa: E402
+
+
+def _rand(rng, shape, cplx):
+    a = rng.standard_normal(shape)
+    return a + 1j * rng.standard_normal(shape) if cplx else a
+
+
+@pytest.mark.parametrize("cplx", [False, True])
+def test_legacy_factor_against_dense_matrix(cplx):
+    """Each factor equals the n x n matrix written entry by entry from the pairing rule."""
+    rng = np.random.default_rng(11)
+    S, n, B = 2, 16, 3
+    for ls in range(4):
+        st = 1 << ls
+        T = _rand(rng, (S, n // 2, 2, 2), cplx)
+        x = _rand(rng, (B, S, n), cplx)
+        y = lo.factor_apply(T, ls, x)
+        for s in range(S):
+            M = np.zeros((n, n), dtype=T.dtype)
+            for i in range(n // 2):
+                low = i % st
+                p = (2 * (i // st) * st + low, 2 * (i // st) * st + low + st)
+                for r in range(2):
+                    for c in range(2):
+                        M[p[r], p[c]] = T[s, i, r, c]
+            assert np.allclose(y[:, s], x[:, s] @ M.T, rtol=1e-12, atol=1e-12)
+
+
+def _bitrev(n):
+    m = n.bit_length() - 1
+    return np.array([int(format(i, f"0{m}b")[::-1], 2) for i in range(n)])
+
+
+def test_legacy_tied_and_untied_products_are_the_fft():
+    """Decimation in time: increasing stride on bit-reversed input with [[1, w], [1, -w]];
+    decimation in frequency: decreasing stride with [[1, 1], [w, -w]] and bit-reversed output.
+    Neither 2x2 is symmetric and w depends on the position inside the group."""
+    rng = np.random.default_rng(12)
+    n, B = 32, 4
+    x = _rand(rng, (B, 1, n), True)
+    ref = np.fft.fft(x, axis=-1)
+    br = _bitrev(n)
+    tied_dit = np.zeros((1, n - 1, 2, 2), dtype=complex)
+    tied_dif = np.zeros((1, n - 1, 2, 2), dtype=complex)
+    for ls in range(5):
+        st = 1 << ls
+        for low in range(st):
+            w = np.exp(-2j * np.pi * low / (2 * st))
+            tied_dit[0, st - 1 + low] = [[1, w], [1, -w]]
+            tied_dif[0, st - 1 + low] = [[1, 1], [w, -w]]
+    assert np.allclose(lo.butterfly_mult(tied_dit, x[..., br], True), ref)
+    assert np.allclose(lo.butterfly_mult(tied_dif, x, False)[..., br], ref)
+    untied = np.stack([lo.tied_expand(tied_dit, ls, n) for ls in range(5)], axis=1)
+    assert np.allclose(lo.butterfly_mult_untied(untied, x[..., br], True), ref)
+    untied = np.stack([lo.tied_expand(tied_dif, ls, n) for ls in range(5)], axis=1)
+    assert np.allclose(lo.butterfly_mult_untied(untied, x, False)[..., br], ref)
+
+
+def test_legacy_rotation_sign_and_orthogonality():
+    theta = np.array([[0.3]])
+    x = np.array([[[2.0, 5.0]]])
+    y = lo.butterfly_ortho_mult_tied(theta, x, True)
+    c, s = np.cos(0.3), np.sin(0.3)
+    assert np.allclose(y[0, 0], [c * 2 - s * 5, s * 2 + c * 5])
+    rng = np.random.default_rng(13)
+    n, m, S = 16, 4, 2
+    x = rng.standard_normal((5, S, n))
+    norm = np.linalg.norm(x, axis=-1)
+    th = rng.uniform(0, 2 * np.pi, (S, 3 * 2 * m, n // 2))
+    assert np.allclose(np.linalg.norm(lo.bbt_ortho_mult_untied(th, x), axis=-1), norm)
+    assert np.allclose(np.linalg.norm(lo.odo_mult_untied(th, np.ones((S, 3, n)), x), axis=-1), norm)
+    tht = rng.uniform(0, 2 * np.pi, (S, 4, n - 1))
+    assert np.allclose(np.linalg.norm(lo.bbt_ortho_mult_tied(tht, x), axis=-1), norm)
+    # one block, unit diagonal: the ODO product is the B B^T product of the same angles
+    assert np.allclose(lo.odo_mult_untied(th[:, :2 * m], np.ones((S, 1, n)), x), lo.bbt_ortho_mult_untied(th[:, :2 * m], x))
+    # and the diagonal sits between the two halves
+    d = rng.standard_normal((S, 1, n))
+    half = lo.butterfly_ortho_mult_untied(th[:, :m][:, ::-1], x, False)
+    assert np.allclose(lo.odo_mult_untied(th[:, :2 * m], d, x), lo.butterfly_ortho_mult_untied(th[:, m:2 * m], half * d[:, 0], True))
+
+
+def test_legacy_fast_format_element_formula():
+    """The converter restated operation by operation against the element formula: position e of
+    the stride-2^i slice holds T[pair(e)][r][r] (plane 0) and T[pair(e)][r][1 - r] (plane 1),
+    r = bit i of e."""
+    rng = np.random.default_rng(14)
+    S, m = 2, 4
+    n = 1 << m
+    tw = rng.standard_normal((S, m, n // 2, 2, 2))
+    fast = lo.twiddle_normal_to_fast_format(tw)
+    assert fast.shape == (S, m, 2, n)
+    for i in range(m):
+        for e in range(n):
+            r = (e >> i) & 1
+            pair = ((e >> (i + 1)) << i) | (e & ((1 << i) - 1))
+            assert np.array_equal(fast[:, i, 0, e], tw[:, i, pair, r, r])
+            assert np.array_equal(fast[:, i, 1, e], tw[:, i, pair, r, 1 - r])
+    assert np.array_equal(lo.twiddle_fast_to_normal_format(fast), tw)
+    x = rng.standard_normal((3, S, n))
+    for inc in (True, False):
+        f = fast if inc else fast[:, ::-1]
+        assert np.allclose(lo.butterfly_mult_untied_fast(f, x, inc), lo.butterfly_mult_untied(tw, x, inc))
+
+
+def _numeric_grad(fn, param, g, eps=1e-6):
+    """Central differences of L = Re(sum(conj(g) * fn(param))) in every real coordinate."""
+    out = np.zeros(param.shape, dtype=param.dtype)
+    flat = param.reshape(-1)
+    res = out.reshape(-1)
+    for k in range(flat.size):
+        for unit in ((1.0, 1j) if np.iscomplexobj(param) else (1.0,)):
+            old = flat[k]
+            flat[k] = old + eps * unit
+            up = np.real(np.sum(np.conj(g) * fn(param)))
+            flat[k] = old - eps * unit
+            dn = np.real(np.sum(np.conj(g) * fn(param)))
+            flat[k] = old
+            res[k] += unit * (up - dn) / (2 * eps)
+    return out
+
+
+def test_legacy_gradients_against_central_differences():
+    rng = np.random.default_rng(15)
+    S, m, B = 2, 3, 3
+    n = 1 << m
+    for cplx in (False, True):
+        x = _rand(rng, (B, S, n), cplx)
+        g = _rand(rng, (B, S, n), cplx)
+        for inc in (True, False):
+            tied = _rand(rng, (S, n - 1, 2, 2), cplx)
+            y, d_tw, d_x = lo.butterfly_mult(tied, x, inc, g)
+            assert np.allclose(d_tw, _numeric_grad(lambda p: lo.butterfly_mult(p, x, inc), tied, g), atol=1e-6)
+            assert np.allclose(d_x, _numeric_grad(lambda p: lo.butterfly_mult(tied, p, inc), x.copy(), g), atol=1e-6)
+            untied = _rand(rng, (S, m, n // 2, 2, 2), cplx)
+            y, d_tw, d_x = lo.butterfly_mult_untied(untied, x, inc, g)
+            assert np.allclose(d_tw, _numeric_grad(lambda p: lo.butterfly_mult_untied(p, x, inc), untied, g), atol=1e-6)
+            assert np.allclose(d_x, _numeric_grad(lambda p: lo.butterfly_mult_untied(untied, p, inc), x.copy(), g), atol=1e-6)
+    x, g = rng.standard_normal((B, S, n)), rng.standard_normal((B, S, n))
+    for inc in (True, False):
+        th = rng.uniform(0, 6, (S, n - 1))
+        _, d_th, d_x = lo.butterfly_ortho_mult_tied(th, x, inc, g)
+        assert np.allclose(d_th, _numeric_grad(lambda p: lo.butterfly_ortho_mult_tied(p, x, inc), th, g), atol=1e-6)
+        th = rng.uniform(0, 6, (S, m, n // 2))
+        _, d_th, d_x = lo.butterfly_ortho_mult_untied(th, x, inc, g)
+        assert np.allclose(d_th, _numeric_grad(lambda p: lo.butterfly_ortho_mult_untied(p, x, inc), th, g), atol=1e-6)
+        assert np.allclose(d_x, _numeric_grad(lambda p: lo.butterfly_ortho_mult_untied(th, p, inc), x.copy(), g), atol=1e-6)
+        fast = rng.standard_normal((S, m, 2, n))
+        _, d_f, d_x = lo.butterfly_mult_untied_fast(fast, x, inc, g)
+        assert np.allclose(d_f, _numeric_grad(lambda p: lo.butterfly_mult_untied_fast(p, x, inc), fast, g), atol=1e-6)
+    tw = rng.standard_normal((S, 2 * 2 * m, n // 2, 2, 2))
+    _, d_tw, d_x = lo.bbt_mult_untied(tw, x, g)
+    assert np.allclose(d_tw, _numeric_grad(lambda p: lo.bbt_mult_untied(p, x), tw, g), atol=1e-6)
+    assert np.allclose(d_x, _numeric_grad(lambda p: lo.bbt_mult_untied(tw, p), x.copy(), g), atol=1e-6)
+    fast = rng.standard_normal((S, 2 * 2 * m, 2, n))
+    _, d_f, d_x = lo.bbt_mult_untied_fast(fast, x, g)
+    assert np.allclose(d_f, _numeric_grad(lambda p: lo.bbt_mult_untied_fast(p, x), fast, g), atol=1e-6)
+    th = rng.uniform(0, 6, (S, 2 * 2 * m, n // 2))
+    _, d_th, _ = lo.bbt_ortho_mult_untied(th, x, g)
+    assert np.allclose(d_th, _numeric_grad(lambda p: lo.bbt_ortho_mult_untied(p, x), th, g), atol=1e-6)
+    tht = rng.uniform(0, 6, (S, 4, n - 1))
+    _, d_th, d_x = lo.bbt_ortho_mult_tied(tht, x, g)
+    assert np.allclose(d_th, _numeric_grad(lambda p: lo.bbt_ortho_mult_tied(p, x), tht, g), atol=1e-6)
+    diag = rng.standard_normal((S, 2, n))
+    _, d_th, d_d, d_x = lo.odo_mult_untied(th, diag, x, g)
+    assert np.allclose(d_th, _numeric_grad(lambda p: lo.odo_mult_untied(p, diag, x), th, g), atol=1e-6)
+    assert np.allclose(d_d, _numeric_grad(lambda p: lo.odo_mult_untied(th, p, x), diag, g), atol=1e-6)
+    assert np.allclose(d_x, _numeric_grad(lambda p: lo.odo_mult_untied(th, diag, p), x.copy(), g), atol=1e-6)
