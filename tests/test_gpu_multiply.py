@@ -204,6 +204,56 @@ def test_c_abi_strided_operands():
     assert torch.equal(y2, y)
 
 
+def _random_case(seed):
+    rng = np.random.default_rng(seed)
+    dtype = np.complex64 if rng.random() < 0.35 else np.float32
+    L = int(rng.integers(1, 14))
+    n = 1 << L
+    nb = int(rng.integers(1, 4))
+    S = int(rng.integers(1, 4))
+    budget = (1 << 20) // (n * S * nb)                       # keeps the oracle to a fraction of a second
+    B = int(rng.integers(1, max(2, min(400, budget + 1))))
+    I = n if rng.random() < 0.4 else int(rng.integers(1, n + 6))
+    O = None if rng.random() < 0.4 else int(rng.integers(1, n + 1))
+    inc = bool(rng.integers(0, 2))
+    layout = ["dense", "stack broadcast", "batch innermost", "padded rows"][int(rng.integers(0, 4))]
+    return rng, dtype, B, S, L, nb, I, O, inc, layout
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_shapes_and_layouts(seed):
+    """Seeded sweep over sizes, block counts, paddings, trims and input layouts through the C ABI."""
+    from butterfly_amd import _capi
+    rng, dtype, B, S, L, nb, I, O, inc, layout = _random_case(5000 + seed)
+    say("random case", seed, np.dtype(dtype).name, B, S, L, nb, I, O, inc, layout)
+    n = 1 << L
+    tw = (randn(rng, (S, nb, L, n // 2, 2, 2), dtype) / np.sqrt(2)).astype(dtype)
+    cols = n if O is None else O
+    g = randn(rng, (B, S, cols), dtype)
+    if layout == "stack broadcast":
+        x1 = randn(rng, (B, I), dtype)
+        x = np.ascontiguousarray(np.broadcast_to(x1[:, None, :], (B, S, I)))
+        x_dev = dev(x1).unsqueeze(1).expand(B, S, I)
+    elif layout == "batch innermost":
+        x = randn(rng, (B, S, I), dtype)
+        x_dev = dev(np.ascontiguousarray(x.transpose(1, 2, 0))).permute(2, 0, 1)
+    elif layout == "padded rows":
+        big = randn(rng, (B, S, I + 3), dtype)
+        x = np.ascontiguousarray(big[:, :, :I])
+        x_dev = dev(big)[:, :, :I]
+    else:
+        x = randn(rng, (B, S, I), dtype)
+        x_dev = dev(x)
+    y_ref = oracle.butterfly_fw(tw, x, inc, O)
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+    y = _capi.multiply_fw(dev(tw), x_dev, inc, O)
+    dtw, dx = _capi.multiply_bw(dev(tw), x_dev, dev(g), inc)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
 BASE4_CASES = [
     (np.float32, 9, 2, 2, 1, None, None, True),
     (np.float32, 9, 2, 3, 2, None, None, False),
