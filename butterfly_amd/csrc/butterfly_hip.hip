@@ -174,19 +174,23 @@ bool span_ok(const int64_t stride[3], int64_t rows, int64_t width, size_t elem)
     return bytes < 2147483000.0;
 }
 
+constexpr int kMaxPasses = 96;
+constexpr int kMaxLogN = 24;  // the chunk index of the register-resident kernels travels in blockIdx.z
+
 struct Pass {
     int t0, t1;     // stage range [t0, t1)
     bool high;
     bool wide;      // forward only: one whole block of a 2048- or 4096-element row (wide.hpp)
     int L, NB;      // LOW: FastPlan<L, NB, inc> on chunks of 2^L elements
     bool inc;
-    int H, NST, PAT;  // HIGH: H high bits, NST stages, bit hb of PAT = high bit paired by stage s
+    int H, NST, PAT;  // HIGH: H adjacent bits from `lb` up, NST stages, bit s of PAT = which of them stage s pairs
+    int lb;
 };
 
 struct PassPlan {
     bool ok = false;
     int npass = 0;
-    Pass pass[40];
+    Pass pass[kMaxPasses];
     int64_t chunks = 1;  // 1024-element chunks per row (LOW passes)
     int max_nst = 0;
 };
@@ -203,7 +207,7 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
 {
     PassPlan pl;
     const int L = (int)p->log_n;
-    if (base4 || L < 1 || L > 12 || p->nblocks < 1 || p->batch <= 0 || p->nstacks <= 0 ||
+    if (base4 || L < 1 || L > kMaxLogN || p->nblocks < 1 || p->batch <= 0 || p->nstacks <= 0 ||
         p->input_size <= 0 || p->output_size <= 0)
         return pl;
     const int NS = L * (int)p->nblocks;
@@ -211,7 +215,7 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
     const int max_nb = p->dtype == BF_C64 ? 1 : 2;
     if (L <= 10) {
         for (int k = 0; k < p->nblocks; k += max_nb) {
-            if (pl.npass == 40) return pl;
+            if (pl.npass == kMaxPasses) return pl;
             Pass &q = pl.pass[pl.npass++];
             q = Pass{};
             q.NB = std::min<int>(max_nb, (int)p->nblocks - k);
@@ -220,9 +224,9 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             q.L = L;
             q.inc = (p->increasing_stride != 0) != ((k & 1) != 0);
         }
-    } else if (forward_only && (p->dtype == BF_F32 || L == 11)) {
+    } else if (L <= 12 && forward_only && (p->dtype == BF_F32 || L == 11)) {
         for (int k = 0; k < p->nblocks; ++k) {
-            if (pl.npass == 40) return pl;
+            if (pl.npass == kMaxPasses) return pl;
             Pass &q = pl.pass[pl.npass++];
             q = Pass{};
             q.wide = true;
@@ -232,23 +236,28 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             q.inc = (p->increasing_stride != 0) != ((k & 1) != 0);
         }
     } else {
+        // bits 0..9: the register-resident kernels on 1024-element chunks; bits from 10 up: one
+        // streaming pass per group of two adjacent bits (the top group has one when L is odd)
         pl.chunks = (int64_t)1 << (L - 10);
+        auto group_of = [](int bit) { return bit < 10 ? -1 : (bit - 10) / 2; };
         int t = 0;
         while (t < NS) {
-            if (pl.npass == 40) return pl;
+            if (pl.npass == kMaxPasses) return pl;
             Pass &q = pl.pass[pl.npass++];
             q = Pass{};
             q.t0 = t;
-            const bool high = stage_bit(p, t) >= 10;
+            const int grp = group_of(stage_bit(p, t));
+            const bool high = grp >= 0;
             int u = t;
-            while (u < NS && (stage_bit(p, u) >= 10) == high && (high || u - t < 10 * max_nb)) ++u;
+            while (u < NS && group_of(stage_bit(p, u)) == grp && (high || u - t < 10 * max_nb)) ++u;
             q.t1 = u;
             q.high = high;
             if (high) {
-                q.H = L - 10;
+                q.lb = 10 + 2 * grp;
+                q.H = std::min(2, L - q.lb);
                 q.NST = u - t;
                 if (q.NST > 2 * q.H) return pl;
-                for (int s = 0; s < q.NST; ++s) q.PAT |= (stage_bit(p, t + s) - 10) << s;
+                for (int s = 0; s < q.NST; ++s) q.PAT |= (stage_bit(p, t + s) - q.lb) << s;
             } else {
                 q.L = 10;
                 if ((u - t) != 10 && (u - t) != 20) return pl;
@@ -301,10 +310,12 @@ struct HighGrid {
     int64_t nparts, rows_per_wg;
 };
 
-HighGrid high_grid(int64_t batch, int64_t nstacks)
+// Row partition of a HIGH pass whose row takes `row_threads` threads (n >> H): about 2048
+// threads per compute unit over all stacks.
+HighGrid high_grid(int64_t batch, int64_t nstacks, int64_t row_threads)
 {
     HighGrid g;
-    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * 2 / nstacks);
+    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * 2 * 1024 / (nstacks * row_threads));
     g.nparts = std::min(want, batch);
     g.rows_per_wg = (batch + g.nparts - 1) / g.nparts;
     g.nparts = (batch + g.rows_per_wg - 1) / g.rows_per_wg;
@@ -320,7 +331,7 @@ bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
         const Pass &q = pl.pass[k];
         if (q.high) {
             // the backward high-bit kernel forms 32-bit offsets from its workgroup's first row
-            if (backward) rows = std::max(rows, high_grid(p->batch, p->nstacks).rows_per_wg + kHighAhead + 1);
+            if (backward) rows = std::max(rows, high_grid(p->batch, p->nstacks, n >> q.H).rows_per_wg + kHighAhead + 1);
             continue;
         }
         const FastGrid g = q.wide ? wide_grid(p->batch, p->nstacks)
@@ -390,8 +401,9 @@ void launch_high_t(bool backward, const HighArgs &a, dim3 grid, hipStream_t stre
 {
     if (backward) {
         // float leaves room for 1024 threads (128 registers each), complex64 for 512
+        // grid.z arrives as the threads a row takes
         constexpr int THREADS = sizeof(T) == 4 ? 1024 : 512;
-        grid.z = 1024 / THREADS;
+        grid.z = grid.z / THREADS;
         hipLaunchKernelGGL((high_bw_kernel<T, H, NST, PAT, THREADS>), grid, dim3(THREADS), 0, stream, a);
     } else
         hipLaunchKernelGGL((high_fw_kernel<T, H, NST, PAT>), grid, dim3(kHighThreads), 0, stream, a);
@@ -436,8 +448,9 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
         const View sv = k == first ? in_view : dense;
         const View dv = k == last - 1 ? out_view : dense;
         if (q.high) {
-            const HighGrid g = high_grid(p->batch, p->nstacks);
+            const HighGrid g = high_grid(p->batch, p->nstacks, n >> q.H);
             HighArgs a = {};
+            a.low_bits = q.lb;
             a.tw = tw;
             a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
             a.tw_stage_stride = (n / 2) * 4;
@@ -448,7 +461,7 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
             a.xo_view = dv;
             a.batch = p->batch;
             a.rows_per_wg = g.rows_per_wg;
-            const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, 1024 / kHighThreads);
+            const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, (unsigned)((n >> q.H) / kHighThreads));
             const int rc = p->dtype == BF_C64 ? launch_high<float2>(q, false, a, grid, stream)
                                               : launch_high<float>(q, false, a, grid, stream);
             if (rc) return rc;
@@ -803,12 +816,13 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
         pl.nchunks = mp.npass;
         pl.slot = 2 * n;
         pl.boundary_bytes = align256((size_t)p->batch * p->nstacks * row_bytes);
-        int64_t nparts = 1;
+        int64_t nparts = 1, slices = 1;  // slices: partial (stage, 2n) slices of the pass that needs most
         for (int k = 0; k < mp.npass; ++k) {
             const Pass &q = mp.pass[k];
-            const int64_t np = q.high ? high_grid(p->batch, p->nstacks).nparts
+            const int64_t np = q.high ? high_grid(p->batch, p->nstacks, n >> q.H).nparts
                                       : fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1).nwg;
             nparts = std::max(nparts, np);
+            slices = std::max(slices, np * (q.t1 - q.t0));
         }
         pl.nparts = nparts;
         size_t off = 0;
@@ -817,7 +831,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
         pl.off_gbuf = off;
         off += mp.npass > 1 ? pl.boundary_bytes : 0;
         pl.off_partials = off;
-        off += align256((size_t)nparts * p->nstacks * mp.max_nst * pl.slot * e);
+        off += align256((size_t)slices * p->nstacks * pl.slot * e);
         pl.total = off;
         return pl;
     }
@@ -991,8 +1005,9 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
             const View giv = k == 0 ? dn_view : dense;
             int64_t nparts = 0;
             if (q.high) {
-                const HighGrid g = high_grid(p->batch, p->nstacks);
+                const HighGrid g = high_grid(p->batch, p->nstacks, n >> q.H);
                 HighArgs a = {};
+                a.low_bits = q.lb;
                 a.tw = tw2;
                 a.tw_stack_stride = sc.tw2_stack_stride;
                 a.tw_stage_stride = (n / 2) * 4;
@@ -1008,7 +1023,8 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                 a.batch = p->batch;
                 a.rows_per_wg = g.rows_per_wg;
                 nparts = g.nparts;
-                const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, 1024 / kHighThreads);
+                // (the launcher sets gridDim.z from the backward kernel's workgroup size)
+                const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, (unsigned)(n >> q.H));
                 rc = p->dtype == BF_C64 ? launch_high<float2>(q, true, a, grid, stream)
                                         : launch_high<float>(q, true, a, grid, stream);
                 if (rc) return rc;

@@ -1,11 +1,13 @@
 // Stages that pair element bits >= 10 of rows longer than 1024.
 //
-// Such a stage couples elements 1024 (or 2048) apart, so a thread takes one low position
-// p in [0, 1024) and holds the 2^H elements {p + j * 1024} of a row in registers; all the
-// stages of the pass run in registers with their 2x2 factors resident for the whole launch.
-// Threads of a workgroup take consecutive p, so every access is a coalesced row segment.
+// A pass handles the stages on H adjacent bits [low_bits, low_bits + H), low_bits >= 10.  A
+// thread takes one setting p of all the other bits and holds the 2^H elements of a row that
+// differ in those H bits in registers; all the stages of the pass run in registers with their
+// 2x2 factors resident for the whole launch.  Threads of a workgroup take consecutive p, whose
+// low ten bits are the element's low ten bits, so every access is a coalesced row segment.
 // The pass is purely streaming: one read and one write of the activation (plus one read of
-// the gradient in the backward pass).
+// the gradient in the backward pass).  Rows of any length are covered by one such pass per
+// group of high bits next to the chunked kernels for bits 0..9.
 #pragma once
 
 #include "common.hpp"
@@ -15,6 +17,12 @@ namespace bf {
 
 constexpr int kHighThreads = 256;
 constexpr int kHighLowBits = 10;  // bits below this are handled by the chunked kernels
+
+// Element index of register j of thread p: the H bits of j inserted at bit position lb of p.
+__device__ __forceinline__ int high_col(int p, int j, int lb, int H)
+{
+    return ((p >> lb) << (lb + H)) | (j << lb) | (p & ((1 << lb) - 1));
+}
 
 struct HighArgs {
     const void *tw;            // twiddle tensor, stack 0
@@ -33,9 +41,10 @@ struct HighArgs {
     int64_t partial_slot;
     int64_t batch;
     int64_t rows_per_wg;
+    int low_bits;              // position of the lowest of the H bits this pass works on (>= 10)
 };
 
-// hb(s): which of the H high bits stage s pairs (bit 10 + hb)
+// hb(s): which of the H bits stage s pairs (bit low_bits + hb)
 template <int PAT>
 __host__ __device__ constexpr int high_bit_of(int s) { return (PAT >> s) & 1; }
 
@@ -58,11 +67,11 @@ struct HighTwiddle {
         static_for<0, NST>([&](auto S) {
             constexpr int s = S;
             constexpr int hb = high_bit_of<PAT>(s);
-            constexpr int b = kHighLowBits + hb;
+            const int b = a.low_bits + hb;
             static_for<0, E / 2>([&](auto Q) {
                 constexpr int q = Q;
                 constexpr int j0 = j0_of(s, q);
-                const int e = (j0 << kHighLowBits) | p;
+                const int e = high_col(p, j0, a.low_bits, H);
                 const int i = ((e >> (b + 1)) << b) | (e & ((1 << b) - 1));
                 const T *src = base + a.tw_stage[s] * a.tw_stage_stride + (int64_t)i * 4;
 #pragma unroll
@@ -90,7 +99,7 @@ __global__ __launch_bounds__(kHighThreads) void high_fw_kernel(HighArgs a)
     int x_col[E], xo_col[E];  // tensor columns of the thread's elements (-1: none)
 #pragma unroll
     for (int j = 0; j < E; ++j) {
-        const int col = (j << kHighLowBits) | p;
+        const int col = high_col(p, j, a.low_bits, H);
         x_col[j] = (int)view_col(a.x_view, col);
         xo_col[j] = (int)view_col(a.xo_view, col);
     }
@@ -135,7 +144,7 @@ __global__ __launch_bounds__(kHighThreads) void high_fw_kernel(HighArgs a)
 // fast.hpp) kHighAhead rows ahead: a lane reads back exactly the dwords it fetched itself, so
 // no barrier is involved, only the wait for the wavefront's own requests.  All operands are
 // addressed with 32-bit offsets from the workgroup's first row (the host checks the span).
-// THREADS low positions per workgroup (gridDim.z = 1024 / THREADS): as many as the registers
+// THREADS positions per workgroup (gridDim.z = (n >> H) / THREADS): as many as the registers
 // allow, so that a workgroup touches long contiguous pieces of every quarter-row.
 constexpr int kHighAhead = 3;   // rows requested ahead; kHighAhead + 1 row slots in LDS
 
@@ -174,7 +183,7 @@ __global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
     int x_off[E], g_off[E], gi_off[E];
 #pragma unroll
     for (int j = 0; j < E; ++j) {
-        const int col = (j << kHighLowBits) | p;
+        const int col = high_col(p, j, a.low_bits, H);
         const int64_t xc = view_col(a.x_view, col), gc = view_col(a.g_view, col), gic = view_col(a.gi_view, col);
         x_off[j] = xc >= 0 ? (int)(xc * a.x_view.se * EB) : kOob;
         g_off[j] = gc >= 0 ? (int)(gc * a.g_view.se * EB) : kOob;
@@ -284,11 +293,11 @@ __global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
     static_for<0, NST>([&](auto S) {
         constexpr int s = S;
         constexpr int hb = high_bit_of<PAT>(s);
-        constexpr int b = kHighLowBits + hb;
+        const int b = a.low_bits + hb;
         static_for<0, E / 2>([&](auto Q) {
             constexpr int q = Q;
             constexpr int j0 = TW::j0_of(s, q);
-            const int e = (j0 << kHighLowBits) | p;
+            const int e = high_col(p, j0, a.low_bits, H);
             const int i = ((e >> (b + 1)) << b) | (e & ((1 << b) - 1));
             T *d = part + (int64_t)s * a.partial_slot + (int64_t)i * 4;
 #pragma unroll

@@ -139,6 +139,41 @@ def test_multi_launch_schedules(case):
     assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
 
 
+LONG_ROW_CASES = [
+    # dtype, B, S, L, nb, I, O, inc -- rows beyond 4096: chunked passes for bits 0..9 and one
+    # streaming pass per group of two higher bits (odd and even numbers of high bits, the block
+    # boundary inside the top group, several row partitions)
+    (np.float32, 9, 1, 13, 1, None, None, True),
+    (np.float32, 9, 2, 13, 2, None, None, False),
+    (np.float32, 7, 1, 14, 2, 16000, 9000, True),
+    (np.float32, 5, 1, 15, 3, None, None, False),
+    (np.float32, 3, 1, 16, 1, None, None, True),
+    (np.float32, 2, 1, 17, 1, None, 70000, False),
+    (np.float32, 300, 1, 13, 1, None, None, True),
+    (np.complex64, 6, 1, 13, 2, None, None, True),
+    (np.complex64, 4, 2, 14, 1, 9000, None, False),
+    (np.complex64, 3, 1, 15, 1, None, None, True),
+    (np.complex64, 120, 1, 13, 1, None, None, False),
+]
+
+
+@pytest.mark.parametrize("case", LONG_ROW_CASES, ids=lambda c: f"{np.dtype(c[0]).name}-B{c[1]}-S{c[2]}-L{c[3]}-nb{c[4]}-I{c[5]}-O{c[6]}-inc{int(c[7])}")
+def test_long_rows(case):
+    from butterfly_amd import _capi
+    dtype, B, S, L, nb, I, O, inc = case
+    say("long-row case", case)
+    rng = np.random.default_rng(1900 + L * 13 + nb)
+    tw, x, g = make_case(rng, dtype, B, S, L, nb, I, O)
+    y_ref = oracle.butterfly_fw(tw, x, inc, O)
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+    y = _capi.multiply_fw(dev(tw), dev(x), inc, O)
+    dtw, dx = _capi.multiply_bw(dev(tw), dev(x), dev(g), inc)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
 COMPLEX_FAST_CASES = [
     # B, S, L, nb, I, O, inc
     (37, 2, 1, 2, None, None, True),
