@@ -18,6 +18,7 @@
 #include "high.hpp"
 #include "wide.hpp"
 #include "fast4.hpp"
+#include "fast4g.hpp"
 #include "bias.hpp"
 
 namespace {
@@ -523,20 +524,34 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
 
 constexpr int kFast4FwRows = 4;
 
-bool fast4_ok(const bf_problem *p, bool base4, bool backward)
+constexpr int kFast4GFwRowsComplex = 2;
+
+// base-4 shapes outside fast4.hpp's aligned float kernels
+bool fast4_general(const bf_problem *p) { return p->dtype != BF_F32 || (p->log_n & 1) != 0; }
+
+int fast4_fw_rows(const bf_problem *p) { return p->dtype == BF_C64 ? kFast4GFwRowsComplex : kFast4FwRows; }
+
+// Which register-resident base-4 kernels take this problem: 0 none (generic kernels), 1 the
+// aligned float kernels of fast4.hpp (even log_n), 2 the general ones of fast4g.hpp (odd
+// log_n, complex64 up to n = 256: beyond that the complex factors outgrow the registers).
+int fast4_kind(const bf_problem *p, bool base4, bool backward)
 {
-    if (!base4 || p->dtype != BF_F32 || p->log_n < 2 || p->log_n > 10 || (p->log_n & 1) || p->nblocks < 1 ||
-        p->batch <= 0 || p->nstacks <= 0 || p->input_size <= 0 || p->output_size <= 0)
-        return false;
+    if (!base4 || p->log_n < 2 || p->log_n > 10 || p->nblocks < 1 || p->batch <= 0 || p->nstacks <= 0 ||
+        p->input_size <= 0 || p->output_size <= 0)
+        return 0;
+    if (p->dtype == BF_C64 && p->log_n > 8) return 0;
     const int64_t n = (int64_t)1 << p->log_n;
-    const FastGrid g = fast_grid(p->batch, (int)p->log_n, p->nstacks, backward ? 1 : kFast4FwRows, 1);
+    const size_t e = elem_bytes(p->dtype);
+    const FastGrid g = fast_grid(p->batch, (int)p->log_n, p->nstacks, backward ? 1 : fast4_fw_rows(p), 1);
     const int64_t rows = (g.groups_per_wg + kFast4FwRows + 2) * g.slots;
     const int64_t dense[3] = {p->nstacks * n, n, 1};
-    if (!span_ok(p->input_stride, rows, n, 4) || !span_ok(p->output_stride, rows, n, 4) || !span_ok(dense, rows, n, 4))
-        return false;
-    if (backward && !span_ok(p->d_input_stride, rows, n, 4)) return false;
-    return true;
+    if (!span_ok(p->input_stride, rows, n, e) || !span_ok(p->output_stride, rows, n, e) || !span_ok(dense, rows, n, e))
+        return 0;
+    if (backward && !span_ok(p->d_input_stride, rows, n, e)) return 0;
+    return fast4_general(p) ? 2 : 1;
 }
+
+bool fast4_ok(const bf_problem *p, bool base4, bool backward) { return fast4_kind(p, base4, backward) != 0; }
 
 template <int L, bool INC>
 void launch_fast4_t(bool backward, const Fast4Args &a, dim3 grid, hipStream_t stream)
@@ -564,14 +579,78 @@ int launch_fast4(int L, bool inc, bool backward, const Fast4Args &a, dim3 grid, 
     return BF_OK;
 }
 
+template <typename T, int L, bool INC>
+void launch_fast4g_t(bool backward, const Fast4GArgs &a, dim3 grid, hipStream_t stream)
+{
+    constexpr int R = sizeof(T) == 4 ? kFast4FwRows : kFast4GFwRowsComplex;
+    if (backward) hipLaunchKernelGGL((fast4g_bw_kernel<T, L, INC>), grid, dim3(kFastThreads), 0, stream, a);
+    else hipLaunchKernelGGL((fast4g_fw_kernel<T, L, INC, R>), grid, dim3(kFastThreads), 0, stream, a);
+}
+
+int launch_fast4g(bool cplx, int L, bool inc, bool backward, const Fast4GArgs &a, dim3 grid, hipStream_t stream)
+{
+#define BF_F4G(LL)                                                                              \
+    case LL * 2 + 0: launch_fast4g_t<float, LL, false>(backward, a, grid, stream); break;        \
+    case LL * 2 + 1: launch_fast4g_t<float, LL, true>(backward, a, grid, stream); break;
+#define BF_C4G(LL)                                                                              \
+    case LL * 2 + 0: launch_fast4g_t<float2, LL, false>(backward, a, grid, stream); break;       \
+    case LL * 2 + 1: launch_fast4g_t<float2, LL, true>(backward, a, grid, stream); break;
+    if (cplx) {
+        switch (L * 2 + (inc ? 1 : 0)) {
+            BF_C4G(2) BF_C4G(3) BF_C4G(4) BF_C4G(5) BF_C4G(6) BF_C4G(7) BF_C4G(8)
+            default: return fail(BF_ERR_UNSUPPORTED, "no base-4 kernel for this shape");
+        }
+    } else {
+        switch (L * 2 + (inc ? 1 : 0)) {
+            BF_F4G(3) BF_F4G(5) BF_F4G(7) BF_F4G(9)
+            default: return fail(BF_ERR_UNSUPPORTED, "no base-4 kernel for this shape");
+        }
+    }
+#undef BF_F4G
+#undef BF_C4G
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
+}
+
+// Operands of block k for the general base-4 kernels
+Fast4GArgs fast4g_block_args(const bf_problem *p, const void *tw4, const void *tw2, int k)
+{
+    const int64_t n = (int64_t)1 << p->log_n;
+    const int L = (int)p->log_n;
+    const size_t e = elem_bytes(p->dtype);
+    Fast4GArgs a = {};
+    a.tw4 = static_cast<const char *>(tw4) + (size_t)k * (L / 2) * (n / 4) * 16 * e;
+    a.tw4_stack_stride = p->nblocks * (L / 2) * (n / 4) * 16;
+    a.tw2 = (L & 1) ? static_cast<const char *>(tw2) + (size_t)k * (n / 2) * 4 * e : nullptr;
+    a.tw2_stack_stride = p->nblocks * (L & 1) * (n / 2) * 4;
+    a.batch = p->batch;
+    return a;
+}
+
 // forward of blocks [first, last) through the base-4 kernels; `scratch` as in multipass_forward
-int fast4_forward(const bf_problem *p, const void *tw4, const void *input, void *output, void *scratch,
-                  const View &in_view, const View &out_view, int first, int last, hipStream_t stream)
+int fast4_forward(const bf_problem *p, const void *tw4, const void *tw2, const void *input, void *output,
+                  void *scratch, const View &in_view, const View &out_view, int first, int last, hipStream_t stream)
 {
     const int64_t n = (int64_t)1 << p->log_n;
     const int L = (int)p->log_n;
     const View dense = dense_view(p->nstacks, n);
-    const FastGrid g = fast_grid(p->batch, L, p->nstacks, kFast4FwRows, 1);
+    const FastGrid g = fast_grid(p->batch, L, p->nstacks, fast4_fw_rows(p), 1);
+    if (fast4_general(p)) {
+        for (int k = first; k < last; ++k) {
+            Fast4GArgs a = fast4g_block_args(p, tw4, tw2, k);
+            a.x_in = k == first ? input : scratch;
+            a.x_view = k == first ? in_view : dense;
+            a.x_out = k == last - 1 ? output : scratch;
+            a.xo_view = k == last - 1 ? out_view : dense;
+            a.ngroups = g.ngroups;
+            a.groups_per_wg = g.groups_per_wg;
+            const bool inc = (p->increasing_stride != 0) != ((k & 1) != 0);
+            const int rc = launch_fast4g(p->dtype == BF_C64, L, inc, false, a,
+                                         dim3((unsigned)g.nwg, (unsigned)p->nstacks), stream);
+            if (rc) return rc;
+        }
+        return BF_OK;
+    }
     for (int k = first; k < last; ++k) {
         Fast4Args a = {};
         a.tw4 = static_cast<const float *>(tw4) + (int64_t)k * (L / 2) * (n / 4) * 16;
@@ -634,7 +713,7 @@ size_t forward_workspace(const bf_problem *p, bool base4)
 {
     if (fast4_ok(p, base4, false)) {
         const int64_t n4 = (int64_t)1 << p->log_n;
-        return p->nblocks > 1 ? align256((size_t)p->batch * p->nstacks * n4 * 4) : 0;
+        return p->nblocks > 1 ? align256((size_t)p->batch * p->nstacks * n4 * elem_bytes(p->dtype)) : 0;
     }
     const PassPlan mp = build_passes(p, base4, true);
     if (!mp.ok || mp.npass <= 1 || !passes_addressable(p, mp, false)) return 0;
@@ -701,9 +780,10 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
         const size_t need = forward_workspace(p, base4);
         if (need > 0 && (!workspace || workspace_bytes < need))
             return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-        rc = fast4_forward(p, tw4, input, output, workspace, in_view, out_view, 0, (int)p->nblocks, stream);
+        rc = fast4_forward(p, tw4, tw2, input, output, workspace, in_view, out_view, 0, (int)p->nblocks, stream);
         if (rc || !bias) return rc;
-        return launch_bias_add<float>(p, bias, output, out_view, stream);
+        return p->dtype == BF_C64 ? launch_bias_add<float2>(p, bias, output, out_view, stream)
+                                  : launch_bias_add<float>(p, bias, output, out_view, stream);
     }
     const PassPlan mp = build_passes(p, base4, true);
     if (mp.ok && passes_addressable(p, mp, false)) {
@@ -803,7 +883,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
         pl.off_gbuf = off;
         off += p->nblocks > 1 ? pl.boundary_bytes : 0;
         pl.off_partials = off;
-        off += align256((size_t)pl.nparts * p->nstacks * (p->log_n / 2) * pl.slot * e);
+        off += align256((size_t)pl.nparts * p->nstacks * sc.per * pl.slot * e);
         pl.total = off;
         return pl;
     }
@@ -942,16 +1022,35 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     if (pl.fast4) {
         const int L = (int)p->log_n;
         const int P = (int)p->nblocks;
-        const int per = L / 2;
+        const int per = sc.per;
+        const bool general = fast4_general(p);
         auto boundary = [&](int k) { return ws + pl.off_boundaries + (size_t)(k - 1) * pl.boundary_bytes; };
         for (int k = 0; k + 1 < P; ++k) {
-            rc = fast4_forward(p, tw4, k == 0 ? input : boundary(k), boundary(k + 1), nullptr,
+            rc = fast4_forward(p, tw4, tw2, k == 0 ? input : boundary(k), boundary(k + 1), nullptr,
                                k == 0 ? x_view : dense, dense, k, k + 1, stream);
             if (rc) return rc;
         }
         const View dn_view = make_view(p->d_input_stride, std::min(p->input_size, n), in_perm);
         const FastGrid g = fast_grid(p->batch, L, p->nstacks, 1, 1);
-        for (int k = P - 1; k >= 0; --k) {
+        for (int k = P - 1; k >= 0 && general; --k) {
+            Fast4GArgs a = fast4g_block_args(p, tw4, tw2, k);
+            a.x_in = k == 0 ? input : boundary(k);
+            a.x_view = k == 0 ? x_view : dense;
+            a.g_out = k == P - 1 ? grad : ws + pl.off_gbuf;
+            a.g_view = k == P - 1 ? g_view : dense;
+            a.g_in = k == 0 ? d_input : ws + pl.off_gbuf;
+            a.gi_view = k == 0 ? dn_view : dense;
+            a.partial = ws + pl.off_partials;
+            a.ngroups = g.ngroups;
+            a.groups_per_wg = g.groups_per_wg;
+            const bool inc = (p->increasing_stride != 0) != ((k & 1) != 0);
+            rc = launch_fast4g(p->dtype == BF_C64, L, inc, true, a, dim3((unsigned)g.nwg, (unsigned)p->nstacks), stream);
+            if (rc) return rc;
+            rc = launch_reduce(p, sc, k * per, (k + 1) * per, g.nwg, ws + pl.off_partials, pl.slot, d_tw2, d_tw4,
+                               stream);
+            if (rc) return rc;
+        }
+        for (int k = P - 1; k >= 0 && !general; --k) {
             Fast4Args a = {};
             a.tw4 = static_cast<const float *>(tw4) + (int64_t)k * per * (n / 4) * 16;
             a.tw_stack_stride = sc.tw4_stack_stride;

@@ -348,6 +348,38 @@ def test_base4_register_resident_kernels(L):
                 assert rel_err(d4.cpu().numpy(), d4_ref) < BW_TOL, (L, nb, inc, B, S, I, O)
 
 
+@pytest.mark.parametrize("dtype,L", [(np.float32, 3), (np.float32, 5), (np.float32, 7), (np.float32, 9)] +
+                         [(np.complex64, L) for L in range(2, 9)],
+                         ids=lambda v: np.dtype(v).name if isinstance(v, type) else str(v))
+def test_base4_general_register_resident_kernels(dtype, L):
+    """Odd log_n (the block ends with a 2x2 stage; bit pairs unaligned for decreasing stride) and
+    complex64: every size, both stride orders, one to three blocks, ragged batch, padded input,
+    sliced output, many row groups per workgroup."""
+    from butterfly_amd import _capi
+    n = 1 << L
+    rng = np.random.default_rng(2700 + L)
+    big = max(300, 5000 // (1 + (n > 64)))
+    for nb in (1, 2, 3):
+        for inc in (True, False):
+            for B, S, I, O in [(1, 1, n, n), (37, 2, n, n), (big, 1, n - 1, n - 1), (19, 4, n + 5, max(1, n // 2))]:
+                say("base4 general case", np.dtype(dtype).name, L, nb, inc, B, S, I, O)
+                tw4 = (randn(rng, (S, nb, L // 2, n // 4, 4, 4), dtype) / 2).astype(dtype)
+                tw2 = (randn(rng, (S, nb, L % 2, n // 2, 2, 2), dtype) / np.sqrt(2)).astype(dtype)
+                x = randn(rng, (B, S, I), dtype)
+                g = randn(rng, (B, S, O), dtype)
+                y_ref = oracle.butterfly_base4_fw(tw4, tw2, x, inc, O)
+                d4_ref, d2_ref, dx_ref = oracle.butterfly_base4_bw(tw4, tw2, x, g, inc)
+                y = _capi.multiply_base4_fw(dev(tw4), dev(tw2), dev(x), inc, O)
+                d4, d2, dx = _capi.multiply_base4_bw(dev(tw4), dev(tw2), dev(x), dev(g), inc)
+                torch.cuda.synchronize()
+                key = (L, nb, inc, B, S, I, O)
+                assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL, key
+                assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL, key
+                assert rel_err(d4.cpu().numpy(), d4_ref) < BW_TOL, key
+                if L % 2:
+                    assert rel_err(d2.cpu().numpy(), d2_ref) < BW_TOL, key
+
+
 def test_operators_match_oracle_and_autograd():
     """torch.ops.torch_butterfly.* end to end: views returned, autograd wired, lazy conj
     and transposed twiddle views accepted."""
