@@ -184,7 +184,7 @@ struct Pass {
     bool wide;      // forward only: one whole block of a 2048- or 4096-element row (wide.hpp)
     int L, NB;      // LOW: FastPlan<L, NB, inc> on chunks of 2^L elements
     bool inc;
-    int H, NST, PAT;  // HIGH: H adjacent bits from `lb` up, NST stages, bit s of PAT = which of them stage s pairs
+    int H, NST, PAT;  // HIGH: H adjacent bits from `lb` up, NST stages, bits 2s, 2s+1 of PAT = which of them stage s pairs
     int lb;
 };
 
@@ -193,7 +193,6 @@ struct PassPlan {
     int npass = 0;
     Pass pass[kMaxPasses];
     int64_t chunks = 1;  // 1024-element chunks per row (LOW passes)
-    int max_nst = 0;
 };
 
 int stage_bit(const bf_problem *p, int t)
@@ -238,9 +237,25 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
         }
     } else {
         // bits 0..9: the register-resident kernels on 1024-element chunks; bits from 10 up: one
-        // streaming pass per group of two adjacent bits (the top group has one when L is odd)
+        // streaming pass per group of adjacent bits.  Groups of two; float rows take groups of
+        // three (eight elements per thread, a slower kernel) where that saves a pass.
         pl.chunks = (int64_t)1 << (L - 10);
-        auto group_of = [](int bit) { return bit < 10 ? -1 : (bit - 10) / 2; };
+        const int hbits = L - 10;
+        const int ngroups3 = p->dtype == BF_F32 ? (hbits + 2) / 3 : 0;   // passes with groups of up to three
+        const int ngroups2 = (hbits + 1) / 2;
+        const int nthree = (ngroups3 > 0 && ngroups3 < ngroups2) ? hbits - 2 * ngroups3 : 0;
+        int group_lb[16], group_bits[16], ngroups = 0;
+        for (int b = 10; b < L; ++ngroups) {
+            group_lb[ngroups] = b;
+            group_bits[ngroups] = std::min(ngroups < nthree ? 3 : 2, L - b);
+            b += group_bits[ngroups];
+        }
+        auto group_of = [&](int bit) {
+            if (bit < 10) return -1;
+            int g = 0;
+            while (bit >= group_lb[g] + group_bits[g]) ++g;
+            return g;
+        };
         int t = 0;
         while (t < NS) {
             if (pl.npass == kMaxPasses) return pl;
@@ -249,16 +264,20 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             q.t0 = t;
             const int grp = group_of(stage_bit(p, t));
             const bool high = grp >= 0;
+            // a group of three bits takes one sweep over them per pass (its factors and sums
+            // fill the registers); smaller groups also take the way back at a block boundary
+            const int lb = high ? group_lb[grp] : 0;
+            const int H = high ? group_bits[grp] : 0;
+            const int cap = high ? (H == 3 ? 3 : 2 * H) : 10 * max_nb;
             int u = t;
-            while (u < NS && group_of(stage_bit(p, u)) == grp && (high || u - t < 10 * max_nb)) ++u;
+            while (u < NS && group_of(stage_bit(p, u)) == grp && u - t < cap) ++u;
             q.t1 = u;
             q.high = high;
             if (high) {
-                q.lb = 10 + 2 * grp;
-                q.H = std::min(2, L - q.lb);
+                q.lb = lb;
+                q.H = H;
                 q.NST = u - t;
-                if (q.NST > 2 * q.H) return pl;
-                for (int s = 0; s < q.NST; ++s) q.PAT |= (stage_bit(p, t + s) - q.lb) << s;
+                for (int s = 0; s < q.NST; ++s) q.PAT |= (stage_bit(p, t + s) - q.lb) << (2 * s);
             } else {
                 q.L = 10;
                 if ((u - t) != 10 && (u - t) != 20) return pl;
@@ -268,7 +287,6 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             t = u;
         }
     }
-    for (int k = 0; k < pl.npass; ++k) pl.max_nst = std::max(pl.max_nst, pl.pass[k].t1 - pl.pass[k].t0);
     pl.ok = true;
     return pl;
 }
@@ -402,8 +420,9 @@ void launch_high_t(bool backward, const HighArgs &a, dim3 grid, hipStream_t stre
 {
     if (backward) {
         // float leaves room for 1024 threads (128 registers each), complex64 for 512
-        // grid.z arrives as the threads a row takes
-        constexpr int THREADS = sizeof(T) == 4 ? 1024 : 512;
+        // grid.z arrives as the threads a row takes; three bits per pass (float only) hold eight
+        // elements and 48 + 48 factor entries and sums per thread: 256 threads
+        constexpr int THREADS = H == 3 ? 256 : (sizeof(T) == 4 ? 1024 : 512);
         grid.z = grid.z / THREADS;
         hipLaunchKernelGGL((high_bw_kernel<T, H, NST, PAT, THREADS>), grid, dim3(THREADS), 0, stream, a);
     } else
@@ -417,9 +436,15 @@ int launch_high(const Pass &q, bool backward, const HighArgs &a, dim3 grid, hipS
     switch (key) {
         case 1 * 1000 + 1 * 100 + 0: launch_high_t<T, 1, 1, 0>(backward, a, grid, stream); break;
         case 1 * 1000 + 2 * 100 + 0: launch_high_t<T, 1, 2, 0>(backward, a, grid, stream); break;
-        case 2 * 1000 + 2 * 100 + 2: launch_high_t<T, 2, 2, 2>(backward, a, grid, stream); break;  // bits 10, 11
-        case 2 * 1000 + 2 * 100 + 1: launch_high_t<T, 2, 2, 1>(backward, a, grid, stream); break;  // bits 11, 10
-        case 2 * 1000 + 4 * 100 + 6: launch_high_t<T, 2, 4, 6>(backward, a, grid, stream); break;  // 10, 11, 11, 10
+        case 2 * 1000 + 2 * 100 + 4: launch_high_t<T, 2, 2, 4>(backward, a, grid, stream); break;    // bits 0, 1 of the group
+        case 2 * 1000 + 2 * 100 + 1: launch_high_t<T, 2, 2, 1>(backward, a, grid, stream); break;    // 1, 0
+        case 2 * 1000 + 4 * 100 + 20: launch_high_t<T, 2, 4, 20>(backward, a, grid, stream); break;  // 0, 1, 1, 0
+        case 3 * 1000 + 3 * 100 + 36:                                                                // 0, 1, 2
+            if constexpr (sizeof(T) == 4) { launch_high_t<T, 3, 3, 36>(backward, a, grid, stream); break; }
+            return fail(BF_ERR_UNSUPPORTED, "no kernel for this high-bit stage pattern");
+        case 3 * 1000 + 3 * 100 + 6:                                                                 // 2, 1, 0
+            if constexpr (sizeof(T) == 4) { launch_high_t<T, 3, 3, 6>(backward, a, grid, stream); break; }
+            return fail(BF_ERR_UNSUPPORTED, "no kernel for this high-bit stage pattern");
         default: return fail(BF_ERR_UNSUPPORTED, "no kernel for this high-bit stage pattern");
     }
     BF_HIP_CHECK(hipGetLastError());

@@ -16,8 +16,6 @@
 namespace bf {
 
 constexpr int kHighThreads = 256;
-constexpr int kHighLowBits = 10;  // bits below this are handled by the chunked kernels
-
 // Element index of register j of thread p: the H bits of j inserted at bit position lb of p.
 __device__ __forceinline__ int high_col(int p, int j, int lb, int H)
 {
@@ -44,9 +42,9 @@ struct HighArgs {
     int low_bits;              // position of the lowest of the H bits this pass works on (>= 10)
 };
 
-// hb(s): which of the H bits stage s pairs (bit low_bits + hb)
+// hb(s): which of the H bits stage s pairs (bit low_bits + hb); two bits of PAT per stage
 template <int PAT>
-__host__ __device__ constexpr int high_bit_of(int s) { return (PAT >> s) & 1; }
+__host__ __device__ constexpr int high_bit_of(int s) { return (PAT >> (2 * s)) & 3; }
 
 template <typename T, int H, int NST, int PAT>
 struct HighTwiddle {
@@ -156,8 +154,9 @@ __global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
     constexpr int W = (int)sizeof(T) / 4;  // dwords per scalar: the planes of a complex row are fetched separately
     constexpr int EB = (int)sizeof(T);
     // complex64 rows would have to be fetched as two strided 32-bit planes, which measured
-    // slower than plain register prefetch: float only
-    constexpr bool DIRECT = W == 1;
+    // slower than plain register prefetch: float only; with eight elements per thread the
+    // requests in flight would overflow the 6-bit wait counter: register prefetch as well
+    constexpr bool DIRECT = W == 1 && H <= 2;
     constexpr int SLOT = 2 * E * W * THREADS;  // dwords per row slot: x and g, E elements, W planes
     __shared__ float rows[DIRECT ? (kHighAhead + 1) * SLOT : 1];
     const int p = blockIdx.z * THREADS + threadIdx.x;
@@ -214,7 +213,7 @@ __global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
     // memory operations issued after the requests of a row and before that row is read: the
     // requests of the kHighAhead following rows and the stores of the kHighAhead rows before it
     constexpr int YOUNGER = kHighAhead * (2 * E * W + E);
-    static_assert(YOUNGER <= 63, "the wait counter holds 6 bits");
+    static_assert(!DIRECT || YOUNGER <= 63, "the wait counter holds 6 bits");
 
     // register flavour: one row ahead
     const __amdgpu_buffer_rsrc_t x_rs = make_rsrc(reinterpret_cast<const T *>(a.x_in) + stack * a.x_view.ss + r0 * a.x_view.sb);
@@ -243,7 +242,7 @@ __global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
         T act[NST][E], g[E];
         if constexpr (DIRECT) {
             fetch_row(row + kHighAhead);
-            wait_rows_in_lds<YOUNGER>();
+            wait_rows_in_lds<DIRECT ? YOUNGER : 0>();
 #pragma unroll
             for (int j = 0; j < E; ++j) {
                 act[0][j] = read_row(row, 0, j);
