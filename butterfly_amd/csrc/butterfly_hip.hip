@@ -581,7 +581,9 @@ bool fast4_ok(const bf_problem *p, bool base4, bool backward) { return fast4_kin
 template <int L, bool INC>
 void launch_fast4_t(bool backward, const Fast4Args &a, dim3 grid, hipStream_t stream)
 {
-    if (backward) hipLaunchKernelGGL((fast4_bw_kernel<L, INC>), grid, dim3(kFastThreads), 0, stream, a);
+    // row groups per backward iteration: as many as the registers next to the factors allow
+    constexpr int RB = L <= 8 ? 4 : 2;
+    if (backward) hipLaunchKernelGGL((fast4_bw_kernel<L, INC, RB>), grid, dim3(kFastThreads), 0, stream, a);
     else hipLaunchKernelGGL((fast4_fw_kernel<L, INC, kFast4FwRows>), grid, dim3(kFastThreads), 0, stream, a);
 }
 
@@ -608,7 +610,9 @@ template <typename T, int L, bool INC>
 void launch_fast4g_t(bool backward, const Fast4GArgs &a, dim3 grid, hipStream_t stream)
 {
     constexpr int R = sizeof(T) == 4 ? kFast4FwRows : kFast4GFwRowsComplex;
-    if (backward) hipLaunchKernelGGL((fast4g_bw_kernel<T, L, INC>), grid, dim3(kFastThreads), 0, stream, a);
+    // row groups per backward iteration: what the registers next to the factors allow
+    constexpr int RB = sizeof(T) == 4 ? (L <= 7 ? 4 : 2) : (L <= 6 ? 2 : 1);
+    if (backward) hipLaunchKernelGGL((fast4g_bw_kernel<T, L, INC, RB>), grid, dim3(kFastThreads), 0, stream, a);
     else hipLaunchKernelGGL((fast4g_fw_kernel<T, L, INC, R>), grid, dim3(kFastThreads), 0, stream, a);
 }
 

@@ -8,8 +8,8 @@
 //   pair on phi bits (2,3): row_half_mirror / row_mirror / row_ror:8
 //   pair on lane bits (4,5): ds_swizzle xor 16, ds_bpermute xor 32 / xor 48
 // and pairs (6,7), (8,9) after the LDS transpose into layout B, where they sit on the phi
-// bits.  Each thread keeps its own ROW of the 4x4 factor (forward, d_twiddle) and its own
-// COLUMN (for d_x): 12 instructions per element and radix-4 stage in the backward pass.
+// bits.  Each thread keeps its own ROW of the 4x4 factor (forward) and its own COLUMN
+// (backward: one set of gradient exchanges serves the d_twiddle column and d_x).
 #pragma once
 
 #include "fast.hpp"
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4_fw_kernel(Fast4Args a)
 {
     using P = Plan4<L, INC>;
     constexpr int NS = P::NS, SLOTS = P::SLOTS;
-    __shared__ float lds[P::NSWAP > 0 ? R * kFastRowWords : 1];
+    __shared__ float lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int lane = t & 63;
     const int stack = blockIdx.y;
@@ -142,14 +142,19 @@ __global__ __launch_bounds__(kFastThreads) void fast4_fw_kernel(Fast4Args a)
             v[r] = buf_load<float>(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
         }
     };
+    // Transposes alternate between two buffers, so one barrier each is enough: a wavefront
+    // writes a buffer again only after the barrier of the transpose in between, which every
+    // wavefront reaches after it has read that buffer.
+    int par = 0;
     auto transpose = [&](float (&v)[R], int to_b) {
         const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
-        __syncthreads();  // the previous transpose's reads are done
+        float *buf = lds + par * R * kFastRowWords;
 #pragma unroll
-        for (int r = 0; r < R; ++r) lds[r * kFastRowWords + wr] = v[r];
+        for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
         __syncthreads();
 #pragma unroll
-        for (int r = 0; r < R; ++r) v[r] = lds[r * kFastRowWords + rd];
+        for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];
+        par ^= 1;
     };
 
     float nxt[R];
@@ -181,12 +186,13 @@ __global__ __launch_bounds__(kFastThreads) void fast4_fw_kernel(Fast4Args a)
     }
 }
 
-template <int L, bool INC>
+// R row groups per iteration: their transposes share the barriers.
+template <int L, bool INC, int R>
 __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
 {
     using P = Plan4<L, INC>;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
-    __shared__ float lds[P::NSWAP > 0 ? kFastRowWords : 1];
+    __shared__ float lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int lane = t & 63;
     const int stack = blockIdx.y;
@@ -194,7 +200,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
 
     Factors4<L, INC, true> f;
     f.load(a.tw4 + stack * a.tw_stack_stride, c);
-    float acc[NS][4];  // acc[s][m] = sum g * (x of the partner at mask m) = dT[r][r ^ m]
+    float acc[NS][4];  // acc[s][m] = sum (g of the partner at mask m) * x = dT[r ^ m][r]
     static_for<0, NS>([&](auto S) {
 #pragma unroll
         for (int m = 0; m < 4; ++m) acc[S][m] = 0.0f;
@@ -214,53 +220,81 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
     const int g_thr = g_col >= 0 ? c.slot * g_row + (int)(g_col * a.g_view.se * 4) : kOob;
     const int gi_thr = gi_col >= 0 ? c.slot * gi_row + (int)(gi_col * a.gi_view.se * 4) : kOob;
 
-    auto transpose = [&](float v, int to_b) -> float {
+    int par = 0;   // see fast4_fw_kernel
+    auto transpose = [&](float (&v)[R], int to_b) {
         const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
+        float *buf = lds + par * R * kFastRowWords;
+#pragma unroll
+        for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
         __syncthreads();
-        lds[wr] = v;
-        __syncthreads();
-        return lds[rd];
+#pragma unroll
+        for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];
+        par ^= 1;
     };
     auto row_ok = [&](int grp) { return grp * SLOTS + c.slot < rows_valid; };
+    auto load_rows = [&](int grel, float (&x)[R], float (&g)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            x[r] = buf_load<float>(x_rs, row_ok(grel + r) ? x_thr : kOob, (grel + r) * SLOTS * x_row);
+            g[r] = buf_load<float>(g_rs, row_ok(grel + r) ? g_thr : kOob, (grel + r) * SLOTS * g_row);
+        }
+    };
 
-    float nx = buf_load<float>(x_rs, row_ok(0) ? x_thr : kOob, 0);
-    float ngr = buf_load<float>(g_rs, row_ok(0) ? g_thr : kOob, 0);
-    for (int grel = 0; grel < ng; ++grel) {
-        float v = nx, gv = ngr;
-        nx = buf_load<float>(x_rs, row_ok(grel + 1) ? x_thr : kOob, (grel + 1) * SLOTS * x_row);
-        ngr = buf_load<float>(g_rs, row_ok(grel + 1) ? g_thr : kOob, (grel + 1) * SLOTS * g_row);
-        float act[NS];
+    float nx[R], ngr[R];
+    load_rows(0, nx, ngr);
+    for (int grel = 0; grel < ng; grel += R) {
+        float v[R], gv[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            v[r] = nx[r];
+            gv[r] = ngr[r];
+        }
+        load_rows(grel + R, nx, ngr);
+        float act[NS][R];
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
             constexpr int KQ = P::kind(s);
-            if constexpr (P::layout(s) != P::layout_before(s)) v = transpose(v, P::layout(s));
-            act[s] = v;
-            if constexpr (s + 1 < NS) {
-                float y = f.row[s][0] * v;
-                y = fmaf(f.row[s][1], partner4<KQ, 1>(v, lane), y);
-                y = fmaf(f.row[s][2], partner4<KQ, 2>(v, lane), y);
-                y = fmaf(f.row[s][3], partner4<KQ, 3>(v, lane), y);
-                v = y;
+            if constexpr (P::layout(s) != P::layout_before(s)) transpose(v, P::layout(s));
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                act[s][r] = v[r];
+                if constexpr (s + 1 < NS) {
+                    float y = f.row[s][0] * v[r];
+                    y = fmaf(f.row[s][1], partner4<KQ, 1>(v[r], lane), y);
+                    y = fmaf(f.row[s][2], partner4<KQ, 2>(v[r], lane), y);
+                    y = fmaf(f.row[s][3], partner4<KQ, 3>(v[r], lane), y);
+                    v[r] = y;
+                }
             }
         });
         static_for<0, NS>([&](auto S) {
             constexpr int s = NS - 1 - S;
             constexpr int KQ = P::kind(s);
-            if constexpr (P::layout(s) != P::layout_after(s)) gv = transpose(gv, P::layout(s));
-            const float xs = act[s];
-            fmac_pinned(acc[s][0], gv, xs);
-            fmac_pinned(acc[s][1], gv, partner4<KQ, 1>(xs, lane));
-            fmac_pinned(acc[s][2], gv, partner4<KQ, 2>(xs, lane));
-            fmac_pinned(acc[s][3], gv, partner4<KQ, 3>(xs, lane));
-            // d_x[c] = sum_r T[r][c] g[r]: own column of the factor, partners' gradients
-            float d = f.colm[s][0] * gv;
-            d = fmaf(f.colm[s][1], partner4<KQ, 1>(gv, lane), d);
-            d = fmaf(f.colm[s][2], partner4<KQ, 2>(gv, lane), d);
-            d = fmaf(f.colm[s][3], partner4<KQ, 3>(gv, lane), d);
-            gv = d;
+            if constexpr (P::layout(s) != P::layout_after(s)) transpose(gv, P::layout(s));
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                // one set of exchanges (of the gradient) serves both products: the thread sums
+                // the COLUMN of d_twiddle that belongs to its element, dT[r ^ m][r] += g(partner m) * x,
+                // and d_x[r] = sum_m T[r ^ m][r] g(partner m)
+                const float xs = act[s][r];
+                const float g1 = partner4<KQ, 1>(gv[r], lane);
+                const float g2 = partner4<KQ, 2>(gv[r], lane);
+                const float g3 = partner4<KQ, 3>(gv[r], lane);
+                fmac_pinned(acc[s][0], gv[r], xs);
+                fmac_pinned(acc[s][1], g1, xs);
+                fmac_pinned(acc[s][2], g2, xs);
+                fmac_pinned(acc[s][3], g3, xs);
+                float d = f.colm[s][0] * gv[r];
+                d = fmaf(f.colm[s][1], g1, d);
+                d = fmaf(f.colm[s][2], g2, d);
+                d = fmaf(f.colm[s][3], g3, d);
+                gv[r] = d;
+            }
         });
-        if constexpr (P::layout(0) != 0) gv = transpose(gv, 0);
-        buf_store(gi_rs, row_ok(grel) ? gi_thr : kOob, grel * SLOTS * gi_row, gv);
+        if constexpr (P::layout(0) != 0) transpose(gv, 0);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            buf_store(gi_rs, row_ok(grel + r) ? gi_thr : kOob, (grel + r) * SLOTS * gi_row, gv[r]);
     }
 
     int t2 = t;
@@ -276,9 +310,9 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
         if constexpr (SLOTS == 1) {
             const int r = (e >> b) & 3;
             const int q = ((e >> (b + 2)) << b) | (e & ((1 << b) - 1));
-            float *d = part + (int64_t)s * (4 * n) + q * 16 + r * 4;
+            float *d = part + (int64_t)s * (4 * n) + q * 16 + r;
 #pragma unroll
-            for (int m = 0; m < 4; ++m) d[r ^ m] = acc[s][m];
+            for (int m = 0; m < 4; ++m) d[(r ^ m) * 4] = acc[s][m];
         } else {
             // add the row slots of this workgroup in ascending order, then one thread per entry
             __syncthreads();
@@ -291,7 +325,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
                 const int eo = o >> 2, m = o & 3;
                 const int r = (eo >> b) & 3;
                 const int q = ((eo >> (b + 2)) << b) | (eo & ((1 << b) - 1));
-                part[(int64_t)s * (4 * n) + q * 16 + r * 4 + (r ^ m)] = sum;
+                part[(int64_t)s * (4 * n) + q * 16 + (r ^ m) * 4 + r] = sum;
             }
         }
     });

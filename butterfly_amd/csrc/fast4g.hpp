@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_fw_kernel(Fast4GArgs a)
     using P = Plan4G<L, INC>;
     constexpr int NS = P::NS, NS4 = P::NS4, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
-    __shared__ T lds[P::NSWAP > 0 ? R * kFastRowWords : 1];
+    __shared__ T lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const FastCoords c = fast_coords<L>(t);
@@ -148,14 +148,19 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_fw_kernel(Fast4GArgs a)
             v[r] = buf_load<T>(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
         }
     };
+    // Transposes alternate between two buffers, so one barrier each is enough: a wavefront
+    // writes a buffer again only after the barrier of the transpose in between, which every
+    // wavefront reaches after it has read that buffer.
+    int par = 0;
     auto transpose = [&](T (&v)[R], int to_b) {
         const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
-        __syncthreads();  // the previous transpose's reads are done
+        T *buf = lds + par * R * kFastRowWords;
 #pragma unroll
-        for (int r = 0; r < R; ++r) lds[r * kFastRowWords + wr] = v[r];
+        for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
         __syncthreads();
 #pragma unroll
-        for (int r = 0; r < R; ++r) v[r] = lds[r * kFastRowWords + rd];
+        for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];
+        par ^= 1;
     };
 
     T nxt[R];
@@ -195,15 +200,17 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_fw_kernel(Fast4GArgs a)
     }
 }
 
-template <typename T, int L, bool INC>
+// R row groups per iteration: their transposes share the barriers.
+template <typename T, int L, bool INC, int R>
 __global__ __launch_bounds__(kFastThreads) void fast4g_bw_kernel(Fast4GArgs a)
 {
     using P = Plan4G<L, INC>;
     constexpr int n = 1 << L, NS = P::NS, NS4 = P::NS4, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
-    // one transpose row; the epilogue's slot reduction reuses the same memory
+    // two transpose buffers of R rows; the epilogue's slot reduction reuses the same memory
     constexpr int kRedWords = SLOTS > 1 ? 4 * 1024 : 1;
-    constexpr int kLdsWords = kRedWords > kFastRowWords ? kRedWords : kFastRowWords;
+    constexpr int kRowWords = P::NSWAP > 0 ? 2 * R * kFastRowWords : 1;
+    constexpr int kLdsWords = kRedWords > kRowWords ? kRedWords : kRowWords;
     __shared__ T lds[kLdsWords];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
@@ -235,61 +242,84 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_bw_kernel(Fast4GArgs a)
     const int g_thr = g_col >= 0 ? c.slot * g_row + (int)(g_col * a.g_view.se * EB) : kOob;
     const int gi_thr = gi_col >= 0 ? c.slot * gi_row + (int)(gi_col * a.gi_view.se * EB) : kOob;
 
-    auto transpose = [&](T v, int to_b) -> T {
+    int par = 0;   // see fast4g_fw_kernel
+    auto transpose = [&](T (&v)[R], int to_b) {
         const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
+        T *buf = lds + par * R * kFastRowWords;
+#pragma unroll
+        for (int r = 0; r < R; ++r) buf[r * kFastRowWords + wr] = v[r];
         __syncthreads();
-        lds[wr] = v;
-        __syncthreads();
-        return lds[rd];
+#pragma unroll
+        for (int r = 0; r < R; ++r) v[r] = buf[r * kFastRowWords + rd];
+        par ^= 1;
     };
     auto row_ok = [&](int grp) { return grp * SLOTS + c.slot < rows_valid; };
+    auto load_rows = [&](int grel, T (&x)[R], T (&g)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            x[r] = buf_load<T>(x_rs, row_ok(grel + r) ? x_thr : kOob, (grel + r) * SLOTS * x_row);
+            g[r] = buf_load<T>(g_rs, row_ok(grel + r) ? g_thr : kOob, (grel + r) * SLOTS * g_row);
+        }
+    };
 
-    T nx = buf_load<T>(x_rs, row_ok(0) ? x_thr : kOob, 0);
-    T ngr = buf_load<T>(g_rs, row_ok(0) ? g_thr : kOob, 0);
-    for (int grel = 0; grel < ng; ++grel) {
-        T v = nx, gv = ngr;
-        nx = buf_load<T>(x_rs, row_ok(grel + 1) ? x_thr : kOob, (grel + 1) * SLOTS * x_row);
-        ngr = buf_load<T>(g_rs, row_ok(grel + 1) ? g_thr : kOob, (grel + 1) * SLOTS * g_row);
-        T act[NS];
+    T nx[R], ngr[R];
+    load_rows(0, nx, ngr);
+    for (int grel = 0; grel < ng; grel += R) {
+        T v[R], gv[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            v[r] = nx[r];
+            gv[r] = ngr[r];
+        }
+        load_rows(grel + R, nx, ngr);
+        T act[NS][R];
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
-            if constexpr (P::layout(s) != P::layout_before(s)) v = transpose(v, P::layout(s));
-            act[s] = v;
-            if constexpr (s + 1 < NS) {   // (the 2x2 stage is always last: only radix-4 stages here)
-                constexpr int K0 = P::kind(P::lo(s)), K1 = P::kind(P::lo(s) + 1);
-                T p1, p2, p3;
-                partners4<K0, K1>(v, c.bperm_addr, p1, p2, p3);
-                T y = mul(f.row[s][0], v);
-                y = mac(y, f.row[s][1], p1);
-                y = mac(y, f.row[s][2], p2);
-                y = mac(y, f.row[s][3], p3);
-                v = y;
+            if constexpr (P::layout(s) != P::layout_before(s)) transpose(v, P::layout(s));
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                act[s][r] = v[r];
+                if constexpr (s + 1 < NS) {   // (the 2x2 stage is always last: only radix-4 stages here)
+                    constexpr int K0 = P::kind(P::lo(s)), K1 = P::kind(P::lo(s) + 1);
+                    T p1, p2, p3;
+                    partners4<K0, K1>(v[r], c.bperm_addr, p1, p2, p3);
+                    T y = mul(f.row[s][0], v[r]);
+                    y = mac(y, f.row[s][1], p1);
+                    y = mac(y, f.row[s][2], p2);
+                    y = mac(y, f.row[s][3], p3);
+                    v[r] = y;
+                }
             }
         });
         static_for<0, NS>([&](auto S) {
             constexpr int s = NS - 1 - S;
-            if constexpr (P::layout(s) != P::layout_after(s)) gv = transpose(gv, P::layout(s));
-            const T xs = act[s];
-            if constexpr (s < NS4) {
-                constexpr int K0 = P::kind(P::lo(s)), K1 = P::kind(P::lo(s) + 1);
-                T g1v, g2v, g3v;
-                partners4<K0, K1>(gv, c.bperm_addr, g1v, g2v, g3v);
-                fmac_pinned(acc[s][0], gv, xs);
-                fmac_pinned(acc[s][1], g1v, xs);
-                fmac_pinned(acc[s][2], g2v, xs);
-                fmac_pinned(acc[s][3], g3v, xs);
-                T d = mul(conj_of(f.colm[s][0]), gv);
-                d = macc(d, f.colm[s][1], g1v);
-                d = macc(d, f.colm[s][2], g2v);
-                d = macc(d, f.colm[s][3], g3v);
-                gv = d;
-            } else {
-                constexpr int K = P::kind(P::lo(s));
-                bw_products<K>(self2, cross2, gv, xs, f.ta, f.tc, c.bperm_addr);
+            if constexpr (P::layout(s) != P::layout_after(s)) transpose(gv, P::layout(s));
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const T xs = act[s][r];
+                if constexpr (s < NS4) {
+                    constexpr int K0 = P::kind(P::lo(s)), K1 = P::kind(P::lo(s) + 1);
+                    T g1v, g2v, g3v;
+                    partners4<K0, K1>(gv[r], c.bperm_addr, g1v, g2v, g3v);
+                    fmac_pinned(acc[s][0], gv[r], xs);
+                    fmac_pinned(acc[s][1], g1v, xs);
+                    fmac_pinned(acc[s][2], g2v, xs);
+                    fmac_pinned(acc[s][3], g3v, xs);
+                    T d = mul(conj_of(f.colm[s][0]), gv[r]);
+                    d = macc(d, f.colm[s][1], g1v);
+                    d = macc(d, f.colm[s][2], g2v);
+                    d = macc(d, f.colm[s][3], g3v);
+                    gv[r] = d;
+                } else {
+                    constexpr int K = P::kind(P::lo(s));
+                    bw_products<K>(self2, cross2, gv[r], xs, f.ta, f.tc, c.bperm_addr);
+                }
             }
         });
-        if constexpr (P::layout(0) != 0) gv = transpose(gv, 0);
-        buf_store(gi_rs, row_ok(grel) ? gi_thr : kOob, grel * SLOTS * gi_row, gv);
+        if constexpr (P::layout(0) != 0) transpose(gv, 0);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            buf_store(gi_rs, row_ok(grel + r) ? gi_thr : kOob, (grel + r) * SLOTS * gi_row, gv[r]);
     }
 
     // ---- partial sums of this workgroup, in the layout of the twiddle tensors
