@@ -19,7 +19,7 @@ SYMBOLS = [
     "bf_butterfly_multiply_bw_workspace_bytes", "bf_butterfly_multiply_bw",
     "bf_butterfly_multiply_bias_fw", "bf_butterfly_bias_grad", "bf_butterfly_bias_grad_workspace_bytes",
     "bf_butterfly_multiply_bias_bw", "bf_butterfly_multiply_bias_bw_workspace_bytes",
-    "bf_butterfly_multiply_perm_fw", "bf_butterfly_multiply_perm_bw",
+    "bf_butterfly_multiply_perm_fw", "bf_butterfly_multiply_perm_bw", "bf_describe_plan",
     "bf_butterfly_multiply_base4_fw", "bf_butterfly_multiply_base4_fw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw",
@@ -71,6 +71,7 @@ def lib():
         L.bf_butterfly_multiply_bias_bw_workspace_bytes.restype = sz
         L.bf_butterfly_multiply_perm_fw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_perm_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_describe_plan.argtypes = [pp, ctypes.c_int, ctypes.c_char_p, sz]
         L.bf_butterfly_multiply_base4_fw.argtypes = [pp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_base4_fw_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_base4_fw_workspace_bytes.restype = sz
@@ -189,6 +190,20 @@ def multiply_bias_bw(twiddle, input, grad, increasing_stride):
                                                _ptr(d_twiddle), _ptr(d_input), _ptr(d_bias), _ptr(ws), nbytes,
                                                _stream()))
     return d_twiddle, d_input, d_bias
+
+
+def describe_plan(dtype_code, batch, nstacks, log_n, nblocks, increasing_stride, backward):
+    """The launch plan of a dense base-2 problem as a list of text lines (host only)."""
+    n = 1 << log_n
+    p = Problem()
+    p.dtype, p.increasing_stride = dtype_code, int(increasing_stride)
+    p.batch, p.nstacks, p.log_n, p.nblocks = batch, nstacks, log_n, nblocks
+    p.input_size = p.output_size = n
+    dense = (ctypes.c_int64 * 3)(nstacks * n, n, 1)
+    p.input_stride = p.output_stride = p.d_input_stride = dense
+    buf = ctypes.create_string_buffer(1 << 14)
+    _check(lib().bf_describe_plan(ctypes.byref(p), int(backward), buf, len(buf)))
+    return buf.value.decode().splitlines()
 
 
 def _table(t, n):

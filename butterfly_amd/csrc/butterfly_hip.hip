@@ -9,6 +9,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <cstring>
 #include <mutex>
 #include <string>
 
@@ -297,8 +298,29 @@ struct FastGrid {
     int64_t slots, ngroups, nwg, groups_per_wg;
 };
 
-// Row-group partition of a LOW pass: `lanes` independent (stack, chunk) columns share the CUs.
-FastGrid fast_grid(int64_t batch, int Lk, int64_t lanes, int rows_in_flight, int wg_per_cu)
+constexpr int64_t kNoRowCap = INT64_MAX / 4;
+constexpr int kRowMargin = 8;  // rows a kernel may address past its share (prefetch, rows in flight)
+
+// Rows within reach of 32-bit byte offsets from a workgroup's first row, over all operands of
+// the call (the kernels address every operand relative to that row).
+int64_t row_cap(const bf_problem *p, bool backward)
+{
+    const int64_t n = (int64_t)1 << p->log_n;
+    const double e = (double)elem_bytes(p->dtype);
+    const int64_t dense[3] = {p->nstacks * n, n, 1};
+    const int64_t *strides[4] = {p->input_stride, p->output_stride, dense, backward ? p->d_input_stride : dense};
+    double cap = (double)kNoRowCap;
+    for (const int64_t *st : strides) {
+        if (st[0] <= 0) continue;
+        cap = std::min(cap, (2147483000.0 / e - (double)n * (double)st[2]) / (double)st[0]);
+    }
+    return cap < 0 ? 0 : (int64_t)cap;
+}
+
+// Row-group partition of a LOW pass: `lanes` independent (stack, chunk) columns share the CUs;
+// a workgroup walks at most max_rows rows (more workgroups than compute units if need be).
+FastGrid fast_grid(int64_t batch, int Lk, int64_t lanes, int rows_in_flight, int wg_per_cu,
+                   int64_t max_rows = kNoRowCap)
 {
     FastGrid g;
     g.slots = 1024 >> Lk;
@@ -307,6 +329,8 @@ FastGrid fast_grid(int64_t batch, int Lk, int64_t lanes, int rows_in_flight, int
     const int64_t iters = (g.ngroups + rows_in_flight - 1) / rows_in_flight;
     g.nwg = std::min(want, iters);
     g.groups_per_wg = ((iters + g.nwg - 1) / g.nwg) * rows_in_flight;
+    const int64_t max_groups = ((max_rows / g.slots - kRowMargin) / rows_in_flight) * rows_in_flight;
+    if (max_groups >= rows_in_flight && g.groups_per_wg > max_groups) g.groups_per_wg = max_groups;
     g.nwg = (g.ngroups + g.groups_per_wg - 1) / g.groups_per_wg;
     return g;
 }
@@ -331,12 +355,13 @@ struct HighGrid {
 
 // Row partition of a HIGH pass whose row takes `row_threads` threads (n >> H): about 2048
 // threads per compute unit over all stacks.
-HighGrid high_grid(int64_t batch, int64_t nstacks, int64_t row_threads)
+HighGrid high_grid(int64_t batch, int64_t nstacks, int64_t row_threads, int64_t max_rows = kNoRowCap)
 {
     HighGrid g;
     const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * 2 * 1024 / (nstacks * row_threads));
     g.nparts = std::min(want, batch);
     g.rows_per_wg = (batch + g.nparts - 1) / g.nparts;
+    if (max_rows - kRowMargin >= 1 && g.rows_per_wg > max_rows - kRowMargin) g.rows_per_wg = max_rows - kRowMargin;
     g.nparts = (batch + g.rows_per_wg - 1) / g.rows_per_wg;
     return g;
 }
@@ -345,17 +370,19 @@ HighGrid high_grid(int64_t batch, int64_t nstacks, int64_t row_threads)
 bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
 {
     const int64_t n = (int64_t)1 << p->log_n;
+    const int64_t cap = row_cap(p, backward);
     int64_t rows = 0;
     for (int k = 0; k < pl.npass; ++k) {
         const Pass &q = pl.pass[k];
         if (q.high) {
             // the backward high-bit kernel forms 32-bit offsets from its workgroup's first row
-            if (backward) rows = std::max(rows, high_grid(p->batch, p->nstacks, n >> q.H).rows_per_wg + kHighAhead + 1);
+            if (backward)
+                rows = std::max(rows, high_grid(p->batch, p->nstacks, n >> q.H, cap).rows_per_wg + kHighAhead + 1);
             continue;
         }
         const FastGrid g = q.wide ? wide_grid(p->batch, p->nstacks)
                                   : fast_grid(p->batch, q.L, p->nstacks * pl.chunks, backward ? 1 : fw_rows(p),
-                                              backward ? 1 : kFastFwWgPerCu);
+                                              backward ? 1 : kFastFwWgPerCu, cap);
         rows = std::max(rows, (g.groups_per_wg + kFastFwRows + 2) * g.slots);
     }
     const int64_t dense[3] = {p->nstacks * n, n, 1};
@@ -474,7 +501,7 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
         const View sv = k == first ? in_view : dense;
         const View dv = k == last - 1 ? out_view : dense;
         if (q.high) {
-            const HighGrid g = high_grid(p->batch, p->nstacks, n >> q.H);
+            const HighGrid g = high_grid(p->batch, p->nstacks, n >> q.H, row_cap(p, false));
             HighArgs a = {};
             a.low_bits = q.lb;
             a.tw = tw;
@@ -520,7 +547,8 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
             else hipLaunchKernelGGL((wide_fw_kernel<float, 11, false>), grid, block, 0, stream, a);
             BF_HIP_CHECK(hipGetLastError());
         } else {
-            const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, fw_rows(p), kFastFwWgPerCu);
+            const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, fw_rows(p), kFastFwWgPerCu,
+                                         row_cap(p, false));
             FastFwArgs a = {};
             a.tw = tw;
             a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
@@ -928,8 +956,8 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
         int64_t nparts = 1, slices = 1;  // slices: partial (stage, 2n) slices of the pass that needs most
         for (int k = 0; k < mp.npass; ++k) {
             const Pass &q = mp.pass[k];
-            const int64_t np = q.high ? high_grid(p->batch, p->nstacks, n >> q.H).nparts
-                                      : fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1).nwg;
+            const int64_t np = q.high ? high_grid(p->batch, p->nstacks, n >> q.H, row_cap(p, true)).nparts
+                                      : fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1, row_cap(p, true)).nwg;
             nparts = std::max(nparts, np);
             slices = std::max(slices, np * (q.t1 - q.t0));
         }
@@ -1133,7 +1161,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
             const View giv = k == 0 ? dn_view : dense;
             int64_t nparts = 0;
             if (q.high) {
-                const HighGrid g = high_grid(p->batch, p->nstacks, n >> q.H);
+                const HighGrid g = high_grid(p->batch, p->nstacks, n >> q.H, row_cap(p, true));
                 HighArgs a = {};
                 a.low_bits = q.lb;
                 a.tw = tw2;
@@ -1157,7 +1185,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                                         : launch_high<float>(q, true, a, grid, stream);
                 if (rc) return rc;
             } else {
-                const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1);
+                const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1, row_cap(p, true));
                 FastBwArgs a = {};
                 a.tw = tw2;
                 a.tw_stack_stride = sc.tw2_stack_stride;
@@ -1175,7 +1203,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                 a.ngroups = g.ngroups;
                 a.groups_per_wg = g.groups_per_wg;
                 nparts = g.nwg;
-                if (k == P - 1 && bias_partial && bias_nparts && q.L == 10 && p->dtype == BF_F32) {
+                if (k == P - 1 && bias_partial && bias_nparts && q.L == 10 && p->dtype == BF_F32 && g.nwg <= kNumCU) {
                     a.bias_partial = bias_partial;
                     a.bias_width = p->output_size;
                     *bias_nparts = g.nwg;
@@ -1407,6 +1435,35 @@ int bf_butterfly_multiply_perm_bw(const bf_problem *p, const void *twiddle, cons
                              in_perm, out_index);
     return backward(p, false, twiddle, nullptr, input, grad, d_twiddle, nullptr, d_input, workspace, workspace_bytes,
                     stream, nullptr, nullptr, in_perm, out_index);
+}
+
+// One line per launch group of the base-2 schedule, e.g. "low t=0..10 L=10 nb=1 inc=1 chunks=8".
+int bf_describe_plan(const bf_problem *p, int backward, char *text, size_t capacity)
+{
+    int rc = check_problem(p, backward != 0);
+    if (rc) return rc;
+    if (!text || capacity == 0) return fail(BF_ERR_INVALID, "text buffer is NULL or empty");
+    std::string out;
+    char line[160];
+    const PassPlan mp = build_passes(p, false, backward == 0);
+    if (!mp.ok || !passes_addressable(p, mp, backward != 0)) {
+        out = "generic\n";
+    } else {
+        for (int k = 0; k < mp.npass; ++k) {
+            const Pass &q = mp.pass[k];
+            if (q.high)
+                snprintf(line, sizeof line, "high t=%d..%d lb=%d bits=%d pattern=%d\n", q.t0, q.t1, q.lb, q.H, q.PAT);
+            else if (q.wide)
+                snprintf(line, sizeof line, "wide t=%d..%d L=%d inc=%d\n", q.t0, q.t1, q.L, (int)q.inc);
+            else
+                snprintf(line, sizeof line, "low t=%d..%d L=%d nb=%d inc=%d chunks=%lld\n", q.t0, q.t1, q.L, q.NB,
+                         (int)q.inc, (long long)mp.chunks);
+            out += line;
+        }
+    }
+    if (out.size() + 1 > capacity) return fail(BF_ERR_INVALID, "text buffer of %zu bytes is too small", capacity);
+    memcpy(text, out.c_str(), out.size() + 1);
+    return BF_OK;
 }
 
 int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4, const void *twiddle2,

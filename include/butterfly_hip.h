@@ -140,6 +140,16 @@ int bf_butterfly_multiply_perm_bw(const bf_problem *p, const void *twiddle, cons
                                   void *d_bias, void *workspace, size_t workspace_bytes,
                                   void *stream);
 
+/* Diagnostic, host only (no device call): how the base-2 forward (backward != 0: backward)
+ * call for this problem is cut into launches, one text line per pass in order --
+ *   "low t=A..B L=.. nb=.. inc=.. chunks=.."   stages A..B-1 on bits 0..9, 1024-element chunks
+ *   "wide t=A..B L=.. inc=.."                   one whole block of a 2048 / 4096 row (forward)
+ *   "high t=A..B lb=.. bits=.. pattern=.."      stages on `bits` adjacent bits from bit lb up
+ *   "generic"                                   the LDS fallback kernels
+ * No counterpart in the reference (its launch plan is butterfly_max5_plan,
+ * csrc/cuda/butterfly_cuda.cu:317-345, internal to the operator).                       */
+int bf_describe_plan(const bf_problem *p, int backward, char *text, size_t capacity);
+
 /* Base-4 forward: per block log_n/2 radix-4 stages from twiddle4
  * (S, nb, log_n/2, n/4, 4, 4), then one 2x2 stage from twiddle2 (S, nb, 1, n/2, 2, 2)
  * when log_n is odd (twiddle2 may be NULL when log_n is even).

@@ -174,6 +174,37 @@ def test_long_rows(case):
     assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
 
 
+def test_operands_beyond_two_gib():
+    """Operands of 3 GiB: workgroups address rows with 32-bit offsets from their first row, so
+    the host gives each one few enough rows.  Forward and d_input rows against the oracle on a
+    sample of rows; d_twiddle against the sum of two half-batch calls (each below 2 GiB)."""
+    from butterfly_amd import _capi
+    L, B = 16, 12288
+    n = 1 << L
+    say("big operands", L, B)
+    torch.manual_seed(77)
+    tw = (torch.randn(1, 1, L, n // 2, 2, 2) / 2 ** 0.5).cuda()
+    x = torch.randn(B, 1, n, device="cuda")
+    g = torch.randn(B, 1, n, device="cuda")
+    y = _capi.multiply_fw(tw, x, True)
+    dtw, dx = _capi.multiply_bw(tw, x, g, True)
+    torch.cuda.synchronize()
+    rows = [0, 1, 47, 48, 49, B // 2 - 1, B // 2, B - 2, B - 1] + list(range(6000, 6144, 16))
+    twn = tw.cpu().numpy()
+    xs, gs = x[rows].cpu().numpy(), g[rows].cpu().numpy()
+    y_ref = oracle.butterfly_fw(twn, xs, True)
+    _, dx_ref = oracle.butterfly_bw(twn, xs, gs, True)
+    assert rel_err(y[rows].cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx[rows].cpu().numpy(), dx_ref) < BW_TOL
+    h = B // 2
+    d1, dxa = _capi.multiply_bw(tw, x[:h], g[:h], True)
+    d2, dxb = _capi.multiply_bw(tw, x[h:], g[h:], True)
+    torch.cuda.synchronize()
+    assert torch.equal(dxa, dx[:h]) and torch.equal(dxb, dx[h:])
+    ref = (d1.double() + d2.double())
+    assert ((dtw.double() - ref).abs().max() / ref.abs().max()).item() < BW_TOL
+
+
 COMPLEX_FAST_CASES = [
     # B, S, L, nb, I, O, inc
     (37, 2, 1, 2, None, None, True),

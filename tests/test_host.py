@@ -246,3 +246,68 @@ def test_permutation_routing_and_helpers_on_the_host():
     assert not permutation.is_2x2_block_diag(np.ones((4, 4)))
     with pytest.raises(ValueError):
         permutation.perm2butterfly(np.array([0, 0, 1]))
+
+
+def _parse_plan(lines):
+    out = []
+    for line in lines:
+        kind, *fields = line.split()
+        d = {"kind": kind}
+        for f in fields:
+            k, v = f.split("=")
+            d[k] = tuple(int(x) for x in v.split("..")) if ".." in v else int(v)
+        out.append(d)
+    return out
+
+
+def test_launch_plans_cover_every_stage_once():
+    """bf_describe_plan (host only): for every row length up to 2^24, both dtypes, both stride
+    orders, forward and backward, the passes cover the stage list exactly once in order; low
+    passes hold whole blocks of ten low bits; a high pass works on at most three adjacent bits
+    and only on stages of exactly those bits; the bit groups tile bits 10..L-1."""
+    from butterfly_amd import _capi
+    for cplx in (0, 1):
+        for L in range(1, 25):
+            for nb in (1, 2, 3):
+                for inc in (True, False):
+                    for backward in (False, True):
+                        batch = 64 if L < 20 else 3
+                        plan = _parse_plan(_capi.describe_plan(cplx, batch, 1, L, nb, inc, backward))
+                        key = (cplx, L, nb, inc, backward)
+                        assert plan and plan[0]["kind"] != "generic", key
+                        bits = []
+                        for k in range(nb):
+                            up = inc != (k % 2 == 1)
+                            bits += list(range(L)) if up else list(range(L - 1, -1, -1))
+                        t = 0
+                        groups = set()
+                        for q in plan:
+                            a, b = q["t"]
+                            assert a == t and b > a, key
+                            t = b
+                            stage_bits = bits[a:b]
+                            if q["kind"] == "low":
+                                assert q["L"] == min(L, 10) and b - a == q["L"] * q["nb"], key
+                                assert all(x < 10 for x in stage_bits), key
+                                assert q["chunks"] == (1 << max(0, L - 10)), key
+                                assert q["nb"] <= (1 if cplx else 2), key
+                                assert q["inc"] == int(stage_bits[0] == 0 and q["L"] > 1 or (q["L"] == 1 and inc != ((a // L) % 2 == 1))), key
+                            elif q["kind"] == "wide":
+                                assert not backward and L in (11, 12) and b - a == L, key
+                            else:
+                                lb, h = q["lb"], q["bits"]
+                                assert q["kind"] == "high" and lb >= 10 and 1 <= h <= (2 if cplx else 3), key
+                                assert all(lb <= x < lb + h for x in stage_bits), key
+                                assert b - a <= (3 if h == 3 else 2 * h), key
+                                for s, x in enumerate(stage_bits):
+                                    assert (q["pattern"] >> (2 * s)) & 3 == x - lb, key
+                                groups.add((lb, h))
+                        assert t == len(bits), key
+                        if groups:
+                            covered = sorted(x for lb, h in groups for x in range(lb, lb + h))
+                            assert covered == list(range(10, L)), key
+    # the configurations the benchmark is quoted on
+    assert _capi.describe_plan(0, 16384, 1, 10, 2, False, True) == ["low t=0..20 L=10 nb=2 inc=0 chunks=1"]
+    assert [l.split()[0] for l in _capi.describe_plan(0, 32768, 1, 12, 2, True, False)] == ["wide", "wide"]
+    assert [l.split()[0] for l in _capi.describe_plan(0, 32768, 1, 12, 2, True, True)] == ["low", "high", "low"]
+    assert [l.split()[0] for l in _capi.describe_plan(0, 2048, 1, 13, 1, True, True)] == ["low", "high"]
