@@ -204,6 +204,16 @@ int stage_bit(const bf_problem *p, int t)
     return inc ? idx : L - 1 - idx;
 }
 
+// Rows (over all stacks) from which the whole-block forward kernel of wide.hpp beats the
+// chunked + high-bit passes: each of its workgroups first loads the factors of a whole block
+// (up to 96 registers per thread), which only pays off over enough rows.  Measured crossovers.
+int64_t wide_min_rows(const bf_problem *p)
+{
+    if (p->log_n == 12) return p->nblocks == 1 ? 2048 : 8192;
+    if (p->dtype == BF_C64) return 256;
+    return p->nblocks == 1 ? 0 : 1024;
+}
+
 PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false)
 {
     PassPlan pl;
@@ -225,7 +235,8 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             q.L = L;
             q.inc = (p->increasing_stride != 0) != ((k & 1) != 0);
         }
-    } else if (L <= 12 && forward_only && (p->dtype == BF_F32 || L == 11)) {
+    } else if (L <= 12 && forward_only && (p->dtype == BF_F32 || L == 11) &&
+               p->batch * p->nstacks >= wide_min_rows(p)) {
         for (int k = 0; k < p->nblocks; ++k) {
             if (pl.npass == kMaxPasses) return pl;
             Pass &q = pl.pass[pl.npass++];

@@ -205,6 +205,34 @@ def test_operands_beyond_two_gib():
     assert ((dtw.double() - ref).abs().max() / ref.abs().max()).item() < BW_TOL
 
 
+WIDE_CASES = [
+    # dtype, B, S, L, nb, I, O, inc -- enough rows for the whole-block forward kernel (the host
+    # picks it from a row count on; below that the chunked passes run)
+    (np.float32, 2100, 1, 12, 1, None, None, True),
+    (np.float32, 1050, 2, 12, 1, 4000, 4090, False),
+    (np.float32, 8200, 1, 12, 2, None, None, True),
+    (np.float32, 1100, 1, 11, 2, None, 2047, False),
+    (np.float32, 3, 1, 11, 1, None, None, True),
+    (np.complex64, 260, 1, 11, 1, None, None, True),
+    (np.complex64, 130, 2, 11, 2, 2000, None, False),
+]
+
+
+@pytest.mark.parametrize("case", WIDE_CASES, ids=lambda c: f"{np.dtype(c[0]).name}-B{c[1]}-S{c[2]}-L{c[3]}-nb{c[4]}-I{c[5]}-O{c[6]}-inc{int(c[7])}")
+def test_whole_block_forward_kernel(case):
+    from butterfly_amd import _capi
+    dtype, B, S, L, nb, I, O, inc = case
+    say("wide case", case)
+    plan = _capi.describe_plan(int(np.dtype(dtype).kind == "c"), B, S, L, nb, inc, False)
+    assert all(line.startswith("wide") for line in plan), plan
+    rng = np.random.default_rng(3100 + L * 13 + nb)
+    tw, x, _ = make_case(rng, dtype, B, S, L, nb, I, O)
+    y_ref = oracle.butterfly_fw(tw, x, inc, O)
+    y = _capi.multiply_fw(dev(tw), dev(x), inc, O)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+
+
 COMPLEX_FAST_CASES = [
     # B, S, L, nb, I, O, inc
     (37, 2, 1, 2, None, None, True),
@@ -512,6 +540,8 @@ BIAS_CASES = [
     (np.float32, 11, 1, 13, 1, None, 8000, True),
     (np.float32, 5000, 1, 10, 1, None, 1000, True),
     (np.float32, 2100, 1, 12, 2, None, 4090, True),
+    (np.float32, 40, 1, 11, 1, None, 2000, True),        # whole-block forward kernel at any batch
+    (np.complex64, 300, 1, 11, 1, None, None, False),
 ]
 
 
@@ -588,6 +618,8 @@ PERM_CASES = [
     (np.complex64, 9, 1, 12, 1, None, 4000, True, "o", False),
     (np.float32, 11, 1, 13, 1, None, 8000, True, "io", True),
     (np.float32, 7, 1, 14, 2, 16000, None, False, "io", False),
+    (np.float32, 40, 1, 11, 1, None, 2000, True, "io", True),      # whole-block forward kernel
+    (np.complex64, 300, 1, 11, 1, None, None, False, "io", False),
 ]
 
 
