@@ -177,6 +177,8 @@ bool span_ok(const int64_t stride[3], int64_t rows, int64_t width, size_t elem)
 }
 
 constexpr int kMaxPasses = 96;
+constexpr int kSpanMaxBits = 5;    // widest span: tiles of 32 consecutive elements per setting of the span's bits
+constexpr int kSpanFromBits = 3;   // rows with fewer bits above 10 keep the streaming passes of high.hpp
 constexpr int kMaxLogN = 24;  // the chunk index of the register-resident kernels travels in blockIdx.z
 
 struct Pass {
@@ -187,6 +189,8 @@ struct Pass {
     bool inc;
     int H, NST, PAT;  // HIGH: H adjacent bits from `lb` up, NST stages, bits 2s, 2s+1 of PAT = which of them stage s pairs
     int lb;
+    bool span;      // LOW kernels on tiles of a span of H high bits from `lb` up (SpanPlan<H, mode>), L = 10, NB = 1
+    int mode;       // 0: one sweep up, 1: one sweep down, 2: up then down
 };
 
 struct PassPlan {
@@ -248,18 +252,18 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             q.inc = (p->increasing_stride != 0) != ((k & 1) != 0);
         }
     } else {
-        // bits 0..9: the register-resident kernels on 1024-element chunks; bits from 10 up: one
-        // streaming pass per group of adjacent bits.  Groups of two; float rows take groups of
-        // three (eight elements per thread, a slower kernel) where that saves a pass.
+        // bits 0..9: the register-resident kernels on 1024-element chunks.  One or two bits above
+        // them (rows of 2048 / 4096): one streaming pass of high.hpp.  More: spans of up to
+        // kSpanMaxBits adjacent bits, as equal as possible, each one pass of the register-resident
+        // kernels over tiles (SpanPlan) -- e.g. n = 2^20: [10..14] [15..19].
         pl.chunks = (int64_t)1 << (L - 10);
         const int hbits = L - 10;
-        const int ngroups3 = p->dtype == BF_F32 ? (hbits + 2) / 3 : 0;   // passes with groups of up to three
-        const int ngroups2 = (hbits + 1) / 2;
-        const int nthree = (ngroups3 > 0 && ngroups3 < ngroups2) ? hbits - 2 * ngroups3 : 0;
+        const bool use_span = hbits >= kSpanFromBits;
+        const int nspans = (hbits + kSpanMaxBits - 1) / kSpanMaxBits;
         int group_lb[16], group_bits[16], ngroups = 0;
         for (int b = 10; b < L; ++ngroups) {
             group_lb[ngroups] = b;
-            group_bits[ngroups] = std::min(ngroups < nthree ? 3 : 2, L - b);
+            group_bits[ngroups] = use_span ? hbits / nspans + (ngroups < hbits % nspans ? 1 : 0) : hbits;
             b += group_bits[ngroups];
         }
         auto group_of = [&](int bit) {
@@ -276,16 +280,25 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             q.t0 = t;
             const int grp = group_of(stage_bit(p, t));
             const bool high = grp >= 0;
-            // a group of three bits takes one sweep over them per pass (its factors and sums
-            // fill the registers); smaller groups also take the way back at a block boundary
+            // a group also takes the way back down where two blocks meet in the row's top bits
             const int lb = high ? group_lb[grp] : 0;
             const int H = high ? group_bits[grp] : 0;
-            const int cap = high ? (H == 3 ? 3 : 2 * H) : 10 * max_nb;
+            const int cap = high ? 2 * H : 10 * max_nb;
             int u = t;
             while (u < NS && group_of(stage_bit(p, u)) == grp && u - t < cap) ++u;
             q.t1 = u;
-            q.high = high;
-            if (high) {
+            q.high = high && !use_span;
+            if (high && use_span) {
+                q.span = true;
+                q.L = 10;
+                q.NB = 1;
+                q.lb = lb;
+                q.H = H;
+                q.NST = u - t;
+                if (q.NST != H && q.NST != 2 * H) return pl;
+                q.mode = q.NST == 2 * H ? 2 : (stage_bit(p, t) == lb ? 0 : 1);
+                q.inc = q.mode != 1;
+            } else if (high) {
                 q.lb = lb;
                 q.H = H;
                 q.NST = u - t;
@@ -409,12 +422,12 @@ void launch_fast_fw_t(bool cplx, const FastFwArgs &a, dim3 grid, hipStream_t str
 {
     if constexpr (NB == 1) {
         if (cplx) {
-            hipLaunchKernelGGL((fast_fw_kernel<float2, L, NB, INC, kFastFwRowsComplex>), grid, dim3(kFastThreads), 0,
+            hipLaunchKernelGGL((fast_fw_kernel<float2, FastPlan<L, NB, INC>, kFastFwRowsComplex>), grid, dim3(kFastThreads), 0,
                                stream, a);
             return;
         }
     }
-    hipLaunchKernelGGL((fast_fw_kernel<float, L, NB, INC, kFastFwRows>), grid, dim3(kFastThreads), 0, stream, a);
+    hipLaunchKernelGGL((fast_fw_kernel<float, FastPlan<L, NB, INC>, kFastFwRows>), grid, dim3(kFastThreads), 0, stream, a);
 }
 
 template <int L, int NB, bool INC>
@@ -422,17 +435,51 @@ void launch_fast_bw_t(bool cplx, bool two_rows, const FastBwArgs &a, dim3 grid, 
 {
     if constexpr (NB == 1) {
         if (cplx) {
-            hipLaunchKernelGGL((fast_bw_kernel<float2, L, NB, INC>), grid, dim3(kFastThreads), 0, stream, a);
+            hipLaunchKernelGGL((fast_bw_kernel<float2, FastPlan<L, NB, INC>>), grid, dim3(kFastThreads), 0, stream, a);
             return;
         }
         if constexpr (L >= 7) {
             if (two_rows) {
-                hipLaunchKernelGGL((fast_bw_kernel<float, L, NB, INC, 2>), grid, dim3(kFastThreads), 0, stream, a);
+                hipLaunchKernelGGL((fast_bw_kernel<float, FastPlan<L, NB, INC>, 2>), grid, dim3(kFastThreads), 0, stream, a);
                 return;
             }
         }
     }
-    hipLaunchKernelGGL((fast_bw_kernel<float, L, NB, INC>), grid, dim3(kFastThreads), 0, stream, a);
+    hipLaunchKernelGGL((fast_bw_kernel<float, FastPlan<L, NB, INC>>), grid, dim3(kFastThreads), 0, stream, a);
+}
+
+// SpanPlan passes: the LOW kernels on the tiles of a span of q.H high bits.
+template <int H, int MODE>
+void launch_span_t(bool cplx, bool backward, bool two_rows, const FastFwArgs *fw, const FastBwArgs *bw, dim3 grid,
+                   hipStream_t stream)
+{
+    using P = SpanPlan<H, MODE>;
+    const dim3 block(kFastThreads);
+    if (!backward) {
+        if (cplx) hipLaunchKernelGGL((fast_fw_kernel<float2, P, kFastFwRowsComplex>), grid, block, 0, stream, *fw);
+        else hipLaunchKernelGGL((fast_fw_kernel<float, P, kFastFwRows>), grid, block, 0, stream, *fw);
+    } else if (cplx) {
+        hipLaunchKernelGGL((fast_bw_kernel<float2, P>), grid, block, 0, stream, *bw);
+    } else if (two_rows) {
+        hipLaunchKernelGGL((fast_bw_kernel<float, P, 2>), grid, block, 0, stream, *bw);
+    } else {
+        hipLaunchKernelGGL((fast_bw_kernel<float, P>), grid, block, 0, stream, *bw);
+    }
+}
+
+int launch_span(bool cplx, const Pass &q, bool backward, bool two_rows, const FastFwArgs *fw, const FastBwArgs *bw,
+                dim3 grid, hipStream_t stream)
+{
+#define BF_SPAN_CASES(HH)                                                                          \
+    case HH * 3 + 0: launch_span_t<HH, 0>(cplx, backward, two_rows, fw, bw, grid, stream); break;   \
+    case HH * 3 + 1: launch_span_t<HH, 1>(cplx, backward, two_rows, fw, bw, grid, stream); break;   \
+    case HH * 3 + 2: launch_span_t<HH, 2>(cplx, backward, two_rows, fw, bw, grid, stream); break;
+    switch (q.H * 3 + q.mode) {
+        BF_SPAN_CASES(2) BF_SPAN_CASES(3) BF_SPAN_CASES(4) BF_SPAN_CASES(5)
+        default: return fail(BF_ERR_UNSUPPORTED, "no kernel for a span of %d bits", q.H);
+    }
+#undef BF_SPAN_CASES
+    return BF_OK;
 }
 
 #define BF_FAST_DISPATCH(FN, Q, ...)                                                     \
@@ -458,9 +505,8 @@ void launch_high_t(bool backward, const HighArgs &a, dim3 grid, hipStream_t stre
 {
     if (backward) {
         // float leaves room for 1024 threads (128 registers each), complex64 for 512
-        // grid.z arrives as the threads a row takes; three bits per pass (float only) hold eight
-        // elements and 48 + 48 factor entries and sums per thread: 256 threads
-        constexpr int THREADS = H == 3 ? 256 : (sizeof(T) == 4 ? 1024 : 512);
+        // grid.z arrives as the threads a row takes
+        constexpr int THREADS = sizeof(T) == 4 ? 1024 : 512;
         grid.z = grid.z / THREADS;
         hipLaunchKernelGGL((high_bw_kernel<T, H, NST, PAT, THREADS>), grid, dim3(THREADS), 0, stream, a);
     } else
@@ -477,12 +523,6 @@ int launch_high(const Pass &q, bool backward, const HighArgs &a, dim3 grid, hipS
         case 2 * 1000 + 2 * 100 + 4: launch_high_t<T, 2, 2, 4>(backward, a, grid, stream); break;    // bits 0, 1 of the group
         case 2 * 1000 + 2 * 100 + 1: launch_high_t<T, 2, 2, 1>(backward, a, grid, stream); break;    // 1, 0
         case 2 * 1000 + 4 * 100 + 20: launch_high_t<T, 2, 4, 20>(backward, a, grid, stream); break;  // 0, 1, 1, 0
-        case 3 * 1000 + 3 * 100 + 36:                                                                // 0, 1, 2
-            if constexpr (sizeof(T) == 4) { launch_high_t<T, 3, 3, 36>(backward, a, grid, stream); break; }
-            return fail(BF_ERR_UNSUPPORTED, "no kernel for this high-bit stage pattern");
-        case 3 * 1000 + 3 * 100 + 6:                                                                 // 2, 1, 0
-            if constexpr (sizeof(T) == 4) { launch_high_t<T, 3, 3, 6>(backward, a, grid, stream); break; }
-            return fail(BF_ERR_UNSUPPORTED, "no kernel for this high-bit stage pattern");
         default: return fail(BF_ERR_UNSUPPORTED, "no kernel for this high-bit stage pattern");
     }
     BF_HIP_CHECK(hipGetLastError());
@@ -577,7 +617,13 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
                 if (bias_done) *bias_done = true;
             }
             const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)pl.chunks);
-            BF_FAST_DISPATCH(launch_fast_fw_t, q, p->dtype == BF_C64, a, grid, stream);
+            if (q.span) {
+                a.low_bits = q.lb;
+                const int rc = launch_span(p->dtype == BF_C64, q, false, false, &a, nullptr, grid, stream);
+                if (rc) return rc;
+            } else {
+                BF_FAST_DISPATCH(launch_fast_fw_t, q, p->dtype == BF_C64, a, grid, stream);
+            }
             BF_HIP_CHECK(hipGetLastError());
         }
     }
@@ -1221,7 +1267,13 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                 }
                 const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)mp.chunks);
                 // two row groups in flight once a workgroup has enough of them to fill the pipeline
-                BF_FAST_DISPATCH(launch_fast_bw_t, q, p->dtype == BF_C64, g.groups_per_wg >= 16, a, grid, stream);
+                if (q.span) {
+                    a.low_bits = q.lb;
+                    rc = launch_span(p->dtype == BF_C64, q, true, g.groups_per_wg >= 16, nullptr, &a, grid, stream);
+                    if (rc) return rc;
+                } else {
+                    BF_FAST_DISPATCH(launch_fast_bw_t, q, p->dtype == BF_C64, g.groups_per_wg >= 16, a, grid, stream);
+                }
                 BF_HIP_CHECK(hipGetLastError());
             }
             rc = launch_reduce(p, sc, q.t0, q.t1, nparts, ws + pl.off_partials, pl.slot, d_tw2, d_tw4, stream);
@@ -1466,6 +1518,9 @@ int bf_describe_plan(const bf_problem *p, int backward, char *text, size_t capac
                 snprintf(line, sizeof line, "high t=%d..%d lb=%d bits=%d pattern=%d\n", q.t0, q.t1, q.lb, q.H, q.PAT);
             else if (q.wide)
                 snprintf(line, sizeof line, "wide t=%d..%d L=%d inc=%d\n", q.t0, q.t1, q.L, (int)q.inc);
+            else if (q.span)
+                snprintf(line, sizeof line, "span t=%d..%d lb=%d bits=%d mode=%d tiles=%lld\n", q.t0, q.t1, q.lb, q.H,
+                         q.mode, (long long)mp.chunks);
             else
                 snprintf(line, sizeof line, "low t=%d..%d L=%d nb=%d inc=%d chunks=%lld\n", q.t0, q.t1, q.L, q.NB,
                          (int)q.inc, (long long)mp.chunks);

@@ -47,28 +47,18 @@ __host__ __device__ constexpr int phi4(int l)
     return ((l & 1) ? 1 : 0) ^ ((l & 2) ? 2 : 0) ^ ((l & 4) ? 7 : 0) ^ ((l & 8) ? 12 : 0);
 }
 
-template <int L, int NB, bool INC>
-struct FastPlan {
-    static constexpr int NS = L * NB;
-    static constexpr int NSWAP = L > 6 ? L - 6 : 0;  // element bits exchanged between layouts
-    static constexpr int SLOTS = 1024 >> L;          // rows a workgroup holds at once
-
-    // element bit paired by stage s
-    static constexpr int bit(int s)
-    {
-        const int k = s / L, idx = s % L;
-        const bool inc = INC != ((k & 1) != 0);
-        return inc ? idx : L - 1 - idx;
-    }
+// What the kernels ask of a plan, derived from its stage -> bit map (D::bit, D::NS, D::LOG).
+template <typename D>
+struct PlanOps {
     // layout (0 = A, 1 = B) in which stage s runs: bits >= 6 need B, bits < NSWAP need A,
     // anything else stays where the previous stage left the data.
     static constexpr int layout(int s)
     {
         int cur = 0;
         for (int j = 0; j <= s; ++j) {
-            const int b = bit(j);
+            const int b = D::bit(j);
             if (b >= 6) cur = 1;
-            else if (b < NSWAP) cur = 0;
+            else if (b < D::NSWAP) cur = 0;
         }
         return cur;
     }
@@ -77,7 +67,7 @@ struct FastPlan {
     // exchange kind: 0..3 DPP pattern for phi bit, 4 swizzle xor 16, 5 bpermute xor 32
     static constexpr int kind(int s)
     {
-        const int b = bit(s);
+        const int b = D::bit(s);
         return b >= 6 ? b - 6 : b;
     }
     // LDS transposes performed before stage s of a forward walk (for buffer parity)
@@ -91,8 +81,66 @@ struct FastPlan {
     }
     static constexpr int fw_transposes_total(int start = 0)
     {
-        int c = fw_transposes_before(NS, start);
-        return c + (layout(NS - 1) != 0 ? 1 : 0);
+        int c = fw_transposes_before(D::NS, start);
+        return c + (layout(D::NS - 1) != 0 ? 1 : 0);
+    }
+};
+
+// NB whole blocks of a row (or 1024-element chunk of a row) of 2^L elements.
+template <int L, int NB, bool INC>
+struct FastPlan : PlanOps<FastPlan<L, NB, INC>> {
+    static constexpr int LOG = L;
+    static constexpr int NS = L * NB;
+    static constexpr int NSWAP = L > 6 ? L - 6 : 0;  // element bits exchanged between layouts
+    static constexpr int SLOTS = 1024 >> L;          // rows a workgroup holds at once
+
+    // element bit paired by stage s
+    static constexpr int bit(int s)
+    {
+        const int k = s / L, idx = s % L;
+        const bool inc = INC != ((k & 1) != 0);
+        return inc ? idx : L - 1 - idx;
+    }
+    // column of the full row behind element e of chunk `tile`; pair index (in a stage's factor
+    // slice) of the pair that element belongs to = pair_base(tile) + pair_index(...)
+    __device__ static __forceinline__ int column(int tile, int e, int) { return (tile << L) + e; }
+    __device__ static __forceinline__ int64_t pair_base(int tile) { return (int64_t)tile * (1 << (L - 1)); }
+    __device__ static __forceinline__ int pair_index(int, int e, int s_bit, int)
+    {
+        return ((e >> (s_bit + 1)) << s_bit) | (e & ((1 << s_bit) - 1));
+    }
+};
+
+// The stages on H adjacent high bits [lb, lb + H) of a long row, run by the same kernels: a
+// workgroup takes a tile of 1024 elements made of 2^(10 - H) consecutive elements (virtual bits
+// 0 .. 9 - H) for each of the 2^H settings of the high bits (virtual bits 10 - H .. 9); the
+// tile index enumerates all other bits.  MODE 0: one sweep up (lb, lb + 1, ...), 1: one sweep
+// down, 2: up then down (two blocks meeting in the row's top bits).
+template <int H, int MODE>
+struct SpanPlan : PlanOps<SpanPlan<H, MODE>> {
+    static_assert(H >= 1 && H <= 6, "tiles keep at least 16 consecutive elements");
+    static constexpr int LOG = 10;
+    static constexpr int NS = MODE == 2 ? 2 * H : H;
+    static constexpr int NSWAP = 4;
+    static constexpr int SLOTS = 1;
+    static constexpr int bit(int s)
+    {
+        const bool up = MODE == 0 || (MODE == 2 && s < H);
+        const int idx = s % H;
+        return 10 - H + (up ? idx : H - 1 - idx);
+    }
+    __device__ static __forceinline__ int column(int tile, int e, int lb)
+    {
+        const int cb = lb - (10 - H);   // tile bits that sit below the span
+        const int lo = e & ((1 << (10 - H)) - 1), gp = e >> (10 - H);
+        return lo | ((tile & ((1 << cb) - 1)) << (10 - H)) | (gp << lb) | ((tile >> cb) << (lb + H));
+    }
+    __device__ static __forceinline__ int64_t pair_base(int) { return 0; }
+    __device__ static __forceinline__ int pair_index(int tile, int e, int s_bit, int lb)
+    {
+        const int col = column(tile, e, lb);
+        const int pb = lb + s_bit - (10 - H);
+        return ((col >> (pb + 1)) << pb) | (col & ((1 << pb) - 1));
     }
 };
 
@@ -322,26 +370,25 @@ struct FastFwArgs {
     int64_t ngroups;           // ceil(batch / SLOTS)
     int64_t groups_per_wg;
     const void *bias;          // NULL, or (S, out_view.width) dense: added to every output row
+    int low_bits;              // SpanPlan passes: position of the lowest high bit of the span
 };
 
 // Loads the factor entries each thread needs for every stage: its row (ta, tb) and, for the
 // backward kernel, the off-diagonal entry of its column (tc).
-template <typename T, int L, int NB, bool INC>
+template <typename T, typename P>
 __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, int64_t stage_stride,
-                                             const int (&tw_stage)[kFastMaxStages], int chunk,
-                                             const FastCoords &c, T (&ta)[L * NB], T (&tb)[L * NB],
-                                             T (&tc)[L * NB], bool want_tc)
+                                             const int (&tw_stage)[kFastMaxStages], int chunk, int low_bits,
+                                             const FastCoords &c, T (&ta)[P::NS], T (&tb)[P::NS],
+                                             T (&tc)[P::NS], bool want_tc)
 {
-    using P = FastPlan<L, NB, INC>;
-    constexpr int n = 1 << L;
-    const T *twp = reinterpret_cast<const T *>(tw) + stack_off + (int64_t)chunk * (n / 2) * 4;
+    const T *twp = reinterpret_cast<const T *>(tw) + stack_off + P::pair_base(chunk) * 4;
     static_for<0, P::NS>([&](auto S) {
         constexpr int s = S;
         constexpr int bit = P::bit(s);
         constexpr int lay = P::layout(s);
         const int e = lay ? c.eB : c.eA;
         const int r = (e >> bit) & 1;
-        const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
+        const int i = P::pair_index(chunk, e, bit, low_bits);
         const T *Tm = twp + tw_stage[s] * stage_stride + i * 4;
         ta[s] = Tm[3 * r];   // T[r][r]
         tb[s] = Tm[r + 1];   // T[r][1 - r]
@@ -384,10 +431,12 @@ __device__ __forceinline__ void transpose_rows(T *buf, int wr, int rd, T (&v)[R]
 #ifndef BF_FAST_FW_WAVES
 #define BF_FAST_FW_WAVES 4
 #endif
-template <typename T, int L, int NB, bool INC, int R>
+// P: FastPlan<L, NB, INC> (whole blocks of a row or chunk) or SpanPlan<H, MODE> (a span of high
+// bits of a long row; gridDim.z = n / 1024 tiles).
+template <typename T, typename P, int R>
 __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel(FastFwArgs a)
 {
-    using P = FastPlan<L, NB, INC>;
+    constexpr int L = P::LOG;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
     // float rows are fetched straight into LDS, two iterations (2 R row groups) ahead, and the
@@ -401,11 +450,11 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
     const FastCoords c = fast_coords<L>(t);
-    const int col = (chunk << L) + c.eA;  // column of this thread's element in the full row
+    const int col = P::column(chunk, c.eA, a.low_bits);  // column of this thread's element in the full row
 
     T ta[NS], tb[NS], tc_unused[NS];
-    load_factors<T, L, NB, INC>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, c, ta, tb,
-                                tc_unused, false);
+    load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb,
+                       tc_unused, false);
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
@@ -435,7 +484,7 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     // LDS flavour: lane l of wavefront w fetches element 64 w + l of each row group, which lands
     // at the padded word 65 w + l of the group's slot; `set` alternates between iterations
     const BufDesc in_desc = make_desc(in_base);
-    const int slot_d = t >> L, col_d = (chunk << L) + (t & (n - 1));
+    const int slot_d = t >> L, col_d = P::column(chunk, t & (n - 1), a.low_bits);
     const int64_t in_col_d = view_col(a.in_view, col_d);
     const int in_dma = in_col_d >= 0 ? slot_d * in_row + (int)(in_col_d * a.in_view.se * EB) : kOob;
     const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
@@ -530,11 +579,13 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     if constexpr (DIRECT) wait_rows_in_lds<0>();  // requests past the last group (they fetch nothing)
 }
 
+
 struct FastBwArgs {
     const void *tw;
     int64_t tw_stack_stride;
     int64_t tw_stage_stride;
     int tw_stage[kFastMaxStages];
+    int low_bits;              // SpanPlan passes: position of the lowest high bit of the span
     int64_t partial_slot;      // scalars per stage in a partial slice: 2 * n_full
     const void *x_in;
     View x_view;
@@ -561,9 +612,8 @@ struct FastBwArgs {
 //
 // DIRECT: the operands arrive in LDS (see fast_bw_kernel) and each walk starts in the layout
 // of its first stage; otherwise they arrive in registers in layout A.
-template <int L, int NB, bool INC, bool DIRECT>
+template <typename P, bool DIRECT>
 struct BwPipe {
-    using P = FastPlan<L, NB, INC>;
     static constexpr int NS = P::NS;
     static constexpr int SF = DIRECT ? P::layout(0) : 0;       // layout the forward walk starts in
     static constexpr int SB = DIRECT ? P::layout(NS - 1) : 0;  // layout the reverse walk starts in
@@ -653,16 +703,16 @@ __device__ __forceinline__ void get_rows(const T *base, int idx, T (&v)[R])
 // R: row groups in flight per walk.  Two are possible where one block of float factors
 // leaves half of the registers free; each barrier and each LDS round trip then serves two
 // rows, and every thread runs four independent dependency chains instead of two.
-template <typename T, int L, int NB, bool INC, int R = 1>
+template <typename T, typename P, int R = 1>
 __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 {
-    using P = FastPlan<L, NB, INC>;
+    constexpr int L = P::LOG;
     constexpr int W = (int)sizeof(T) / 4;
     static_assert(R == 1 || (R == 2 && W == 1), "two row groups in flight: float only");
     // float rows are fetched straight into LDS; complex64 has no LDS to spare for that at
     // 9-10 stages and fetches into registers
     constexpr bool DIRECT = W == 1;
-    using Q = BwPipe<L, NB, INC, DIRECT>;
+    using Q = BwPipe<P, DIRECT>;
     using Pair = typename PairOf<T>::type;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
@@ -687,10 +737,10 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
     const FastCoords c = fast_coords<L>(t);
-    const int col = (chunk << L) + c.eA;  // column of this thread's element in the full row
+    const int col = P::column(chunk, c.eA, a.low_bits);  // column of this thread's element in the full row
 
     T ta[NS], tb[NS], tc[NS], acc_self[NS], acc_cross[NS];
-    load_factors<T, L, NB, INC>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, c, ta, tb, tc,
+    load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb, tc,
                                 COL);
     static_for<0, NS>([&](auto S) {
         acc_self[S] = zero_of(T());
@@ -738,7 +788,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // --- operand fetch, LDS flavour: lane l of wavefront w fetches element 64 w + l of the row
     // group, which lands at the padded word 65 w + l of the slot
     const BufDesc x_desc = make_desc(x_base), g_desc = make_desc(g_base);
-    const int slot_d = t >> L, col_d = (chunk << L) + (t & (n - 1));
+    const int slot_d = t >> L, col_d = P::column(chunk, t & (n - 1), a.low_bits);
     const int64_t x_col_d = view_col(a.x_view, col_d), g_col_d = view_col(a.g_view, col_d);
     const int x_dma = x_col_d >= 0 ? slot_d * x_row + (int)(x_col_d * a.x_view.se * EB) : kOob;
     const int g_dma = g_col_d >= 0 ? slot_d * g_row + (int)(g_col_d * a.g_view.se * EB) : kOob;
@@ -921,7 +971,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const FastCoords c2 = fast_coords<L>(t2);
     if constexpr (BIAS_SUM) {
         if (bias_on) {
-            const int64_t bcol = ((int64_t)chunk << L) + (Q::SB ? c2.eB : c2.eA);
+            const int64_t bcol = P::column(chunk, Q::SB ? c2.eB : c2.eA, a.low_bits);
             if (bcol < a.bias_width)
                 reinterpret_cast<float *>(a.bias_partial)[((int64_t)blockIdx.x * gridDim.y + stack) * a.bias_width +
                                                           bcol] = lds_bias[t2];
@@ -930,7 +980,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // One partial slice per workgroup.  When the workgroup holds several rows at once
     // (n < 1024) the per-row-slot sums are first added through LDS in ascending slot order.
     T *part = reinterpret_cast<T *>(a.partial) + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * a.partial_slot +
-              (int64_t)chunk * (n / 2) * 4;
+              P::pair_base(chunk) * 4;
     if constexpr (SLOTS == 1) {
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
@@ -938,7 +988,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             constexpr int lay = P::layout(s);
             const int e = lay ? c2.eB : c2.eA;
             const int r = (e >> bit) & 1;
-            const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
+            const int i = P::pair_index(chunk, e, bit, a.low_bits);
             T *d = part + (int64_t)s * a.partial_slot + i * 4;
             d[3 * r] = acc_self[s];    // dT[r][r]
             d[COL ? 2 - r : r + 1] = acc_cross[s];   // dT[1 - r][r] (column form) or dT[r][1 - r]
@@ -962,7 +1012,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 #pragma unroll 4
                 for (int sl = 1; sl < SLOTS; ++sl) sum = add(sum, red[sl * 2 * n + t2]);
                 const int r = (eo >> bit) & 1;
-                const int i = ((eo >> (bit + 1)) << bit) | (eo & ((1 << bit) - 1));
+                const int i = P::pair_index(chunk, eo, bit, a.low_bits);
                 // j = 0: dT[r][r], j = 1: dT[1 - r][r] (column form) or dT[r][1 - r]
                 part[(int64_t)s * a.partial_slot + i * 4 + (j ? (COL ? 2 - r : r + 1) : 3 * r)] = sum;
             }

@@ -6,8 +6,8 @@
 // 2x2 factors resident for the whole launch.  Threads of a workgroup take consecutive p, whose
 // low ten bits are the element's low ten bits, so every access is a coalesced row segment.
 // The pass is purely streaming: one read and one write of the activation (plus one read of
-// the gradient in the backward pass).  Rows of any length are covered by one such pass per
-// group of high bits next to the chunked kernels for bits 0..9.
+// the gradient in the backward pass).  Used for rows of 2048 and 4096 (one or two high bits);
+// longer rows run their high bits through the kernels of fast.hpp on tiles (SpanPlan).
 #pragma once
 
 #include "common.hpp"
@@ -154,9 +154,8 @@ __global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
     constexpr int W = (int)sizeof(T) / 4;  // dwords per scalar: the planes of a complex row are fetched separately
     constexpr int EB = (int)sizeof(T);
     // complex64 rows would have to be fetched as two strided 32-bit planes, which measured
-    // slower than plain register prefetch: float only; with eight elements per thread the
-    // requests in flight would overflow the 6-bit wait counter: register prefetch as well
-    constexpr bool DIRECT = W == 1 && H <= 2;
+    // slower than plain register prefetch: float only
+    constexpr bool DIRECT = W == 1;
     constexpr int SLOT = 2 * E * W * THREADS;  // dwords per row slot: x and g, E elements, W planes
     __shared__ float rows[DIRECT ? (kHighAhead + 1) * SLOT : 1];
     const int p = blockIdx.z * THREADS + threadIdx.x;
@@ -213,7 +212,7 @@ __global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
     // memory operations issued after the requests of a row and before that row is read: the
     // requests of the kHighAhead following rows and the stores of the kHighAhead rows before it
     constexpr int YOUNGER = kHighAhead * (2 * E * W + E);
-    static_assert(!DIRECT || YOUNGER <= 63, "the wait counter holds 6 bits");
+    static_assert(YOUNGER <= 63, "the wait counter holds 6 bits");
 
     // register flavour: one row ahead
     const __amdgpu_buffer_rsrc_t x_rs = make_rsrc(reinterpret_cast<const T *>(a.x_in) + stack * a.x_view.ss + r0 * a.x_view.sb);
@@ -242,7 +241,7 @@ __global__ __launch_bounds__(THREADS) void high_bw_kernel(HighArgs a)
         T act[NST][E], g[E];
         if constexpr (DIRECT) {
             fetch_row(row + kHighAhead);
-            wait_rows_in_lds<DIRECT ? YOUNGER : 0>();
+            wait_rows_in_lds<YOUNGER>();
 #pragma unroll
             for (int j = 0; j < E; ++j) {
                 act[0][j] = read_row(row, 0, j);

@@ -264,7 +264,8 @@ def test_launch_plans_cover_every_stage_once():
     """bf_describe_plan (host only): for every row length up to 2^24, both dtypes, both stride
     orders, forward and backward, the passes cover the stage list exactly once in order; low
     passes hold whole blocks of ten low bits; a high pass works on at most three adjacent bits
-    and only on stages of exactly those bits; the bit groups tile bits 10..L-1."""
+    and only on stages of exactly those bits, a span pass on at most five in one sweep up, one
+    sweep down or both; the bit groups tile bits 10..L-1."""
     from butterfly_amd import _capi
     for cplx in (0, 1):
         for L in range(1, 25):
@@ -294,11 +295,17 @@ def test_launch_plans_cover_every_stage_once():
                                 assert q["inc"] == int(stage_bits[0] == 0 and q["L"] > 1 or (q["L"] == 1 and inc != ((a // L) % 2 == 1))), key
                             elif q["kind"] == "wide":
                                 assert not backward and L in (11, 12) and b - a == L, key
+                            elif q["kind"] == "span":
+                                lb, h = q["lb"], q["bits"]
+                                assert lb >= 10 and 1 <= h <= 5 and q["tiles"] == (1 << (L - 10)), key
+                                up, down = list(range(lb, lb + h)), list(range(lb + h - 1, lb - 1, -1))
+                                assert stage_bits == [up, down, up + down][q["mode"]], key
+                                groups.add((lb, h))
                             else:
                                 lb, h = q["lb"], q["bits"]
-                                assert q["kind"] == "high" and lb >= 10 and 1 <= h <= (2 if cplx else 3), key
+                                assert q["kind"] == "high" and lb == 10 and 1 <= h <= 2 and L <= 12, key
                                 assert all(lb <= x < lb + h for x in stage_bits), key
-                                assert b - a <= (3 if h == 3 else 2 * h), key
+                                assert b - a <= 2 * h, key
                                 for s, x in enumerate(stage_bits):
                                     assert (q["pattern"] >> (2 * s)) & 3 == x - lb, key
                                 groups.add((lb, h))
@@ -310,4 +317,5 @@ def test_launch_plans_cover_every_stage_once():
     assert _capi.describe_plan(0, 16384, 1, 10, 2, False, True) == ["low t=0..20 L=10 nb=2 inc=0 chunks=1"]
     assert [l.split()[0] for l in _capi.describe_plan(0, 32768, 1, 12, 2, True, False)] == ["wide", "wide"]
     assert [l.split()[0] for l in _capi.describe_plan(0, 32768, 1, 12, 2, True, True)] == ["low", "high", "low"]
-    assert [l.split()[0] for l in _capi.describe_plan(0, 2048, 1, 13, 1, True, True)] == ["low", "high"]
+    assert [l.split()[0] for l in _capi.describe_plan(0, 2048, 1, 13, 1, True, True)] == ["low", "span"]
+    assert [l.split()[0] for l in _capi.describe_plan(0, 16, 1, 20, 1, True, False)] == ["low", "span", "span"]
