@@ -16,7 +16,6 @@
 #include "common.hpp"
 #include "generic.hpp"
 #include "fast.hpp"
-#include "high.hpp"
 #include "wide.hpp"
 #include "fast4.hpp"
 #include "fast4g.hpp"
@@ -154,17 +153,17 @@ constexpr int kFastFwRows = BF_FAST_FW_ROWS;  // row groups in flight per forwar
 constexpr int kFastFwWgPerCu = BF_FAST_FW_WGS;  // forward workgroups resident per compute unit
 constexpr int kFastFwRowsComplex = 2;       // complex64: half as many (LDS and registers double)
 
-// ---- register-resident multi-pass path (float and complex64, base-2, n <= 4096) ---------------------------
+// ---- register-resident multi-pass path (float and complex64, base-2, n <= 2^24) -------------------------
 //
-// The flat stage list is cut into passes, one kernel launch each:
-//   * a LOW pass runs up to 20 consecutive stages that pair element bits below 10 with the
-//     twiddle-stationary kernels of fast.hpp (rows longer than 1024 are treated as
-//     independent 1024-element chunks);
-//   * a HIGH pass runs the stages that pair bits 10 and 11 with the streaming kernels of
-//     high.hpp;
-//   * the forward call alone replaces the LOW / HIGH passes of one block by a single WIDE pass
-//     (wide.hpp) where the factors of a whole block fit the registers: float at n = 2048 and
-//     4096, complex64 at n = 2048.
+// The flat stage list is cut into passes, one kernel launch each, all with the
+// twiddle-stationary kernels of fast.hpp:
+//   * a LOW pass runs up to 20 consecutive stages that pair element bits below 10 (rows longer
+//     than 1024 are treated as independent 1024-element chunks);
+//   * a SPAN pass runs the stages on up to five adjacent bits from bit 10 up, on tiles of 1024
+//     elements that take all settings of those bits (SpanPlan);
+//   * the forward call alone replaces the LOW / SPAN passes of one block by a single WIDE pass
+//     (wide.hpp) where the factors of a whole block fit the registers and enough rows share
+//     them: float at n = 2048 and 4096, complex64 at n = 2048.
 // n <= 1024 with one or two blocks is a single LOW pass: each row is read once and written
 // once.  Longer schedules pass the activation through the workspace between launches.
 
@@ -178,18 +177,15 @@ bool span_ok(const int64_t stride[3], int64_t rows, int64_t width, size_t elem)
 
 constexpr int kMaxPasses = 96;
 constexpr int kSpanMaxBits = 5;    // widest span: tiles of 32 consecutive elements per setting of the span's bits
-constexpr int kSpanFromBits = 3;   // rows with fewer bits above 10 keep the streaming passes of high.hpp
 constexpr int kMaxLogN = 24;  // the chunk index of the register-resident kernels travels in blockIdx.z
 
 struct Pass {
     int t0, t1;     // stage range [t0, t1)
-    bool high;
     bool wide;      // forward only: one whole block of a 2048- or 4096-element row (wide.hpp)
     int L, NB;      // LOW: FastPlan<L, NB, inc> on chunks of 2^L elements
     bool inc;
-    int H, NST, PAT;  // HIGH: H adjacent bits from `lb` up, NST stages, bits 2s, 2s+1 of PAT = which of them stage s pairs
-    int lb;
-    bool span;      // LOW kernels on tiles of a span of H high bits from `lb` up (SpanPlan<H, mode>), L = 10, NB = 1
+    bool span;      // SPAN: SpanPlan<H, mode> on tiles, H adjacent bits from `lb` up (L = 10, NB = 1)
+    int H, lb;
     int mode;       // 0: one sweep up, 1: one sweep down, 2: up then down
 };
 
@@ -209,7 +205,7 @@ int stage_bit(const bf_problem *p, int t)
 }
 
 // Rows (over all stacks) from which the whole-block forward kernel of wide.hpp beats the
-// chunked + high-bit passes: each of its workgroups first loads the factors of a whole block
+// chunked + span passes: each of its workgroups first loads the factors of a whole block
 // (up to 96 registers per thread), which only pays off over enough rows.  Measured crossovers.
 int64_t wide_min_rows(const bf_problem *p)
 {
@@ -252,18 +248,16 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             q.inc = (p->increasing_stride != 0) != ((k & 1) != 0);
         }
     } else {
-        // bits 0..9: the register-resident kernels on 1024-element chunks.  One or two bits above
-        // them (rows of 2048 / 4096): one streaming pass of high.hpp.  More: spans of up to
-        // kSpanMaxBits adjacent bits, as equal as possible, each one pass of the register-resident
-        // kernels over tiles (SpanPlan) -- e.g. n = 2^20: [10..14] [15..19].
+        // bits 0..9: the kernels on 1024-element chunks; the bits above them: spans of up to
+        // kSpanMaxBits adjacent bits, as equal as possible, each one pass of the same kernels over
+        // tiles (SpanPlan) -- n = 4096: [10,11]; n = 2^20: [10..14] [15..19].
         pl.chunks = (int64_t)1 << (L - 10);
         const int hbits = L - 10;
-        const bool use_span = hbits >= kSpanFromBits;
         const int nspans = (hbits + kSpanMaxBits - 1) / kSpanMaxBits;
         int group_lb[16], group_bits[16], ngroups = 0;
         for (int b = 10; b < L; ++ngroups) {
             group_lb[ngroups] = b;
-            group_bits[ngroups] = use_span ? hbits / nspans + (ngroups < hbits % nspans ? 1 : 0) : hbits;
+            group_bits[ngroups] = hbits / nspans + (ngroups < hbits % nspans ? 1 : 0);
             b += group_bits[ngroups];
         }
         auto group_of = [&](int bit) {
@@ -287,22 +281,15 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             int u = t;
             while (u < NS && group_of(stage_bit(p, u)) == grp && u - t < cap) ++u;
             q.t1 = u;
-            q.high = high && !use_span;
-            if (high && use_span) {
+            if (high) {
                 q.span = true;
                 q.L = 10;
                 q.NB = 1;
                 q.lb = lb;
                 q.H = H;
-                q.NST = u - t;
-                if (q.NST != H && q.NST != 2 * H) return pl;
-                q.mode = q.NST == 2 * H ? 2 : (stage_bit(p, t) == lb ? 0 : 1);
+                if (u - t != H && u - t != 2 * H) return pl;
+                q.mode = u - t == 2 * H ? 2 : (stage_bit(p, t) == lb ? 0 : 1);
                 q.inc = q.mode != 1;
-            } else if (high) {
-                q.lb = lb;
-                q.H = H;
-                q.NST = u - t;
-                for (int s = 0; s < q.NST; ++s) q.PAT |= (stage_bit(p, t + s) - q.lb) << (2 * s);
             } else {
                 q.L = 10;
                 if ((u - t) != 10 && (u - t) != 20) return pl;
@@ -372,24 +359,6 @@ FastGrid wide_grid(int64_t batch, int64_t nstacks)
     return g;
 }
 
-// Row partition of a HIGH pass (4 workgroups of 256 low positions per row partition and stack).
-struct HighGrid {
-    int64_t nparts, rows_per_wg;
-};
-
-// Row partition of a HIGH pass whose row takes `row_threads` threads (n >> H): about 2048
-// threads per compute unit over all stacks.
-HighGrid high_grid(int64_t batch, int64_t nstacks, int64_t row_threads, int64_t max_rows = kNoRowCap)
-{
-    HighGrid g;
-    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * 2 * 1024 / (nstacks * row_threads));
-    g.nparts = std::min(want, batch);
-    g.rows_per_wg = (batch + g.nparts - 1) / g.nparts;
-    if (max_rows - kRowMargin >= 1 && g.rows_per_wg > max_rows - kRowMargin) g.rows_per_wg = max_rows - kRowMargin;
-    g.nparts = (batch + g.rows_per_wg - 1) / g.rows_per_wg;
-    return g;
-}
-
 // True when every pass can address its operands with 32-bit offsets.
 bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
 {
@@ -398,12 +367,6 @@ bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
     int64_t rows = 0;
     for (int k = 0; k < pl.npass; ++k) {
         const Pass &q = pl.pass[k];
-        if (q.high) {
-            // the backward high-bit kernel forms 32-bit offsets from its workgroup's first row
-            if (backward)
-                rows = std::max(rows, high_grid(p->batch, p->nstacks, n >> q.H, cap).rows_per_wg + kHighAhead + 1);
-            continue;
-        }
         const FastGrid g = q.wide ? wide_grid(p->batch, p->nstacks)
                                   : fast_grid(p->batch, q.L, p->nstacks * pl.chunks, backward ? 1 : fw_rows(p),
                                               backward ? 1 : kFastFwWgPerCu, cap);
@@ -475,7 +438,7 @@ int launch_span(bool cplx, const Pass &q, bool backward, bool two_rows, const Fa
     case HH * 3 + 1: launch_span_t<HH, 1>(cplx, backward, two_rows, fw, bw, grid, stream); break;   \
     case HH * 3 + 2: launch_span_t<HH, 2>(cplx, backward, two_rows, fw, bw, grid, stream); break;
     switch (q.H * 3 + q.mode) {
-        BF_SPAN_CASES(2) BF_SPAN_CASES(3) BF_SPAN_CASES(4) BF_SPAN_CASES(5)
+        BF_SPAN_CASES(1) BF_SPAN_CASES(2) BF_SPAN_CASES(3) BF_SPAN_CASES(4) BF_SPAN_CASES(5)
         default: return fail(BF_ERR_UNSUPPORTED, "no kernel for a span of %d bits", q.H);
     }
 #undef BF_SPAN_CASES
@@ -500,35 +463,6 @@ int launch_span(bool cplx, const Pass &q, bool backward, bool two_rows, const Fa
     case LL * 4 + 2: FN<LL, 2, false>(__VA_ARGS__); break;      \
     case LL * 4 + 3: FN<LL, 2, true>(__VA_ARGS__); break;
 
-template <typename T, int H, int NST, int PAT>
-void launch_high_t(bool backward, const HighArgs &a, dim3 grid, hipStream_t stream)
-{
-    if (backward) {
-        // float leaves room for 1024 threads (128 registers each), complex64 for 512
-        // grid.z arrives as the threads a row takes
-        constexpr int THREADS = sizeof(T) == 4 ? 1024 : 512;
-        grid.z = grid.z / THREADS;
-        hipLaunchKernelGGL((high_bw_kernel<T, H, NST, PAT, THREADS>), grid, dim3(THREADS), 0, stream, a);
-    } else
-        hipLaunchKernelGGL((high_fw_kernel<T, H, NST, PAT>), grid, dim3(kHighThreads), 0, stream, a);
-}
-
-template <typename T>
-int launch_high(const Pass &q, bool backward, const HighArgs &a, dim3 grid, hipStream_t stream)
-{
-    const int key = q.H * 1000 + q.NST * 100 + q.PAT;
-    switch (key) {
-        case 1 * 1000 + 1 * 100 + 0: launch_high_t<T, 1, 1, 0>(backward, a, grid, stream); break;
-        case 1 * 1000 + 2 * 100 + 0: launch_high_t<T, 1, 2, 0>(backward, a, grid, stream); break;
-        case 2 * 1000 + 2 * 100 + 4: launch_high_t<T, 2, 2, 4>(backward, a, grid, stream); break;    // bits 0, 1 of the group
-        case 2 * 1000 + 2 * 100 + 1: launch_high_t<T, 2, 2, 1>(backward, a, grid, stream); break;    // 1, 0
-        case 2 * 1000 + 4 * 100 + 20: launch_high_t<T, 2, 4, 20>(backward, a, grid, stream); break;  // 0, 1, 1, 0
-        default: return fail(BF_ERR_UNSUPPORTED, "no kernel for this high-bit stage pattern");
-    }
-    BF_HIP_CHECK(hipGetLastError());
-    return BF_OK;
-}
-
 void fill_stage_table(int *dst, int cap, const Pass &q)
 {
     for (int s = 0; s < cap; ++s) dst[s] = q.t0 + std::min(s, q.t1 - q.t0 - 1);
@@ -551,25 +485,7 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
         void *dst = k == last - 1 ? output : scratch;
         const View sv = k == first ? in_view : dense;
         const View dv = k == last - 1 ? out_view : dense;
-        if (q.high) {
-            const HighGrid g = high_grid(p->batch, p->nstacks, n >> q.H, row_cap(p, false));
-            HighArgs a = {};
-            a.low_bits = q.lb;
-            a.tw = tw;
-            a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
-            a.tw_stage_stride = (n / 2) * 4;
-            fill_stage_table(a.tw_stage, 4, q);
-            a.x_in = src;
-            a.x_view = sv;
-            a.x_out = dst;
-            a.xo_view = dv;
-            a.batch = p->batch;
-            a.rows_per_wg = g.rows_per_wg;
-            const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, (unsigned)((n >> q.H) / kHighThreads));
-            const int rc = p->dtype == BF_C64 ? launch_high<float2>(q, false, a, grid, stream)
-                                              : launch_high<float>(q, false, a, grid, stream);
-            if (rc) return rc;
-        } else if (q.wide) {
+        if (q.wide) {
             const FastGrid g = wide_grid(p->batch, p->nstacks);
             FastFwArgs a = {};
             a.tw = tw;
@@ -1013,8 +929,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
         int64_t nparts = 1, slices = 1;  // slices: partial (stage, 2n) slices of the pass that needs most
         for (int k = 0; k < mp.npass; ++k) {
             const Pass &q = mp.pass[k];
-            const int64_t np = q.high ? high_grid(p->batch, p->nstacks, n >> q.H, row_cap(p, true)).nparts
-                                      : fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1, row_cap(p, true)).nwg;
+            const int64_t np = fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1, row_cap(p, true)).nwg;
             nparts = std::max(nparts, np);
             slices = std::max(slices, np * (q.t1 - q.t0));
         }
@@ -1217,31 +1132,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
             void *gin = k == 0 ? d_input : ws + pl.off_gbuf;
             const View giv = k == 0 ? dn_view : dense;
             int64_t nparts = 0;
-            if (q.high) {
-                const HighGrid g = high_grid(p->batch, p->nstacks, n >> q.H, row_cap(p, true));
-                HighArgs a = {};
-                a.low_bits = q.lb;
-                a.tw = tw2;
-                a.tw_stack_stride = sc.tw2_stack_stride;
-                a.tw_stage_stride = (n / 2) * 4;
-                fill_stage_table(a.tw_stage, 4, q);
-                a.x_in = xin;
-                a.x_view = xv;
-                a.g_out = gout;
-                a.g_view = gv;
-                a.g_in = gin;
-                a.gi_view = giv;
-                a.partial = ws + pl.off_partials;
-                a.partial_slot = pl.slot;
-                a.batch = p->batch;
-                a.rows_per_wg = g.rows_per_wg;
-                nparts = g.nparts;
-                // (the launcher sets gridDim.z from the backward kernel's workgroup size)
-                const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, (unsigned)(n >> q.H));
-                rc = p->dtype == BF_C64 ? launch_high<float2>(q, true, a, grid, stream)
-                                        : launch_high<float>(q, true, a, grid, stream);
-                if (rc) return rc;
-            } else {
+            {
                 const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1, row_cap(p, true));
                 FastBwArgs a = {};
                 a.tw = tw2;
@@ -1514,9 +1405,7 @@ int bf_describe_plan(const bf_problem *p, int backward, char *text, size_t capac
     } else {
         for (int k = 0; k < mp.npass; ++k) {
             const Pass &q = mp.pass[k];
-            if (q.high)
-                snprintf(line, sizeof line, "high t=%d..%d lb=%d bits=%d pattern=%d\n", q.t0, q.t1, q.lb, q.H, q.PAT);
-            else if (q.wide)
+            if (q.wide)
                 snprintf(line, sizeof line, "wide t=%d..%d L=%d inc=%d\n", q.t0, q.t1, q.L, (int)q.inc);
             else if (q.span)
                 snprintf(line, sizeof line, "span t=%d..%d lb=%d bits=%d mode=%d tiles=%lld\n", q.t0, q.t1, q.lb, q.H,

@@ -144,7 +144,8 @@ int bf_butterfly_multiply_perm_bw(const bf_problem *p, const void *twiddle, cons
  * call for this problem is cut into launches, one text line per pass in order --
  *   "low t=A..B L=.. nb=.. inc=.. chunks=.."   stages A..B-1 on bits 0..9, 1024-element chunks
  *   "wide t=A..B L=.. inc=.."                   one whole block of a 2048 / 4096 row (forward)
- *   "high t=A..B lb=.. bits=.. pattern=.."      stages on `bits` adjacent bits from bit lb up
+ *   "span t=A..B lb=.. bits=.. mode=.. tiles=.." stages on `bits` adjacent bits from bit lb up
+ *                                               (mode 0 one sweep up, 1 down, 2 up then down)
  *   "generic"                                   the LDS fallback kernels
  * No counterpart in the reference (its launch plan is butterfly_max5_plan,
  * csrc/cuda/butterfly_cuda.cu:317-345, internal to the operator).                       */
