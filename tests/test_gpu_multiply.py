@@ -95,7 +95,7 @@ def test_register_resident_kernels_all_sizes(L):
 
 
 MULTIPASS_CASES = [
-    # B, S, L, nb, I, O, inc -- more than two blocks and rows of 2048 / 4096 (chunked + high-bit passes)
+    # B, S, L, nb, I, O, inc -- more than two blocks and rows of 2048 / 4096 (chunk + span passes)
     (40, 2, 9, 3, None, None, True),
     (40, 2, 9, 4, None, None, False),
     (33, 1, 10, 5, 1000, 900, False),
@@ -140,9 +140,9 @@ def test_multi_launch_schedules(case):
 
 
 LONG_ROW_CASES = [
-    # dtype, B, S, L, nb, I, O, inc -- rows beyond 4096: chunked passes for bits 0..9 and one
-    # streaming pass per group of two higher bits (odd and even numbers of high bits, the block
-    # boundary inside the top group, several row partitions)
+    # dtype, B, S, L, nb, I, O, inc -- rows beyond 4096: chunk passes for bits 0..9 and one span
+    # pass per group of up to five higher bits (one and two spans, the block boundary inside the
+    # top span, several row partitions)
     (np.float32, 9, 1, 13, 1, None, None, True),
     (np.float32, 9, 2, 13, 2, None, None, False),
     (np.float32, 7, 1, 14, 2, 16000, 9000, True),
@@ -528,7 +528,7 @@ def test_headline_size_properties():
 
 BIAS_CASES = [
     # dtype, B, S, L, nb, I, O, inc -- every kind of last pass: fast (fused), wide (fused),
-    # high-bit and generic (separate add), several stacks, trimmed outputs
+    # span and generic (separate add), several stacks, trimmed outputs
     (np.float32, 37, 2, 5, 2, 20, 27, True),
     (np.float32, 300, 1, 10, 2, None, None, False),
     (np.float32, 41, 3, 7, 1, None, 100, True),
@@ -603,7 +603,7 @@ def test_bias_operator_autograd():
 
 PERM_CASES = [
     # dtype, B, S, L, nb, I, O, inc, tables ("io" = both, "i", "o"), bias -- every kind of first
-    # and last pass: register and LDS row fetch, wide, high-bit, generic; padded inputs,
+    # and last pass: register and LDS row fetch, wide, span, generic; padded inputs,
     # trimmed outputs, several stacks
     (np.float32, 37, 1, 5, 2, 20, 27, True, "io", True),
     (np.float32, 300, 1, 10, 2, None, None, False, "io", True),
