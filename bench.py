@@ -1,13 +1,16 @@
 """Benchmark of the butterfly multiply on one MI355X, through torch.ops.torch_butterfly.
 
-    python bench.py [--steps K] [--warmup W] [--config cfg2] [--no-cpu-baseline] [--calibrate-copy]
+    python bench.py [--steps K] [--warmup W] [--settle-ms T] [--config cfg2] [--no-cpu-baseline] [--calibrate-copy]
 
 The default workload (cfg2) is the headline one: forward + backward, batch 16384, n = 1024,
 fp32, nblocks = 2, decreasing stride first.  The other configurations of the baseline list
 (cfg1, cfg3, cfg4, cfg5) can be selected with --config.  One JSON line is printed.
 
 ``value`` is algorithmic bytes (2 row passes forward, 3 backward, plus twiddle traffic) per
-second over the K timed steps, operands resident in HBM.  ``roofline`` describes the
+second over the K timed steps, operands resident in HBM.  Before the W warmup steps the same
+step runs untimed for T milliseconds (default 250): the GPU needs a few tens of milliseconds
+of sustained load to reach its steady clocks, and K steps of a 0.2 ms workload would
+otherwise be timed entirely inside that ramp.  ``roofline`` describes the
 dominant call (the backward pass where there is one), timed with device events on the launch
 stream.  ``cpu_baseline`` is the single-threaded reference C++ (or, for base-4 and where the
 reference build is absent, the repo's CPU restatement) timed on this host on a bounded sample.
@@ -177,6 +180,10 @@ def main():
     ap.add_argument("--shape", default=None, metavar="B,S,LOG_N,NBLOCKS,f32|c64[,inc|dec]",
                     help="forward + backward at an arbitrary shape instead of a named configuration")
     ap.add_argument("--batch", type=int, default=None, help="run the configuration at another batch size")
+    ap.add_argument("--settle-ms", type=float, default=250.0,
+                    help="run untimed steps for this long before the warmup steps: the GPU raises its clocks "
+                         "over the first tens of milliseconds of sustained load, and kernels launched in that "
+                         "window run 10-20 %% slower than in steady state")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of the input (a kernel of known traffic, for scaling "
@@ -259,10 +266,18 @@ def main():
         fw_call = lambda: ops.butterfly_multiply_fw(tws[0], x, inc, None)
         bw_call = lambda: ops.butterfly_multiply_bw(tws[0], x, grad, inc)
 
-    for _ in range(args.warmup):
+    def untimed_step():
         fw_call()
         if c["bw"]:
             bw_call()
+
+    settle_t0 = time.perf_counter()
+    while (time.perf_counter() - settle_t0) * 1e3 < args.settle_ms:
+        for _ in range(4):
+            untimed_step()
+        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        untimed_step()
     torch.cuda.synchronize()
     if args.calibrate_copy:
         dst = torch.empty_like(x)
@@ -296,7 +311,7 @@ def main():
     dom_gbs = dom_b / (dom_ms * 1e-3) / 1e9
     line = {
         "metric": c["metric"], "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "warmup": args.warmup, "settle_ms": args.settle_ms, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "c64" if c["cplx"] else "f32", "data": "synthetic",
         "config": {"workload": c["workload"]},
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
