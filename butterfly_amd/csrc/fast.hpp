@@ -211,6 +211,45 @@ __device__ __forceinline__ void bw_products(T &self, T &cross, T &g, T x, T ta, 
     g = macc(mul(conj_of(ta), g), tc, gp);
 }
 
+// float and a DPP exchange: both uses of the partner's g read it through the DPP operand of the
+// multiply-add itself, so no move materialises it.  The two plain instructions in front keep
+// the two wait states a DPP read needs after a VALU write of the same register, whatever the
+// compiler schedules in front of the block.
+#define BF_BW_PRODUCTS_DPP(CTRL)                                                                   \
+    asm volatile("v_fmac_f32_e32 %0, %3, %4\n\t"                                                   \
+                 "v_mul_f32_e32 %2, %5, %3\n\t"                                                    \
+                 "v_fmac_f32_dpp %1, %3, %4 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"  \
+                 "v_fmac_f32_dpp %2, %3, %6 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1"       \
+                 : "+v"(self), "+v"(cross), "=&v"(m)                                               \
+                 : "v"(g), "v"(x), "v"(ta), "v"(tc))
+
+template <int K>
+__device__ __forceinline__ void bw_products_dpp(float &self, float &cross, float &g, float x, float ta, float tc)
+{
+    static_assert(K >= 0 && K < 4, "DPP exchange kinds only");
+    float m;
+    if constexpr (K == 0) BF_BW_PRODUCTS_DPP("quad_perm:[1,0,3,2]");
+    else if constexpr (K == 1) BF_BW_PRODUCTS_DPP("quad_perm:[2,3,0,1]");
+    else if constexpr (K == 2) BF_BW_PRODUCTS_DPP("row_half_mirror");
+    else BF_BW_PRODUCTS_DPP("row_mirror");
+    g = m;
+}
+#undef BF_BW_PRODUCTS_DPP
+
+template <int K>
+__device__ __forceinline__ void bw_products(float &self, float &cross, float &g, float x, float ta, float tc,
+                                            int bperm_addr)
+{
+    if constexpr (K < 4) {
+        bw_products_dpp<K>(self, cross, g, x, ta, tc);
+    } else {
+        const float gp = partner<K>(g, bperm_addr);
+        fmac_pinned(self, g, x);
+        fmac_pinned(cross, gp, x);
+        g = fmaf(tc, gp, ta * g);
+    }
+}
+
 // The same stage written with the factor row (ta = T[me][me], tb = T[me][p]) that the forward
 // replay holds anyway: two exchanges, but no third factor entry to keep.
 //   cross += g * conj(x_p)               dT[me][p]
