@@ -81,6 +81,18 @@ CONFIGS = {
                       metric="special.fft(4096) module fwd+bwd GB/s, bit reversal as a separate gather",
                       workload="cfg3 (module level, unfused): the same two modules run one after the other "
                                "(PyTorch gather, then butterfly_multiply); for comparison with cfg3m"),
+    "diag": dict(batch=16384, nstacks=1, log_n=10, nblocks=2, inc=False, cplx=False, base4=False, bw=True,
+                 cpu_batch=16384, module="diag-fused",
+                 metric="Diagonal-Butterfly(1024, nblocks 2)-Diagonal fwd+bwd GB/s, batch 16384 fp32, diagonals folded in",
+                 workload="module level: FusedSequential(Diagonal(1024), Butterfly(1024, 1024, bias=False, nblocks=2, "
+                          "increasing_stride=False), Diagonal(1024)), forward + autograd backward (d_input, "
+                          "d_twiddle, both d_diagonal), input (16384,1024) fp32; the diagonals are multiplied into "
+                          "the layer's first / last factor"),
+    "diag-sep": dict(batch=16384, nstacks=1, log_n=10, nblocks=2, inc=False, cplx=False, base4=False, bw=True,
+                     cpu_batch=16384, module="diag-sep",
+                     metric="Diagonal-Butterfly(1024, nblocks 2)-Diagonal fwd+bwd GB/s, diagonals as elementwise ops",
+                     workload="module level, unfused: the same three modules in a plain nn.Sequential; for "
+                              "comparison with diag"),
     "legacy": dict(batch=2048, nstacks=1, log_n=9, nblocks=1, inc=True, cplx=False, base4=False, bw=True,
                    cpu_batch=2048, module="legacy",
                    metric="legacy butterfly.Butterfly(512, 512, tied_weight=False) fwd+bwd GB/s, batch 2048 fp32",
@@ -232,6 +244,22 @@ def main():
         def fw_call():
             state["y"] = layer(xm)
         bw_call = lambda: torch.autograd.grad(state["y"], (xm, layer[1].twiddle), gm)
+    elif c.get("module", "").startswith("diag"):
+        from butterfly_amd.diagonal import Diagonal
+        from butterfly_amd.permutation import FusedSequential
+        n = 1 << c["log_n"]
+        layer = FusedSequential(Diagonal(n), butterfly_amd.Butterfly(n, n, bias=False, nblocks=c["nblocks"],
+                                                                     increasing_stride=c["inc"]), Diagonal(n)).to(dev)
+        if c["module"] == "diag-sep":
+            layer = torch.nn.Sequential(*layer)
+        xm = x.reshape(c["batch"], -1).requires_grad_()
+        gm = grad.reshape(c["batch"], -1)
+        params = [xm] + list(layer.parameters())
+        state = {}
+
+        def fw_call():
+            state["y"] = layer(xm)
+        bw_call = lambda: torch.autograd.grad(state["y"], params, gm)
     elif c.get("module") == "legacy":
         from butterfly_amd import legacy
         layer = legacy.Butterfly(1 << c["log_n"], 1 << c["log_n"], bias=False, tied_weight=False).to(dev)

@@ -20,6 +20,7 @@ SYMBOLS = [
     "bf_butterfly_multiply_bias_fw", "bf_butterfly_bias_grad", "bf_butterfly_bias_grad_workspace_bytes",
     "bf_butterfly_multiply_bias_bw", "bf_butterfly_multiply_bias_bw_workspace_bytes",
     "bf_butterfly_multiply_perm_fw", "bf_butterfly_multiply_perm_bw", "bf_describe_plan",
+    "bf_butterfly_scale_twiddle", "bf_butterfly_scale_twiddle_bw",
     "bf_butterfly_multiply_base4_fw", "bf_butterfly_multiply_base4_fw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw",
@@ -72,6 +73,9 @@ def lib():
         L.bf_butterfly_multiply_perm_fw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_perm_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_describe_plan.argtypes = [pp, ctypes.c_int, ctypes.c_char_p, sz]
+        i32, i64 = ctypes.c_int, ctypes.c_int64
+        L.bf_butterfly_scale_twiddle.argtypes = [i32, i64, i64, i64, i32, vp, vp, i64, vp, i64, vp, vp]
+        L.bf_butterfly_scale_twiddle_bw.argtypes = [i32, i64, i64, i64, i32, vp, vp, i64, vp, i64, vp, vp, vp, vp, vp]
         L.bf_butterfly_multiply_base4_fw.argtypes = [pp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_base4_fw_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_base4_fw_workspace_bytes.restype = sz
@@ -204,6 +208,41 @@ def describe_plan(dtype_code, batch, nstacks, log_n, nblocks, increasing_stride,
     buf = ctypes.create_string_buffer(1 << 14)
     _check(lib().bf_describe_plan(ctypes.byref(p), int(backward), buf, len(buf)))
     return buf.value.decode().splitlines()
+
+
+def _scale_args(twiddle, in_scale, out_scale):
+    assert twiddle.is_cuda and twiddle.is_contiguous() and twiddle.dim() == 6
+    for v in (in_scale, out_scale):
+        assert v is None or (v.is_cuda and v.is_contiguous() and v.dim() == 1 and v.dtype == twiddle.dtype)
+    return (_dtype_code(twiddle), twiddle.shape[0], twiddle.shape[1], twiddle.shape[2])
+
+
+def scale_twiddle(twiddle, in_scale, out_scale, increasing_stride):
+    """Factors of diag(out_scale) B diag(in_scale) (either scale may be None)."""
+    head = _scale_args(twiddle, in_scale, out_scale)
+    out = torch.empty_like(twiddle)
+    _check(lib().bf_butterfly_scale_twiddle(
+        *head, int(increasing_stride), _ptr(twiddle),
+        None if in_scale is None else _ptr(in_scale), 0 if in_scale is None else in_scale.numel(),
+        None if out_scale is None else _ptr(out_scale), 0 if out_scale is None else out_scale.numel(),
+        _ptr(out), _stream()))
+    return out
+
+
+def scale_twiddle_bw(twiddle, in_scale, out_scale, increasing_stride, grad):
+    """(d_twiddle, d_in_scale, d_out_scale) of scale_twiddle for the gradient `grad` of its result."""
+    head = _scale_args(twiddle, in_scale, out_scale)
+    assert grad.is_cuda and grad.is_contiguous() and grad.shape == twiddle.shape and grad.dtype == twiddle.dtype
+    d_tw = torch.empty_like(twiddle)
+    d_in = None if in_scale is None else torch.empty_like(in_scale)
+    d_out = None if out_scale is None else torch.empty_like(out_scale)
+    _check(lib().bf_butterfly_scale_twiddle_bw(
+        *head, int(increasing_stride), _ptr(twiddle),
+        None if in_scale is None else _ptr(in_scale), 0 if in_scale is None else in_scale.numel(),
+        None if out_scale is None else _ptr(out_scale), 0 if out_scale is None else out_scale.numel(),
+        _ptr(grad), _ptr(d_tw), None if d_in is None else _ptr(d_in), None if d_out is None else _ptr(d_out),
+        _stream()))
+    return d_tw, d_in, d_out
 
 
 def _table(t, n):

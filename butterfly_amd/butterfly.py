@@ -34,6 +34,48 @@ def _ortho_complex(core_shape):
     return torch.stack((top, bot), -2)
 
 
+def scale_twiddle(twiddle, increasing_stride, in_scale=None, out_scale=None):
+    """twiddle (stacks, nblocks, log_n, n/2, 2, 2) of the product B with diag(out_scale) B
+    diag(in_scale) folded in: the columns of the first applied factor take in_scale, the rows
+    of the last applied one out_scale.  in_scale has up to n entries (every stack reads the same
+    input), out_scale up to stacks * n (the stacks' outputs side by side); missing entries are 1.
+    Differentiable in all three arguments."""
+    for v in (in_scale, out_scale):
+        if v is not None and v.is_complex() and not twiddle.is_complex():
+            raise ValueError("a complex diagonal cannot be folded into real factors")
+    if twiddle.is_cuda and twiddle.dtype in (torch.float32, torch.complex64):
+        # one small kernel forward, two backward (n-sized work, a single autograd node)
+        cast = lambda v: None if v is None else v.to(twiddle.dtype)
+        return torch.ops.torch_butterfly.butterfly_scale_twiddle(twiddle, cast(in_scale), cast(out_scale),
+                                                                 increasing_stride)
+    stacks, nblocks, log_n, half = twiddle.shape[:4]
+    n = 2 * half
+
+    def pairs(vec, rows, stride):
+        # (rows, n) entries by element -> (rows, n/2, 2) by pair index and position in the pair
+        if vec.shape[-1] < rows * n:
+            vec = torch.nn.functional.pad(vec, (0, rows * n - vec.shape[-1]), value=1.0)
+        return vec.reshape(rows, n // (2 * stride), 2, stride).transpose(-1, -2).reshape(rows, half, 2)
+
+    flat = twiddle.reshape(stacks, nblocks * log_n, half, 2, 2)
+    first, last = flat[:, 0], flat[:, -1]
+    if in_scale is not None:
+        stride = 1 if increasing_stride else half
+        cols = pairs(in_scale, 1, stride)[:, :, None, :]
+        if nblocks * log_n == 1:
+            last = last * cols
+        first = first * cols
+    if out_scale is not None:
+        last_increasing = increasing_stride != ((nblocks - 1) % 2 == 1)
+        stride = half if last_increasing else 1
+        last = last * pairs(out_scale, stacks, stride)[:, :, :, None]
+        if nblocks * log_n == 1:
+            first = last
+    if nblocks * log_n == 1:
+        return last.reshape(twiddle.shape)
+    return torch.cat((first.unsqueeze(1), flat[:, 1:-1], last.unsqueeze(1)), 1).reshape(twiddle.shape)
+
+
 class Butterfly(nn.Module):
     """Product of ``nblocks * log_n`` butterfly factors (block-diagonal 2x2 stages).
 
@@ -109,7 +151,8 @@ class Butterfly(nn.Module):
                 if self.nblocks > 1:
                     tw[:, 1:] = torch.eye(2, dtype=tw.dtype)
 
-    def forward(self, input, transpose=False, conjugate=False, subtwiddle=False, in_perm=None, out_index=None):
+    def forward(self, input, transpose=False, conjugate=False, subtwiddle=False, in_perm=None, out_index=None,
+                in_scale=None, out_scale=None):
         """input (batch, *, in_size) -> (batch, *, out_size).
 
         transpose / conjugate apply the transposed / conjugated matrix; subtwiddle uses only
@@ -118,7 +161,17 @@ class Butterfly(nn.Module):
 
         in_perm / out_index (int32 tables of n entries, see FixedPermutation.column_table): a
         fixed permutation in front of / behind the layer, applied by the layer's own kernels;
-        they describe the untransposed layer (transpose swaps their roles)."""
+        they describe the untransposed layer (transpose swaps their roles).
+
+        in_scale / out_scale (vectors of in_size / out_size entries): a diagonal matrix directly
+        in front of / behind the layer (between the layer and the permutation of in_perm /
+        out_index, if there is one).  They are multiplied into the first / last factor, an
+        n-sized operation that autograd differentiates, instead of into the activations."""
+        if in_scale is not None or out_scale is not None:
+            if subtwiddle or transpose:
+                raise ValueError("in_scale / out_scale cannot be combined with subtwiddle or transpose")
+            if out_scale is not None and self.bias is not None:
+                raise ValueError("a diagonal behind the layer cannot be folded past the bias")
         if in_perm is not None or out_index is not None:
             if subtwiddle:
                 raise ValueError("column tables cannot be combined with subtwiddle")
@@ -139,6 +192,8 @@ class Butterfly(nn.Module):
             output_size = None
         if conjugate and self.complex:
             twiddle = twiddle.conj()
+        if in_scale is not None or out_scale is not None:
+            twiddle = scale_twiddle(twiddle, self.increasing_stride, in_scale, out_scale)
         if transpose:
             # (prod of stages)^T: transpose every 2x2 and reverse the stage and block order
             twiddle = twiddle.transpose(-1, -2).flip([1, 2])

@@ -15,6 +15,7 @@
 
 #include "common.hpp"
 #include "generic.hpp"
+#include "scale.hpp"
 #include "fast.hpp"
 #include "wide.hpp"
 #include "fast4.hpp"
@@ -1441,6 +1442,77 @@ int bf_butterfly_multiply_base4_bw(const bf_problem *p, const void *twiddle4, co
 {
     return backward(p, true, twiddle2, twiddle4, input, grad, d_twiddle2, d_twiddle4, d_input,
                     workspace, workspace_bytes, stream);
+}
+
+static int scale_twiddle(bool bw, int dtype, int64_t nstacks, int64_t nblocks, int64_t log_n, int increasing_stride,
+                         const void *twiddle, const void *in_scale, int64_t in_len, const void *out_scale,
+                         int64_t out_len, const void *grad, void *out, void *d_in, void *d_out, void *stream)
+{
+    if (dtype != BF_F32 && dtype != BF_C64) return fail(BF_ERR_INVALID, "dtype must be BF_F32 or BF_C64");
+    if (nstacks < 0 || nblocks < 1 || log_n < 1 || log_n > 30)
+        return fail(BF_ERR_INVALID, "nstacks >= 0, nblocks >= 1 and log_n in [1, 30] are required");
+    const int64_t n = (int64_t)1 << log_n;
+    if (nstacks > 65535 || nblocks * log_n > (1 << 20))
+        return fail(BF_ERR_UNSUPPORTED, "more than 65535 stacks or 2^20 stages are not supported");
+    if (in_scale && (in_len < 0 || in_len > n)) return fail(BF_ERR_INVALID, "in_len must be in [0, n]");
+    if (out_scale && (out_len < 0 || out_len > nstacks * n)) return fail(BF_ERR_INVALID, "out_len must be in [0, nstacks * n]");
+    if (nstacks == 0) return BF_OK;
+    if (!twiddle || !out || (bw && !grad)) return fail(BF_ERR_INVALID, "a factor tensor is NULL");
+    if (bw && ((in_scale && in_len > 0 && !d_in) || (out_scale && out_len > 0 && !d_out)))
+        return fail(BF_ERR_INVALID, "a diagonal is given without room for its gradient");
+    ScaleArgs a{};
+    a.tw = twiddle;
+    a.in_scale = in_scale;
+    a.out_scale = out_scale;
+    a.grad = grad;
+    a.out = out;
+    a.d_in = d_in;
+    a.d_out = d_out;
+    a.in_len = in_scale ? in_len : 0;
+    a.out_len = out_scale ? out_len : 0;
+    a.nstacks = (int)nstacks;
+    a.nstages = (int)(nblocks * log_n);
+    a.log_n = (int)log_n;
+    const bool last_increasing = (increasing_stride != 0) != (((nblocks - 1) & 1) != 0);
+    a.first_log_stride = increasing_stride ? 0 : (int)log_n - 1;
+    a.last_log_stride = last_increasing ? (int)log_n - 1 : 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t entries = nstacks * a.nstages * 2 * n;
+    const dim3 grid((unsigned)((entries + kScaleThreads - 1) / kScaleThreads)), block(kScaleThreads);
+    if (!bw) {
+        if (dtype == BF_F32) hipLaunchKernelGGL((scale_twiddle_kernel<float, false>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((scale_twiddle_kernel<float2, false>), grid, block, 0, st, a);
+        BF_HIP_CHECK(hipGetLastError());
+        return BF_OK;
+    }
+    if (dtype == BF_F32) hipLaunchKernelGGL((scale_twiddle_kernel<float, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((scale_twiddle_kernel<float2, true>), grid, block, 0, st, a);
+    BF_HIP_CHECK(hipGetLastError());
+    const int64_t diag = a.in_len + a.out_len;
+    if (diag > 0) {
+        const dim3 dgrid((unsigned)((diag + kScaleThreads - 1) / kScaleThreads));
+        if (dtype == BF_F32) hipLaunchKernelGGL((scale_twiddle_grad_kernel<float>), dgrid, block, 0, st, a);
+        else hipLaunchKernelGGL((scale_twiddle_grad_kernel<float2>), dgrid, block, 0, st, a);
+        BF_HIP_CHECK(hipGetLastError());
+    }
+    return BF_OK;
+}
+
+int bf_butterfly_scale_twiddle(int dtype, int64_t nstacks, int64_t nblocks, int64_t log_n, int increasing_stride,
+                               const void *twiddle, const void *in_scale, int64_t in_len, const void *out_scale,
+                               int64_t out_len, void *scaled, void *stream)
+{
+    return scale_twiddle(false, dtype, nstacks, nblocks, log_n, increasing_stride, twiddle, in_scale, in_len, out_scale,
+                         out_len, nullptr, scaled, nullptr, nullptr, stream);
+}
+
+int bf_butterfly_scale_twiddle_bw(int dtype, int64_t nstacks, int64_t nblocks, int64_t log_n, int increasing_stride,
+                                  const void *twiddle, const void *in_scale, int64_t in_len, const void *out_scale,
+                                  int64_t out_len, const void *grad, void *d_twiddle, void *d_in_scale,
+                                  void *d_out_scale, void *stream)
+{
+    return scale_twiddle(true, dtype, nstacks, nblocks, log_n, increasing_stride, twiddle, in_scale, in_len, out_scale,
+                         out_len, grad, d_twiddle, d_in_scale, d_out_scale, stream);
 }
 
 }  // extern "C"

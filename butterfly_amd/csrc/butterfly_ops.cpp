@@ -393,6 +393,117 @@ Tensor butterfly_multiply_perm(Tensor twiddle, Tensor input, c10::optional<Tenso
     return ButterflyMultiplyPerm::apply(twiddle, input, in_perm, out_index, bias, increasing_stride, output_size);
 }
 
+// ---- diagonals folded into the factors ------------------------------------------------------
+//
+// twiddle (S, nb, log_n, n/2, 2, 2) -> the factors of diag(out_scale) B diag(in_scale): what a
+// Diagonal module in front of / behind a Butterfly (torch_butterfly/diagonal.py:31-38) does to
+// the activations, done to the first / last factor instead.  in_scale up to n entries,
+// out_scale up to S * n, same dtype as twiddle; undefined = no diagonal on that side.
+struct ScaleShapes {
+    int64_t nstacks, nblocks, log_n;
+};
+
+ScaleShapes scale_shapes(const Tensor &twiddle, const Tensor &in_scale, const Tensor &out_scale, const char *who)
+{
+    CHECK_DEVICE(twiddle);
+    CHECK_DIM(twiddle, 6);
+    ScaleShapes s{twiddle.size(0), twiddle.size(1), twiddle.size(2)};
+    TORCH_CHECK(s.log_n >= 1 && s.log_n <= 30 && s.nblocks >= 1, who, ": twiddle must have at least one factor");
+    const int64_t n = (int64_t)1 << s.log_n;
+    CHECK_SHAPE(twiddle, s.nstacks, s.nblocks, s.log_n, n / 2, 2, 2);
+    dtype_code(twiddle, who);
+    for (const Tensor *v : {&in_scale, &out_scale}) {
+        if (!v->defined()) continue;
+        TORCH_CHECK(v->device() == twiddle.device(), who, ": diagonals must be on the device of twiddle");
+        TORCH_CHECK(v->dim() == 1, who, ": diagonals must be vectors");
+        TORCH_CHECK(v->scalar_type() == twiddle.scalar_type(), who, ": diagonals must have the dtype of twiddle");
+    }
+    TORCH_CHECK(!in_scale.defined() || in_scale.size(0) <= n, who, ": in_scale has more than n entries");
+    TORCH_CHECK(!out_scale.defined() || out_scale.size(0) <= s.nstacks * n, who,
+                ": out_scale has more than nstacks * n entries");
+    return s;
+}
+
+Tensor butterfly_scale_twiddle_fw(const Tensor twiddle, c10::optional<Tensor> in_scale,
+                                  c10::optional<Tensor> out_scale, bool increasing_stride)
+{
+    const char *who = "butterfly_scale_twiddle_fw";
+    const Tensor din = opt(in_scale), dout = opt(out_scale);
+    const ScaleShapes s = scale_shapes(twiddle, din, dout, who);
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(twiddle.device());
+    const Tensor tw = dense(twiddle);
+    const Tensor a = din.defined() ? dense(din) : din, b = dout.defined() ? dense(dout) : dout;
+    Tensor out = at::empty_like(tw);
+    check_rc(bf_butterfly_scale_twiddle(dtype_code(tw, who), s.nstacks, s.nblocks, s.log_n, increasing_stride,
+                                        tw.data_ptr(), a.defined() ? a.data_ptr() : nullptr,
+                                        a.defined() ? a.size(0) : 0, b.defined() ? b.data_ptr() : nullptr,
+                                        b.defined() ? b.size(0) : 0, out.data_ptr(), current_stream()),
+             who);
+    return out;
+}
+
+// (d_twiddle, d_in_scale, d_out_scale); an empty tensor stands for the gradient of an absent diagonal
+std::tuple<Tensor, Tensor, Tensor> butterfly_scale_twiddle_bw(const Tensor twiddle, c10::optional<Tensor> in_scale,
+                                                              c10::optional<Tensor> out_scale, const Tensor grad,
+                                                              bool increasing_stride)
+{
+    const char *who = "butterfly_scale_twiddle_bw";
+    const Tensor din = opt(in_scale), dout = opt(out_scale);
+    const ScaleShapes s = scale_shapes(twiddle, din, dout, who);
+    CHECK_DEVICE(grad);
+    TORCH_CHECK(grad.sizes() == twiddle.sizes() && grad.scalar_type() == twiddle.scalar_type() &&
+                    grad.device() == twiddle.device(),
+                who, ": grad must match twiddle in shape, dtype and device");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(twiddle.device());
+    const Tensor tw = dense(twiddle), g = dense(grad);
+    const Tensor a = din.defined() ? dense(din) : din, b = dout.defined() ? dense(dout) : dout;
+    Tensor d_tw = at::empty_like(tw);
+    Tensor d_a = at::empty({a.defined() ? a.size(0) : 0}, tw.options());
+    Tensor d_b = at::empty({b.defined() ? b.size(0) : 0}, tw.options());
+    check_rc(bf_butterfly_scale_twiddle_bw(dtype_code(tw, who), s.nstacks, s.nblocks, s.log_n, increasing_stride,
+                                           tw.data_ptr(), a.defined() ? a.data_ptr() : nullptr,
+                                           a.defined() ? a.size(0) : 0, b.defined() ? b.data_ptr() : nullptr,
+                                           b.defined() ? b.size(0) : 0, g.data_ptr(), d_tw.data_ptr(),
+                                           d_a.data_ptr(), d_b.data_ptr(), current_stream()),
+             who);
+    return {d_tw, d_a, d_b};
+}
+
+class ButterflyScaleTwiddle : public torch::autograd::Function<ButterflyScaleTwiddle> {
+public:
+    static Tensor forward(AutogradContext *ctx, Tensor twiddle, c10::optional<Tensor> in_scale,
+                          c10::optional<Tensor> out_scale, bool increasing_stride)
+    {
+        ctx->saved_data["increasing_stride"] = increasing_stride;
+        ctx->saved_data["has_in"] = in_scale.has_value();
+        ctx->saved_data["has_out"] = out_scale.has_value();
+        variable_list saved = {twiddle};
+        if (in_scale.has_value()) saved.push_back(in_scale.value());
+        if (out_scale.has_value()) saved.push_back(out_scale.value());
+        ctx->save_for_backward(saved);
+        return butterfly_scale_twiddle_fw(twiddle, in_scale, out_scale, increasing_stride);
+    }
+
+    static variable_list backward(AutogradContext *ctx, variable_list grad_output)
+    {
+        const auto saved = ctx->get_saved_variables();
+        const bool has_in = ctx->saved_data["has_in"].toBool(), has_out = ctx->saved_data["has_out"].toBool();
+        c10::optional<Tensor> in_scale, out_scale;
+        size_t next = 1;
+        if (has_in) in_scale = saved[next++];
+        if (has_out) out_scale = saved[next++];
+        auto r = butterfly_scale_twiddle_bw(saved[0], in_scale, out_scale, grad_output[0],
+                                            ctx->saved_data["increasing_stride"].toBool());
+        return {std::get<0>(r), has_in ? std::get<1>(r) : Tensor(), has_out ? std::get<2>(r) : Tensor(), Tensor()};
+    }
+};
+
+Tensor butterfly_scale_twiddle(Tensor twiddle, c10::optional<Tensor> in_scale, c10::optional<Tensor> out_scale,
+                               bool increasing_stride)
+{
+    return ButterflyScaleTwiddle::apply(twiddle, in_scale, out_scale, increasing_stride);
+}
+
 // ---- base-4 -----------------------------------------------------------------------------
 
 Shapes base4_shapes(const Tensor &twiddle4, const Tensor &twiddle2, const Tensor &input, const char *who)
@@ -511,6 +622,9 @@ TORCH_LIBRARY(torch_butterfly, m)
     m.def("butterfly_multiply_perm_fw", butterfly_multiply_perm_fw);
     m.def("butterfly_multiply_perm_bw", butterfly_multiply_perm_bw);
     m.def("butterfly_multiply_perm", butterfly_multiply_perm);
+    m.def("butterfly_scale_twiddle_fw", butterfly_scale_twiddle_fw);
+    m.def("butterfly_scale_twiddle_bw", butterfly_scale_twiddle_bw);
+    m.def("butterfly_scale_twiddle", butterfly_scale_twiddle);
     m.def("butterfly_multiply_base4_fw", butterfly_multiply_base4_fw);
     m.def("butterfly_multiply_base4_bw", butterfly_multiply_base4_bw);
     m.def("butterfly_multiply_base4", butterfly_multiply_base4);

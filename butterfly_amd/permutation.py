@@ -63,39 +63,66 @@ class FixedPermutation(nn.Module):
 
 
 class FusedSequential(nn.Sequential):
-    """nn.Sequential (same children, indexing and state) whose forward folds a
-    FixedPermutation standing directly in front of or behind a Butterfly into that layer's
-    kernels, so it costs no pass of its own over the activations.  Any other sequence of
-    children runs one after the other as usual."""
+    """nn.Sequential (same children, indexing and state) whose forward folds what stands
+    directly around a Butterfly into that layer's own call: a FixedPermutation in front of or
+    behind it becomes part of the kernels' first read / last write, and a Diagonal between that
+    permutation and the layer (or alone next to the layer) is multiplied into the layer's first /
+    last factor, so neither costs a pass of its own over the activations.  The accepted
+    patterns are [FixedPermutation] [Diagonal] Butterfly [Diagonal] [FixedPermutation]; any
+    other sequence of children runs one after the other as usual."""
 
     def forward(self, input):
         from .butterfly import Butterfly, ButterflyBmm  # (butterfly.py does not import this module)
+        from .diagonal import Diagonal
         mods = list(self)
 
         def is_layer(m):
             return isinstance(m, Butterfly) and not isinstance(m, ButterflyBmm)
 
+        def is_perm(m, size):
+            return isinstance(m, FixedPermutation) and m.permutation.dim() == 1 and m.permutation.numel() == size
+
+        def is_scale(m, size, layer):
+            return (isinstance(m, Diagonal) and m.diagonal.dim() == 1 and m.diagonal.numel() == size
+                    and (layer.complex or not m.diagonal.is_complex()))
+
         i = 0
         while i < len(mods):
-            m = mods[i]
-            front = None
-            if (isinstance(m, FixedPermutation) and i + 1 < len(mods) and is_layer(mods[i + 1])
-                    and m.permutation.dim() == 1 and m.permutation.numel() == mods[i + 1].in_size
-                    and input.is_cuda):
-                front, m = m, mods[i + 1]
-                i += 1
-            if is_layer(m) and input.is_cuda:
-                back = None
-                if (i + 1 < len(mods) and isinstance(mods[i + 1], FixedPermutation) and m.nstacks == 1
-                        and mods[i + 1].permutation.dim() == 1 and mods[i + 1].permutation.numel() == m.out_size):
-                    back = mods[i + 1]
-                    i += 1
-                n = 1 << m.log_n
-                input = m(input, in_perm=None if front is None else front.column_table(n, False),
-                          out_index=None if back is None else back.column_table(n, True))
+            # the layer that a permutation and / or a diagonal at position i would lead to
+            j = i
+            while j < len(mods) and j - i < 2 and isinstance(mods[j], (FixedPermutation, Diagonal)):
+                j += 1
+            layer = mods[j] if j < len(mods) and is_layer(mods[j]) else None
+            front = scale_in = None
+            if layer is not None and input.is_cuda and input.is_complex() == layer.complex:
+                lead = mods[i:j]
+                if len(lead) == 2 and is_perm(lead[0], layer.in_size) and is_scale(lead[1], layer.in_size, layer):
+                    front, scale_in = lead
+                elif len(lead) == 1 and is_perm(lead[0], layer.in_size):
+                    front = lead[0]
+                elif len(lead) == 1 and is_scale(lead[0], layer.in_size, layer):
+                    scale_in = lead[0]
+                elif lead:
+                    layer = None
             else:
-                input = m(input)
-            i += 1
+                layer = None if j > i else layer
+            if layer is None or not input.is_cuda or input.is_complex() != layer.complex:
+                input = mods[i](input)
+                i += 1
+                continue
+            i = j + 1
+            back = scale_out = None
+            if i < len(mods) and layer.bias is None and is_scale(mods[i], layer.out_size, layer):
+                scale_out = mods[i]
+                i += 1
+            if i < len(mods) and layer.nstacks == 1 and is_perm(mods[i], layer.out_size):
+                back = mods[i]
+                i += 1
+            n = 1 << layer.log_n
+            input = layer(input, in_perm=None if front is None else front.column_table(n, False),
+                          out_index=None if back is None else back.column_table(n, True),
+                          in_scale=None if scale_in is None else scale_in.diagonal,
+                          out_scale=None if scale_out is None else scale_out.diagonal)
         return input
 
 

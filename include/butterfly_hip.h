@@ -151,6 +151,29 @@ int bf_butterfly_multiply_perm_bw(const bf_problem *p, const void *twiddle, cons
  * csrc/cuda/butterfly_cuda.cu:317-345, internal to the operator).                       */
 int bf_describe_plan(const bf_problem *p, int backward, char *text, size_t capacity);
 
+/* Diagonal matrices directly in front of and behind a butterfly product, folded into its
+ * factors: scaled = the factors of diag(out_scale) B diag(in_scale), i.e. twiddle
+ * (S, nblocks, log_n, n/2, 2, 2) with the columns of the first applied factor multiplied by
+ * in_scale and the rows of the last applied one by out_scale.  in_scale: in_len <= n entries
+ * (every stack reads the same input); out_scale: out_len <= S * n entries (the stacks'
+ * outputs side by side); entries past the lengths count as 1, either pointer may be NULL.
+ * All tensors dense, of the given dtype; no workspace.  Replaces the elementwise passes of
+ * Diagonal modules next to a Butterfly (torch_butterfly/diagonal.py:31-38, as chained by
+ * torch_butterfly/special.py:364-391 and :684-711) by work on the factors alone.          */
+int bf_butterfly_scale_twiddle(int dtype, int64_t nstacks, int64_t nblocks, int64_t log_n,
+                               int increasing_stride, const void *twiddle, const void *in_scale,
+                               int64_t in_len, const void *out_scale, int64_t out_len,
+                               void *scaled, void *stream);
+
+/* Its backward: from grad, the gradient with respect to `scaled`, d_twiddle (shape of
+ * twiddle), d_in_scale (in_len entries) and d_out_scale (out_len entries), all fully
+ * overwritten; PyTorch's convention for complex gradients; fixed summation order.        */
+int bf_butterfly_scale_twiddle_bw(int dtype, int64_t nstacks, int64_t nblocks, int64_t log_n,
+                                  int increasing_stride, const void *twiddle, const void *in_scale,
+                                  int64_t in_len, const void *out_scale, int64_t out_len,
+                                  const void *grad, void *d_twiddle, void *d_in_scale,
+                                  void *d_out_scale, void *stream);
+
 /* Base-4 forward: per block log_n/2 radix-4 stages from twiddle4
  * (S, nb, log_n/2, n/4, 4, 4), then one 2x2 stage from twiddle2 (S, nb, 1, n/2, 2, 2)
  * when log_n is odd (twiddle2 may be NULL when log_n is even).

@@ -755,3 +755,76 @@ def test_library_calls_replay_from_a_captured_graph(shape):
         dtw_e, dx_e, db_e = _capi.multiply_bias_bw(tw, x, g, inc)
         torch.cuda.synchronize()
         assert torch.equal(y, y_e) and torch.equal(dx, dx_e) and torch.equal(dtw, dtw_e) and torch.equal(db, db_e), rep
+
+
+def test_scale_twiddle_through_the_c_abi():
+    """Diagonals folded into the end factors: the library's result against a direct numpy
+    evaluation of diag(out) (factor) diag(in) entry by entry, its gradients against the sums
+    that definition gives (complex ones with the conjugates PyTorch's convention puts there),
+    and the operator's autograd wiring."""
+    from butterfly_amd import _capi
+    import butterfly_amd  # noqa: F401
+    rng = np.random.default_rng(21)
+
+    def element(p, pos, stride):
+        return (p // stride) * 2 * stride + pos * stride + p % stride
+
+    cases = [(np.float32, True, 1, 1, 1, 2, 2), (np.float32, False, 2, 1, 1, 1, 3), (np.complex64, True, 2, 2, 3, 7, 15),
+             (np.float32, False, 1, 2, 10, 1024, 1000), (np.complex64, False, 3, 3, 5, 32, 96), (np.float32, True, 2, 4, 4, 0, 32)]
+    for dtype, inc, S, nb, L, in_len, out_len in cases:
+        n = 1 << L
+        for use_in, use_out in [(True, True), (True, False), (False, True)]:
+            say("scale_twiddle", np.dtype(dtype).name, inc, S, nb, L, in_len, out_len, use_in, use_out)
+            tw = randn(rng, (S, nb, L, n // 2, 2, 2), dtype)
+            d = randn(rng, (in_len,), dtype) if use_in else None
+            e = randn(rng, (out_len,), dtype) if use_out else None
+            g = randn(rng, tw.shape, dtype)
+            fin = np.ones((S, nb * L, n // 2, 2, 2), np.complex128)
+            fout = np.ones_like(fin)
+            s_first = 1 if inc else n // 2
+            s_last = n // 2 if (inc != ((nb - 1) % 2 == 1)) else 1
+            p = np.arange(n // 2)
+            for pos in range(2):
+                if d is not None:
+                    idx = element(p, pos, s_first)
+                    fin[:, 0, :, :, pos] = np.where(idx < in_len, np.concatenate([d, np.ones(n)])[idx], 1)[None, :, None]
+                if e is not None:
+                    for s in range(S):
+                        idx = s * n + element(p, pos, s_last)
+                        fout[s, -1, :, pos, :] = np.where(idx < out_len, np.concatenate([e, np.ones(S * n)])[idx], 1)[:, None]
+            flat = tw.reshape(fin.shape).astype(np.complex128)
+            ref = (flat * fin * fout).reshape(tw.shape)
+            dev = lambda a: None if a is None else torch.from_numpy(a).cuda()
+            got = _capi.scale_twiddle(dev(tw), dev(d), dev(e), inc).cpu().numpy()
+            assert rel_err(got, ref) < 1e-6
+            gf = g.reshape(fin.shape).astype(np.complex128)
+            d_tw_ref = (gf * np.conj(fin * fout)).reshape(tw.shape)
+            d_tw, d_in, d_out = _capi.scale_twiddle_bw(dev(tw), dev(d), dev(e), inc, dev(g))
+            assert rel_err(d_tw.cpu().numpy(), d_tw_ref) < 1e-6
+            if d is not None and in_len:
+                contrib = gf[:, 0] * np.conj(flat[:, 0] * fout[:, 0])          # (S, n/2, r, c)
+                d_in_ref = np.zeros(n, np.complex128)
+                for pos in range(2):
+                    np.add.at(d_in_ref, element(p, pos, s_first), contrib[:, :, :, pos].sum(axis=(0, 2)))
+                assert rel_err(d_in.cpu().numpy(), d_in_ref[:in_len]) < 1e-5
+            if e is not None and out_len:
+                contrib = gf[:, -1] * np.conj(flat[:, -1] * fin[:, -1])
+                d_out_ref = np.zeros((S, n), np.complex128)
+                for pos in range(2):
+                    d_out_ref[:, element(p, pos, s_last)] += contrib[:, :, pos, :].sum(axis=2)
+                assert rel_err(d_out.cpu().numpy(), d_out_ref.reshape(-1)[:out_len]) < 1e-5
+            # the operator under autograd returns the same three gradients
+            t = dev(tw).requires_grad_()
+            dd = None if d is None else dev(d).requires_grad_()
+            ee = None if e is None else dev(e).requires_grad_()
+            y = torch.ops.torch_butterfly.butterfly_scale_twiddle(t, dd, ee, inc)
+            leaves = [v for v in (t, dd, ee) if v is not None]
+            grads = torch.autograd.grad(y, leaves, dev(g))
+            assert torch.equal(grads[0], d_tw)
+            if dd is not None:
+                assert torch.equal(grads[1], d_in)
+            if ee is not None:
+                assert torch.equal(grads[-1], d_out)
+    with pytest.raises(RuntimeError):
+        torch.ops.torch_butterfly.butterfly_scale_twiddle(torch.randn(1, 1, 3, 4, 2, 2).cuda(),
+                                                          torch.randn(9).cuda(), None, True)

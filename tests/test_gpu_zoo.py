@@ -291,3 +291,66 @@ def test_fused_sequential_equals_separate_permutations():
     M = fq(sq(fp(eye))).T                          # columns M e_j
     got = sq(xc, transpose=True, in_perm=fp.column_table(128, False), out_index=fq.column_table(128, True))
     assert close(got, xc @ M, rtol=1e-3, atol=1e-3)
+
+
+def test_fused_sequential_folds_diagonals():
+    """A Diagonal next to a Butterfly inside a FusedSequential is multiplied into the layer's
+    first / last factor; outputs and every gradient (input, factors, diagonals, bias) must
+    match the same children run one after the other."""
+    from torch import nn
+    from butterfly_amd import Butterfly, special
+    from butterfly_amd.diagonal import Diagonal
+    from butterfly_amd.permutation import FixedPermutation, FusedSequential
+    torch.manual_seed(5)
+    calls = []
+
+    def compare(fused, x, folded_layers):
+        plain = nn.Sequential(*fused)
+        hooks = [m.register_forward_hook(lambda mod, a, o: calls.append(type(mod).__name__)) for m in fused]
+        xa = x.clone().requires_grad_()
+        xb = x.clone().requires_grad_()
+        calls.clear()
+        ya = fused(xa)
+        assert calls.count("Diagonal") == 0 and calls.count("Butterfly") == folded_layers, calls
+        yb = plain(xb)
+        for h in hooks:
+            h.remove()
+        assert close(ya, yb, rtol=1e-4, atol=1e-4)
+        g = torch.randn_like(ya)
+        params = list(fused.parameters())
+        ga = torch.autograd.grad(ya, [xa] + params, g)
+        gb = torch.autograd.grad(yb, [xb] + params, g)
+        for a, b in zip(ga, gb):
+            assert close(a, b, rtol=1e-3, atol=1e-3)
+
+    for n, nblocks, inc, cplx in [(8, 1, True, False), (64, 2, False, False), (1024, 2, False, False),
+                                  (256, 3, True, True), (2048, 1, False, False), (2, 1, True, True)]:
+        say("diagonal fold", n, nblocks, inc, cplx)
+        layer = Butterfly(n, n, bias=False, complex=cplx, increasing_stride=inc, nblocks=nblocks).cuda()
+        seq = FusedSequential(Diagonal(n, complex=cplx), layer, Diagonal(n, complex=cplx)).cuda()
+        x = crand(19, n) if cplx else torch.randn(19, n, device="cuda")
+        compare(seq, x, 1)
+    say("diagonals inside permutations, real diagonal on a complex layer")
+    layer = Butterfly(128, 128, bias=False, complex=True, nblocks=2).cuda()
+    seq = FusedSequential(FixedPermutation(torch.randperm(128)), Diagonal(128), layer,
+                          Diagonal(128, complex=True), FixedPermutation(torch.randperm(128))).cuda()
+    compare(seq, crand(6, 128), 1)
+    say("odd sizes, stacks, bias in front of the second diagonal")
+    layer = Butterfly(100, 300, bias=False).cuda()        # n = 128, 3 stacks: both diagonals fold
+    seq = FusedSequential(Diagonal(100), layer, Diagonal(300)).cuda()
+    compare(seq, torch.randn(7, 100, device="cuda"), 1)
+    layer = Butterfly(100, 90, bias=True).cuda()          # bias: only the front diagonal folds
+    seq = FusedSequential(Diagonal(100), layer, Diagonal(90)).cuda()
+    plain = nn.Sequential(*seq)
+    x = torch.randn(7, 100, device="cuda")
+    assert close(seq(x), plain(x), rtol=1e-4, atol=1e-4)
+    say("chains of layers")
+    h = special.hadamard_diagonal(torch.randn(3, 64).sign(), normalized=True, separate_diagonal=True).cuda()
+    assert isinstance(h, FusedSequential)
+    compare(h, torch.randn(11, 64, device="cuda"), 3)
+    say("the layer's own arguments")
+    layer = Butterfly(64, 64, bias=True).cuda()
+    with pytest.raises(ValueError):
+        layer(torch.randn(2, 64, device="cuda"), out_scale=torch.ones(64, device="cuda"))
+    with pytest.raises(ValueError):
+        layer(torch.randn(2, 64, device="cuda"), transpose=True, in_scale=torch.ones(64, device="cuda"))

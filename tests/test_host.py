@@ -132,6 +132,31 @@ def test_torch_restatement_gradients_match_oracle():
         assert rel_err(dx.numpy(), dx_ref) < 1e-12
 
 
+def test_scale_twiddle_folds_diagonals_into_the_end_factors():
+    """diag(out) B diag(in), evaluated by the oracle on twiddles with the diagonals folded in,
+    against the oracle's B applied between explicit elementwise products; short diagonals
+    leave the remaining entries alone."""
+    from butterfly_amd.butterfly import scale_twiddle
+    rng = np.random.default_rng(11)
+    for dtype in (np.float64, np.complex128):
+        for inc in (True, False):
+            for nb, L, S in [(1, 1, 1), (1, 1, 2), (1, 3, 2), (2, 4, 1), (3, 2, 2)]:
+                n = 1 << L
+                tw = randn(rng, (S, nb, L, n // 2, 2, 2), dtype)
+                x = randn(rng, (5, S, n), dtype)
+                d = randn(rng, (max(1, n - 1),), dtype)
+                e = randn(rng, (max(1, S * n - 1),), dtype)
+                dfull = np.concatenate([d, np.ones(n - d.size, dtype)])
+                efull = np.concatenate([e, np.ones(S * n - e.size, dtype)]).reshape(S, n)
+                ref = oracle.butterfly_fw(tw, x * dfull, inc) * efull
+                folded = scale_twiddle(torch.from_numpy(tw), inc, torch.from_numpy(d), torch.from_numpy(e))
+                assert rel_err(oracle.butterfly_fw(folded.numpy(), x, inc), ref) < 1e-12
+                only_in = scale_twiddle(torch.from_numpy(tw), inc, torch.from_numpy(d), None)
+                assert rel_err(oracle.butterfly_fw(only_in.numpy(), x, inc), oracle.butterfly_fw(tw, x * dfull, inc)) < 1e-12
+                only_out = scale_twiddle(torch.from_numpy(tw), inc, None, torch.from_numpy(e))
+                assert rel_err(oracle.butterfly_fw(only_out.numpy(), x, inc), oracle.butterfly_fw(tw, x, inc) * efull) < 1e-12
+
+
 def apply_cpu(b, x):
     """Evaluate a Butterfly module's matrix on the CPU through the oracle (host-logic check
     of the twiddle a constructor produced; the module's own forward needs the device)."""
