@@ -211,8 +211,8 @@ int stage_bit(const bf_problem *p, int t)
 int64_t wide_min_rows(const bf_problem *p)
 {
     if (p->log_n == 12) return p->nblocks == 1 ? 2048 : 8192;
-    if (p->dtype == BF_C64) return 256;
-    return p->nblocks == 1 ? 0 : 1024;
+    if (p->dtype == BF_C64) return p->nblocks == 1 ? 0 : 2048;
+    return p->nblocks == 1 ? 0 : 4096;
 }
 
 PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false)

@@ -211,10 +211,10 @@ WIDE_CASES = [
     (np.float32, 2100, 1, 12, 1, None, None, True),
     (np.float32, 1050, 2, 12, 1, 4000, 4090, False),
     (np.float32, 8200, 1, 12, 2, None, None, True),
-    (np.float32, 1100, 1, 11, 2, None, 2047, False),
+    (np.float32, 4100, 1, 11, 2, None, 2047, False),
     (np.float32, 3, 1, 11, 1, None, None, True),
     (np.complex64, 260, 1, 11, 1, None, None, True),
-    (np.complex64, 130, 2, 11, 2, 2000, None, False),
+    (np.complex64, 1030, 2, 11, 2, 2000, None, False),
 ]
 
 
