@@ -194,6 +194,61 @@ def bbt_ortho_mult_untied(twiddle, input):
     return bbt_mult_untied(_rotation(twiddle), input, fast=False)
 
 
+def _conv2d_patches(twiddle, input, kernel_size, padding):
+    """The (batch * h_out * w_out, kernel_size^2 * c_out / c_in, c_in) operand of the
+    convolution-as-butterflies: one row per output pixel, one stack per kernel position (and
+    copy of the input channels, when c_out is a multiple of c_in)
+    (butterfly_multiply.py:509-520)."""
+    b_in, c_in, h_in, w_in = input.shape
+    positions = kernel_size * kernel_size
+    if twiddle.shape[0] % positions:
+        raise ValueError("twiddle must hold a multiple of kernel_size^2 stacks")
+    copies = twiddle.shape[0] // positions
+    if c_in != 1 << _log2(c_in):
+        raise ValueError("c_in must be a power of 2")
+    h_out = h_in + 2 * padding - (kernel_size - 1)
+    w_out = w_in + 2 * padding - (kernel_size - 1)
+    patches = F.unfold(input, kernel_size=kernel_size, dilation=1, padding=padding, stride=1)
+    patches = patches.view(b_in, c_in, positions, h_out * w_out).permute(0, 3, 2, 1)
+    patches = patches.reshape(b_in * h_out * w_out, positions, 1, c_in)
+    return patches.expand(-1, positions, copies, c_in).reshape(b_in * h_out * w_out, positions * copies, c_in)
+
+
+def butterfly_mult_conv2d(twiddle, input, kernel_size, padding, increasing_stride=True):
+    """twiddle (nstack, log n, n / 2, 2, 2), n = c_in, nstack = kernel_size^2 * c_out / c_in;
+    input (batch, c_in, h, w) -> (batch * h_out * w_out, nstack, c_in): every kernel position's
+    patch through its own butterflies, stride 1, square kernels (butterfly_multiply.py:491-583)."""
+    return butterfly_mult_untied(twiddle, _conv2d_patches(twiddle, input, kernel_size, padding), increasing_stride)
+
+
+def bbt_mult_conv2d(twiddle, input, kernel_size, padding):
+    """The same with B B^T products: twiddle (nstack, nblocks * 2 log n, n / 2, 2, 2)
+    (butterfly_multiply.py:626-664)."""
+    return bbt_mult_untied(twiddle, _conv2d_patches(twiddle, input, kernel_size, padding), fast=False)
+
+
+def butterfly_mult_factors(twiddle, input, increasing_stride=True, return_intermediates=False):
+    """Tied weights without a stack dimension: twiddle (n - 1, 2, 2[, 2]), input (batch, n[, 2])
+    (butterfly_multiply.py:696-730).  The reference runs one kernel per factor, for debugging;
+    here the product is one call, and only ``return_intermediates`` (the input and the value
+    after every factor, stacked) walks the factors one by one, in PyTorch operations."""
+    if not return_intermediates:
+        return butterfly_mult(twiddle.unsqueeze(0), input.unsqueeze(1), increasing_stride).squeeze(1)
+    cplx = input.dim() == 3
+    n = input.shape[1]
+    m = _log2(n)
+    x = _as_complex(input) if cplx else input
+    t = _as_complex(twiddle) if cplx else twiddle
+    values = [x]
+    for log_stride in (range(m) if increasing_stride else range(m - 1, -1, -1)):
+        stride = 1 << log_stride
+        f = t[stride - 1:2 * stride - 1]                             # (stride, 2, 2)
+        pairs = values[-1].reshape(-1, n // (2 * stride), 2, stride)
+        values.append(torch.einsum("srp,bgps->bgrs", f, pairs).reshape(-1, n))
+    out = torch.stack(values)
+    return torch.view_as_real(out) if cplx else out
+
+
 def _tied_blocks(factors, m):
     """Tied factors (nstack, nchunks, n - 1, 2, 2), chunk k running with decreasing (even k) or
     increasing (odd k) stride -> (nstack, nchunks, log n, n / 2, 2, 2) in order of application."""

@@ -285,3 +285,98 @@ def test_bmm_layer_equals_a_loop_over_layers():
     bmm = ButterflyBmm(16, 16, mb, True, False, False, param="odo", nblocks=2).cuda()
     bmm(torch.randn(batch, mb, 16, device="cuda")).square().sum().backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in bmm.parameters())
+
+
+def im2col(x, k, pad):
+    """(b, c, h, w) -> patches (b * h_out * w_out, k * k, c): the input channels under every
+    kernel position of every output pixel, by explicit loops; and the index bookkeeping that
+    lets the adjoint be formed the same way."""
+    b, c, h, w = x.shape
+    xp = np.zeros((b, c, h + 2 * pad, w + 2 * pad), x.dtype)
+    xp[:, :, pad:pad + h, pad:pad + w] = x
+    ho, wo = h + 2 * pad - (k - 1), w + 2 * pad - (k - 1)
+    out = np.zeros((b, ho, wo, k * k, c), x.dtype)
+    for i in range(k):
+        for j in range(k):
+            out[:, :, :, i * k + j, :] = xp[:, :, i:i + ho, j:j + wo].transpose(0, 2, 3, 1)
+    return out.reshape(b * ho * wo, k * k, c)
+
+
+def col2im(dp, shape, k, pad):
+    """Adjoint of im2col: patch gradients (b * h_out * w_out, k * k, c) summed back onto the image."""
+    b, c, h, w = shape
+    ho, wo = h + 2 * pad - (k - 1), w + 2 * pad - (k - 1)
+    dp = dp.reshape(b, ho, wo, k * k, c)
+    dxp = np.zeros((b, c, h + 2 * pad, w + 2 * pad), dp.dtype)
+    for i in range(k):
+        for j in range(k):
+            dxp[:, :, i:i + ho, j:j + wo] += dp[:, :, :, i * k + j, :].transpose(0, 3, 1, 2)
+    return dxp[:, :, pad:pad + h, pad:pad + w]
+
+
+@pytest.mark.parametrize("c,h,w,k,pad,copies", [(8, 5, 6, 3, 1, 1), (16, 4, 4, 3, 0, 2), (4, 7, 3, 1, 0, 3), (32, 6, 6, 5, 2, 1)])
+def test_conv2d_multiplies(c, h, w, k, pad, copies):
+    """butterfly_mult_conv2d / bbt_mult_conv2d: every kernel position's patch through its own
+    butterflies, against explicit patch extraction + the numpy restatement, with the gradient
+    of the image formed by the explicit adjoint of the patch extraction."""
+    from butterfly_amd import legacy
+    m = c.bit_length() - 1
+    rng = np.random.default_rng(700 + c + k)
+    b = 3
+    S = k * k * copies
+    x = rnd(rng, (b, c, h, w))
+    patches = np.repeat(im2col(x, k, pad)[:, :, None, :], copies, axis=2).reshape(-1, S, c)
+    g = rnd(rng, patches.shape)
+    back = lambda t: t.detach().cpu().numpy().astype(np.float64)
+    for inc in (True, False):
+        say("conv2d multiply", c, h, w, k, pad, copies, inc)
+        tw = rnd(rng, (S, m, c // 2, 2, 2)) / math.sqrt(2)
+        y_ref, dtw_ref, dp_ref = lo.butterfly_mult_untied(tw, patches, inc, g)
+        dx_ref = col2im(dp_ref.reshape(-1, k * k, copies, c).sum(axis=2), x.shape, k, pad)
+        tw_d, x_d = dev(tw).requires_grad_(), dev(x).requires_grad_()
+        y = legacy.butterfly_mult_conv2d(tw_d, x_d, k, pad, inc)
+        dtw, dx = grads(y, (tw_d, x_d), dev(g))
+        assert rel_err(back(y), y_ref) < FW_TOL
+        assert rel_err(back(dx), dx_ref) < BW_TOL and rel_err(back(dtw), dtw_ref) < BW_TOL
+    say("bbt conv2d", c, h, w, k, pad, copies)
+    tw = rnd(rng, (S, 2 * 2 * m, c // 2, 2, 2)) / math.sqrt(2)
+    y_ref, dtw_ref, dp_ref = lo.bbt_mult_untied(tw, patches, g)
+    dx_ref = col2im(dp_ref.reshape(-1, k * k, copies, c).sum(axis=2), x.shape, k, pad)
+    tw_d, x_d = dev(tw).requires_grad_(), dev(x).requires_grad_()
+    y = legacy.bbt_mult_conv2d(tw_d, x_d, k, pad)
+    dtw, dx = grads(y, (tw_d, x_d), dev(g))
+    assert rel_err(back(y), y_ref) < FW_TOL
+    assert rel_err(back(dx), dx_ref) < BW_TOL and rel_err(back(dtw), dtw_ref) < BW_TOL
+    # a 1 x 1 kernel with one copy is the plain untied multiply over the pixels
+    if k == 1 and copies == 1:
+        flat = dev(x).permute(0, 2, 3, 1).reshape(-1, 1, c)
+        assert torch.allclose(legacy.butterfly_mult_conv2d(tw_d[:, :m], dev(x), 1, 0, True),
+                              legacy.butterfly_mult_untied(tw_d[:, :m], flat, True))
+
+
+@pytest.mark.parametrize("n,cplx", [(2, False), (16, True), (64, False)])
+def test_mult_factors(n, cplx):
+    """butterfly_mult_factors: the tied product without a stack dimension, and its stack of
+    intermediate values factor by factor."""
+    from butterfly_amd import legacy
+    m = n.bit_length() - 1
+    rng = np.random.default_rng(800 + n)
+    x, g = rnd(rng, (7, n), cplx), rnd(rng, (7, n), cplx)
+    to_dev, back = (pairs, unpairs) if cplx else (dev, lambda t: t.detach().cpu().numpy().astype(np.float64))
+    for inc in (True, False):
+        say("mult_factors", n, cplx, inc)
+        tied = rnd(rng, (n - 1, 2, 2), cplx) / math.sqrt(2)
+        y_ref, dtw_ref, dx_ref = lo.butterfly_mult(tied[None], x[:, None], inc, g[:, None])
+        tw_d, x_d = to_dev(tied).requires_grad_(), to_dev(x).requires_grad_()
+        y = legacy.butterfly_mult_factors(tw_d, x_d, inc)
+        dtw, dx = grads(y, (tw_d, x_d), to_dev(g))
+        assert rel_err(back(y), y_ref[:, 0]) < FW_TOL
+        assert rel_err(back(dx), dx_ref[:, 0]) < BW_TOL and rel_err(back(dtw), dtw_ref[0]) < BW_TOL
+        steps = legacy.butterfly_mult_factors(tw_d, x_d, inc, return_intermediates=True)
+        assert steps.shape[0] == m + 1
+        value = x[:, None]
+        assert rel_err(back(steps[0]), value[:, 0]) < FW_TOL
+        for i, log_stride in enumerate(range(m) if inc else range(m - 1, -1, -1)):
+            value = lo.factor_apply(lo.tied_expand(tied[None], log_stride, n), log_stride, value)
+            assert rel_err(back(steps[i + 1]), value[:, 0]) < FW_TOL
+        assert rel_err(back(steps[-1]), y_ref[:, 0]) < FW_TOL
