@@ -65,6 +65,60 @@ __device__ __forceinline__ float partner4(float v, int lane)
     }
 }
 
+// Forward radix-4 stage on DPP lanes for two rows at once: y = sum_m row[m] * (v of partner m),
+// the partners read through the DPP operand of the multiply-add.  Two rows per block keep two
+// instructions between any write of v0 / v1 (the previous stage's last instructions) and its
+// first DPP read, the wait states that read needs.
+#define BF_FW4_BLOCK(C1, C2, C3)                                                                     \
+    asm volatile("v_mul_f32_e32 %0, %4, %2\n\t"                                                      \
+                 "v_mul_f32_e32 %1, %4, %3\n\t"                                                      \
+                 "v_fmac_f32_dpp %0, %2, %5 " C1 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %1, %3, %5 " C1 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %0, %2, %6 " C2 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %1, %3, %6 " C2 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %0, %2, %7 " C3 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %1, %3, %7 " C3 " row_mask:0xf bank_mask:0xf bound_ctrl:1"           \
+                 : "=&v"(y0), "=&v"(y1)                                                              \
+                 : "v"(v0), "v"(v1), "v"(row[0]), "v"(row[1]), "v"(row[2]), "v"(row[3]))
+
+template <int KQ>
+__device__ __forceinline__ void fw4_pair_dpp(float &v0, float &v1, const float (&row)[4])
+{
+    static_assert(KQ == 0 || KQ == 1, "DPP exchange kinds only");
+    float y0, y1;
+    if constexpr (KQ == 0) BF_FW4_BLOCK("quad_perm:[1,0,3,2]", "quad_perm:[2,3,0,1]", "quad_perm:[3,2,1,0]");
+    else BF_FW4_BLOCK("row_half_mirror", "row_mirror", "row_ror:8");
+    v0 = y0;
+    v1 = y1;
+}
+#undef BF_FW4_BLOCK
+
+// Reverse radix-4 stage on DPP lanes, one row: the column sums acc[m] += g(partner m) * x and
+// g <- sum_m col[m] * g(partner m), every partner read through a DPP operand; the two plain
+// instructions in front are the wait states after the write of g.
+#define BF_BW4_BLOCK(C1, C2, C3)                                                                     \
+    asm volatile("v_fmac_f32_e32 %0, %5, %6\n\t"                                                     \
+                 "v_mul_f32_e32 %4, %7, %5\n\t"                                                      \
+                 "v_fmac_f32_dpp %1, %5, %6 " C1 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %4, %5, %8 " C1 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %2, %5, %6 " C2 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %4, %5, %9 " C2 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %3, %5, %6 " C3 " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"      \
+                 "v_fmac_f32_dpp %4, %5, %10 " C3 " row_mask:0xf bank_mask:0xf bound_ctrl:1"          \
+                 : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "=&v"(d)                  \
+                 : "v"(g), "v"(x), "v"(col[0]), "v"(col[1]), "v"(col[2]), "v"(col[3]))
+
+template <int KQ>
+__device__ __forceinline__ void bw4_dpp(float (&acc)[4], float &g, float x, const float (&col)[4])
+{
+    static_assert(KQ == 0 || KQ == 1, "DPP exchange kinds only");
+    float d;
+    if constexpr (KQ == 0) BF_BW4_BLOCK("quad_perm:[1,0,3,2]", "quad_perm:[2,3,0,1]", "quad_perm:[3,2,1,0]");
+    else BF_BW4_BLOCK("row_half_mirror", "row_mirror", "row_ror:8");
+    g = d;
+}
+#undef BF_BW4_BLOCK
+
 struct Fast4Args {
     const float *tw4;          // factors of this block, stack 0: (L/2, n/4, 4, 4)
     int64_t tw_stack_stride;
@@ -168,13 +222,18 @@ __global__ __launch_bounds__(kFastThreads) void fast4_fw_kernel(Fast4Args a)
             constexpr int s = S;
             constexpr int KQ = P::kind(s);
             if constexpr (P::layout(s) != P::layout_before(s)) transpose(v, P::layout(s));
+            if constexpr (KQ < 2 && R % 2 == 0) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                float y = f.row[s][0] * v[r];
-                y = fmaf(f.row[s][1], partner4<KQ, 1>(v[r], lane), y);
-                y = fmaf(f.row[s][2], partner4<KQ, 2>(v[r], lane), y);
-                y = fmaf(f.row[s][3], partner4<KQ, 3>(v[r], lane), y);
-                v[r] = y;
+                for (int r = 0; r < R; r += 2) fw4_pair_dpp<KQ>(v[r], v[r + 1], f.row[s]);
+            } else {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    float y = f.row[s][0] * v[r];
+                    y = fmaf(f.row[s][1], partner4<KQ, 1>(v[r], lane), y);
+                    y = fmaf(f.row[s][2], partner4<KQ, 2>(v[r], lane), y);
+                    y = fmaf(f.row[s][3], partner4<KQ, 3>(v[r], lane), y);
+                    v[r] = y;
+                }
             }
         });
         if constexpr (P::layout(NS - 1) != 0) transpose(v, 0);
@@ -256,14 +315,20 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
             constexpr int KQ = P::kind(s);
             if constexpr (P::layout(s) != P::layout_before(s)) transpose(v, P::layout(s));
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                act[s][r] = v[r];
-                if constexpr (s + 1 < NS) {
-                    float y = f.row[s][0] * v[r];
-                    y = fmaf(f.row[s][1], partner4<KQ, 1>(v[r], lane), y);
-                    y = fmaf(f.row[s][2], partner4<KQ, 2>(v[r], lane), y);
-                    y = fmaf(f.row[s][3], partner4<KQ, 3>(v[r], lane), y);
-                    v[r] = y;
+            for (int r = 0; r < R; ++r) act[s][r] = v[r];
+            if constexpr (s + 1 < NS) {
+                if constexpr (KQ < 2 && R % 2 == 0) {
+#pragma unroll
+                    for (int r = 0; r < R; r += 2) fw4_pair_dpp<KQ>(v[r], v[r + 1], f.row[s]);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        float y = f.row[s][0] * v[r];
+                        y = fmaf(f.row[s][1], partner4<KQ, 1>(v[r], lane), y);
+                        y = fmaf(f.row[s][2], partner4<KQ, 2>(v[r], lane), y);
+                        y = fmaf(f.row[s][3], partner4<KQ, 3>(v[r], lane), y);
+                        v[r] = y;
+                    }
                 }
             }
         });
@@ -277,6 +342,10 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
                 // the COLUMN of d_twiddle that belongs to its element, dT[r ^ m][r] += g(partner m) * x,
                 // and d_x[r] = sum_m T[r ^ m][r] g(partner m)
                 const float xs = act[s][r];
+                if constexpr (KQ < 2) {
+                    bw4_dpp<KQ>(acc[s], gv[r], xs, f.colm[s]);
+                    continue;
+                }
                 const float g1 = partner4<KQ, 1>(gv[r], lane);
                 const float g2 = partner4<KQ, 2>(gv[r], lane);
                 const float g3 = partner4<KQ, 3>(gv[r], lane);
