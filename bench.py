@@ -202,7 +202,7 @@ def main():
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py measures one GPU; --gpus must be 1 (rows shard trivially, see DESIGN.md)")
+        sys.exit("bench.py measures one GPU; --gpus must be 1 (the rows of a batch would shard across GPUs; only d_twiddle would need a reduction)")
     c = CONFIGS[args.config]
     if args.shape:
         f = args.shape.split(",")
