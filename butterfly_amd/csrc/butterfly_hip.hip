@@ -46,7 +46,7 @@ int fail(int code, const char *fmt, ...)
             return fail(BF_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));     \
     } while (0)
 
-constexpr size_t kLdsBytes = 160 * 1024;        // LDS per compute unit on gfx950
+// (gfx950 has 160 KiB of LDS per compute unit)
 constexpr size_t kGenericFwLds = 128 * 1024;    // most a generic forward workgroup stages
 constexpr size_t kGenericBwLds = 144 * 1024;    // most a generic backward workgroup stages
 constexpr int kMaxGrid = 1 << 30;
