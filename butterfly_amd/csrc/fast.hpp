@@ -437,13 +437,23 @@ struct FastFwArgs {
     int low_bits;              // SpanPlan passes: position of the lowest high bit of the span
 };
 
+// (lets the float-only branch of load_factors compile for complex64, where it is never taken)
+template <typename T>
+__device__ __forceinline__ T from_float(float v);
+template <>
+__device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float2 from_float<float2>(float v) { return make_float2(v, 0.0f); }
+
 // Loads the factor entries each thread needs for every stage: its row (ta, tb) and, for the
 // backward kernel, the off-diagonal entry of its column (tc).
-template <typename T, typename P>
+// `loaded(S)` runs right after stage S has its entries (the backward kernel parks some of them in
+// LDS there, which frees their registers before the next blocks arrive).
+template <typename T, typename P, typename F>
 __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, int64_t stage_stride,
                                              const int (&tw_stage)[kFastMaxStages], int chunk, int low_bits,
                                              const FastCoords &c, T (&ta)[P::NS], T (&tb)[P::NS],
-                                             T (&tc)[P::NS], bool want_tc)
+                                             T (&tc)[P::NS], bool want_tc, F &&loaded)
 {
     const T *twp = reinterpret_cast<const T *>(tw) + stack_off + P::pair_base(chunk) * 4;
     static_for<0, P::NS>([&](auto S) {
@@ -454,10 +464,41 @@ __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, 
         const int r = (e >> bit) & 1;
         const int i = P::pair_index(chunk, e, bit, low_bits);
         const T *Tm = twp + tw_stage[s] * stage_stride + i * 4;
-        ta[s] = Tm[3 * r];   // T[r][r]
-        tb[s] = Tm[r + 1];   // T[r][1 - r]
-        if (want_tc) tc[s] = Tm[2 - r];   // T[1 - r][r]
+        if (sizeof(T) == 4 && want_tc) {
+            // float, all three entries: the whole 2x2 block as one 16-byte load (the factor
+            // tensor is dense and 16-byte aligned), then a pick by r -- a third of the load
+            // instructions, each fully used, instead of three 4-byte loads that each drag a
+            // 16-byte-strided set of cache lines through L1.  (Two entries, or complex64 ones,
+            // are faster loaded one by one.)
+            const float4 b = *reinterpret_cast<const float4 *>(Tm);
+            float pa = r ? b.w : b.x;   // T[r][r]
+            float pb = r ? b.z : b.y;   // T[r][1 - r]
+            float pc = r ? b.y : b.z;   // T[1 - r][r]
+            // pin the picks here: left alone, the compiler keeps the whole blocks (twice the
+            // registers) and picks at the first use
+            asm volatile("" : "+v"(pa), "+v"(pb), "+v"(pc));
+            ta[s] = from_float<T>(pa);
+            tb[s] = from_float<T>(pb);
+            tc[s] = from_float<T>(pc);
+        } else {
+            ta[s] = Tm[3 * r];   // T[r][r]
+            tb[s] = Tm[r + 1];   // T[r][1 - r]
+            if (want_tc) tc[s] = Tm[2 - r];   // T[1 - r][r]
+        }
+        loaded(S);
+        if constexpr (P::NS > 10 && s % 5 == 4) {
+            if (sizeof(T) == 4 && want_tc) __builtin_amdgcn_sched_barrier(0);
+        }
     });
+}
+
+template <typename T, typename P>
+__device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, int64_t stage_stride,
+                                             const int (&tw_stage)[kFastMaxStages], int chunk, int low_bits,
+                                             const FastCoords &c, T (&ta)[P::NS], T (&tb)[P::NS],
+                                             T (&tc)[P::NS], bool want_tc)
+{
+    load_factors<T, P>(tw, stack_off, stage_stride, tw_stage, chunk, low_bits, c, ta, tb, tc, want_tc, [](auto) {});
 }
 
 // Moves the R values a thread holds (one per row in flight) through LDS: written at word
@@ -805,12 +846,13 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 
     T ta[NS], tb[NS], tc[NS], acc_self[NS], acc_cross[NS];
     load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb, tc,
-                                COL);
+                       COL, [&](auto S) {
+                           if constexpr (TB_LDS) lds_tb[S * kFastThreads + t] = tb[S];
+                           if constexpr (S < NTA) lds_ta[S * kFastThreads + t] = ta[S];
+                       });
     static_for<0, NS>([&](auto S) {
         acc_self[S] = zero_of(T());
         acc_cross[S] = zero_of(T());
-        if constexpr (TB_LDS) lds_tb[S * kFastThreads + t] = tb[S];
-        if constexpr (S < NTA) lds_ta[S * kFastThreads + t] = ta[S];
     });
     auto tb_of = [&](auto S) -> T {
         if constexpr (TB_LDS) return lds_tb[S * kFastThreads + t];
