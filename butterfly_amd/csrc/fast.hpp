@@ -785,6 +785,13 @@ __device__ __forceinline__ float pair_g(float2 p) { return p.y; }
 __device__ __forceinline__ float2 pair_x(float4 p) { return make_float2(p.x, p.y); }
 __device__ __forceinline__ float2 pair_g(float4 p) { return make_float2(p.z, p.w); }
 
+// two adjacent entries as one store
+__device__ __forceinline__ void store_pair(float *p, float a, float b) { *reinterpret_cast<float2 *>(p) = make_float2(a, b); }
+__device__ __forceinline__ void store_pair(float2 *p, float2 a, float2 b)
+{
+    *reinterpret_cast<float4 *>(p) = make_float4(a.x, a.y, b.x, b.y);
+}
+
 // The R values a thread holds for one walk (one per row group in flight) as one LDS access.
 template <typename T, int R>
 __device__ __forceinline__ void put_rows(T *base, int idx, const T (&v)[R])
@@ -1096,8 +1103,13 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             const int r = (e >> bit) & 1;
             const int i = P::pair_index(chunk, e, bit, a.low_bits);
             T *d = part + (int64_t)s * a.partial_slot + i * 4;
-            d[3 * r] = acc_self[s];    // dT[r][r]
-            d[COL ? 2 - r : r + 1] = acc_cross[s];   // dT[1 - r][r] (column form) or dT[r][1 - r]
+            // The thread writes row r of the 2x2 block as one access: dT[r][r] is its own sum,
+            // dT[r][1 - r] its own cross sum (row form) or the cross sum of the pair's other
+            // thread, which holds dT[1 - (1 - r)][1 - r] (column form: one more exchange).
+            T other;
+            if constexpr (COL) other = partner<P::kind(s)>(acc_cross[s], c2.bperm_addr);
+            else other = acc_cross[s];
+            store_pair(d + 2 * r, r ? other : acc_self[s], r ? acc_self[s] : other);
         });
     } else {
         // (the factor slots in LDS are dead by now and serve as the staging area)
