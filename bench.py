@@ -30,7 +30,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per backward call of cfg2 (main kernel + reduce) from rocprofv3 FETCH_SIZE / WRITE_SIZE
 # scaled by a 64 MiB copy; see profiles/butterfly_fw_bw_cfg2_hbm_traffic.md
-CFG2_BW_TRAFFIC_BYTES = 289.4e6
+CFG2_BW_TRAFFIC_BYTES = 288.9e6
 
 CONFIGS = {
     # name: batch, nstacks, log_n, nblocks, increasing_stride, complex, base4, backward, cpu sample batch
