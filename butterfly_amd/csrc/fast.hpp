@@ -271,36 +271,11 @@ __device__ __forceinline__ float fw_product(float v, float ta, float tb, int bpe
     return fmaf(ta, v, p);
 }
 
-// complex64 on a DPP exchange: the partner's two words are read through the DPP operands of the
-// four multiply-adds that use them instead of being moved into registers first; the four plain
-// instructions in front are more than the two wait states a DPP read needs after a write of v.
-#define BF_FW_PRODUCT_C64_DPP(CTRL)                                                                 \
-    asm volatile("v_mul_f32_e32 %0, %2, %6\n\t"                                                     \
-                 "v_mul_f32_e32 %1, %2, %7\n\t"                                                     \
-                 "v_fma_f32 %0, -%3, %7, %0\n\t"                                                    \
-                 "v_fmac_f32_e32 %1, %3, %6\n\t"                                                    \
-                 "v_fmac_f32_dpp %0, %6, %4 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"   \
-                 "v_fmac_f32_dpp %1, %7, %4 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"   \
-                 "v_fmac_f32_dpp %0, -%7, %5 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"  \
-                 "v_fmac_f32_dpp %1, %6, %5 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1"        \
-                 : "=&v"(y.x), "=&v"(y.y)                                                           \
-                 : "v"(ta.x), "v"(ta.y), "v"(tb.x), "v"(tb.y), "v"(v.x), "v"(v.y))
-
 template <int K>
 __device__ __forceinline__ float2 fw_product(float2 v, float2 ta, float2 tb, int bperm_addr)
 {
-    if constexpr (K < 4) {
-        float2 y;
-        if constexpr (K == 0) BF_FW_PRODUCT_C64_DPP("quad_perm:[1,0,3,2]");
-        else if constexpr (K == 1) BF_FW_PRODUCT_C64_DPP("quad_perm:[2,3,0,1]");
-        else if constexpr (K == 2) BF_FW_PRODUCT_C64_DPP("row_half_mirror");
-        else BF_FW_PRODUCT_C64_DPP("row_mirror");
-        return y;
-    } else {
-        return mac(mul(ta, v), tb, partner<K>(v, bperm_addr));
-    }
+    return mac(mul(ta, v), tb, partner<K>(v, bperm_addr));
 }
-#undef BF_FW_PRODUCT_C64_DPP
 
 // Per-thread coordinates in both layouts.
 struct FastCoords {
