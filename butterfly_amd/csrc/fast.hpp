@@ -456,8 +456,16 @@ __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, 
             tb[s] = from_float<T>(pb);
             tc[s] = from_float<T>(pc);
         } else {
-            ta[s] = Tm[3 * r];   // T[r][r]
-            tb[s] = Tm[r + 1];   // T[r][1 - r]
+            // the thread's row of the block, T[r][0] and T[r][1], is contiguous: one load
+            if constexpr (sizeof(T) == 4) {
+                const float2 v = *reinterpret_cast<const float2 *>(Tm + 2 * r);
+                ta[s] = r ? v.y : v.x;   // T[r][r]
+                tb[s] = r ? v.x : v.y;   // T[r][1 - r]
+            } else {
+                const float4 v = *reinterpret_cast<const float4 *>(Tm + 2 * r);
+                ta[s] = r ? make_float2(v.z, v.w) : make_float2(v.x, v.y);
+                tb[s] = r ? make_float2(v.x, v.y) : make_float2(v.z, v.w);
+            }
             if (want_tc) tc[s] = Tm[2 - r];   // T[1 - r][r]
         }
         loaded(S);
