@@ -95,8 +95,22 @@ __global__ __launch_bounds__(kFastThreads) void wide_fw_kernel(FastFwArgs a)
                 const int r = (e >> bit) & 1;
                 const int i = ((e >> (bit + 1)) << bit) | (e & ((1 << bit) - 1));
                 const T *Tm = twp + s * a.tw_stage_stride + i * 4;
-                ta[s][q] = Tm[3 * r];
-                tb[s][q] = Tm[r + 1];
+                // the row T[r][0], T[r][1] of the block is contiguous: one load (not at n = 4096,
+                // where 96 entries nearly fill the registers and two plain loads per entry pair measure faster)
+                if constexpr (sizeof(T) == 4 && NS * Q > 32) {
+                    ta[s][q] = Tm[3 * r];
+                    tb[s][q] = Tm[r + 1];
+                } else if constexpr (sizeof(T) == 4) {
+                    const float2 v = *reinterpret_cast<const float2 *>(Tm + 2 * r);
+                    ta[s][q] = r ? v.y : v.x;
+                    tb[s][q] = r ? v.x : v.y;
+                    // (pinned: picked late, the loaded pair and the picks would both stay live)
+                    asm volatile("" : "+v"(ta[s][q]), "+v"(tb[s][q]));
+                } else {
+                    const float4 v = *reinterpret_cast<const float4 *>(Tm + 2 * r);
+                    ta[s][q] = r ? make_float2(v.z, v.w) : make_float2(v.x, v.y);
+                    tb[s][q] = r ? make_float2(v.x, v.y) : make_float2(v.z, v.w);
+                }
             }
         });
     }
