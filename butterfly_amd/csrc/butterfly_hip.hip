@@ -823,6 +823,8 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
             return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
         if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
             return fail(BF_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+        if ((reinterpret_cast<uintptr_t>(tw2) & 15) != 0)
+            return fail(BF_ERR_INVALID, "twiddle must be 16-byte aligned");
         bool bias_done = false;
         rc = multipass_forward(p, mp, tw2, input, output, workspace, in_view, out_view, 0, mp.npass, stream, bias,
                                &bias_done);
@@ -1039,6 +1041,8 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
         return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", pl.total, workspace_bytes);
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
         return fail(BF_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+    if (!base4 && ((reinterpret_cast<uintptr_t>(tw2) | reinterpret_cast<uintptr_t>(d_tw2)) & 15) != 0)
+        return fail(BF_ERR_INVALID, "twiddle and d_twiddle must be 16-byte aligned");
 
     const View x_view = make_view(p->input_stride, std::min(p->input_size, n), in_perm);
     const View g_view = make_view(p->output_stride, std::min(p->output_size, n), out_index);

@@ -55,7 +55,14 @@ void *current_stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(
 void check_rc(int rc, const char *who) { TORCH_CHECK(rc == BF_OK, who, ": ", bf_last_error()); }
 
 // Dense copy of a (small) twiddle tensor; also materialises lazy conjugation.
-Tensor dense(const Tensor &t) { return t.resolve_conj().contiguous(); }
+// dense and 16-byte aligned (the kernels read factor blocks with 16-byte loads): a contiguous view
+// at an odd offset into its storage is copied
+Tensor dense(const Tensor &t)
+{
+    Tensor d = t.resolve_conj().contiguous();
+    if (d.numel() > 0 && (reinterpret_cast<uintptr_t>(d.data_ptr()) & 15) != 0) d = d.clone();
+    return d;
+}
 
 struct Shapes {
     int64_t batch, nstacks, nblocks, log_n, n, input_size;
