@@ -498,10 +498,11 @@ def test_backward_is_bitwise_reproducible():
 
 
 def test_headline_size_properties():
-    """Batch 16384, n = 1024, nblocks = 2, decreasing stride first.  Too big for the scalar
-    oracle in seconds, so: (i) a 512-row slice against the oracle, (ii) linearity in the
-    batch (rows are independent), (iii) the adjoint identity <y, g> = <x, d_input>,
-    (iv) d_twiddle equals the sum of d_twiddle over batch chunks."""
+    """Batch 16384, n = 1024, nblocks = 2, decreasing stride first, through size-independent
+    properties (the element-by-element comparison of all 16384 rows with the oracle is
+    test_gpu_quoted_configs.py::test_headline_shape_at_full_size): (i) a 512-row slice against
+    the oracle, (ii) the adjoint identity <y, g> = <x, d_input>, (iii) d_twiddle equals the sum
+    of d_twiddle over batch chunks (rows are independent)."""
     from butterfly_amd import _capi
     rng = np.random.default_rng(41)
     B, L, nb = 16384, 10, 2
