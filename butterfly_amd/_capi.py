@@ -24,7 +24,10 @@ SYMBOLS = [
     "bf_butterfly_multiply_base4_fw", "bf_butterfly_multiply_base4_fw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw",
+    "bf_butterfly_multiply_bw_noalloc",
 ]
+
+NOALLOC_SCRATCH_BYTES = 48 << 20
 
 
 class Problem(ctypes.Structure):
@@ -82,6 +85,7 @@ def lib():
         L.bf_butterfly_multiply_base4_bw_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_base4_bw_workspace_bytes.restype = sz
         L.bf_butterfly_multiply_base4_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_bw_noalloc.argtypes = [pp, vp, vp, vp, vp, vp, vp]
         _lib = L
     return _lib
 
@@ -304,6 +308,23 @@ def multiply_bw(twiddle, input, grad, increasing_stride):
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_bw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
                                           _ptr(d_twiddle), _ptr(d_input), _ptr(ws), nbytes, _stream()))
+    return d_twiddle, d_input
+
+
+def multiply_bw_noalloc(twiddle, input, grad, increasing_stride, d_twiddle=None, d_input=None):
+    """Backward through the entry point that brings its own scratch area: the caller passes
+    operands and results only (results are allocated here when not given)."""
+    assert twiddle.is_contiguous() and twiddle.is_cuda and input.is_cuda and grad.is_cuda
+    nb, log_n = twiddle.shape[1], twiddle.shape[2]
+    p = make_problem(input, log_n, nb, increasing_stride, grad.shape[2])
+    p.output_stride = _strides(grad)
+    if d_twiddle is None:
+        d_twiddle = torch.empty_like(twiddle)
+    if d_input is None:
+        d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
+    p.d_input_stride = _strides(d_input)
+    _check(lib().bf_butterfly_multiply_bw_noalloc(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
+                                                  _ptr(d_twiddle), _ptr(d_input), _stream()))
     return d_twiddle, d_input
 
 

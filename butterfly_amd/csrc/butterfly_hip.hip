@@ -1232,9 +1232,61 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     return BF_OK;
 }
 
+// ---- built-in scratch for callers that cannot allocate ----------------------------------------
+//
+// One fixed array per GPU, held from the moment the library's code is loaded on that GPU until the
+// process ends.  In host code `scratch` is only a handle for the symbol: the memory is reached
+// through the address hipGetSymbolAddress returns for the device that is current, looked up once
+// per device and kept.  Each GPU has its own copy at its own address.
+constexpr size_t kScratchBytes = (size_t)48 << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];
+
+int scratch_of_current_device(void **ptr)
+{
+    int device = -1;
+    BF_HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices)
+        return fail(BF_ERR_UNSUPPORTED, "device ordinal %d is outside the %d the library keeps scratch addresses for",
+                    device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void *address = nullptr;
+        BF_HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+        if (!address) return fail(BF_ERR_HIP, "hipGetSymbolAddress returned no address for the built-in scratch");
+        g_scratch_ptr[device] = address;
+    }
+    *ptr = g_scratch_ptr[device];
+    return BF_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+int bf_butterfly_multiply_bw_noalloc(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
+                                     void *d_twiddle, void *d_input, void *stream)
+{
+    int rc = check_problem(p, true);
+    if (rc) return rc;
+    const BwPlan pl = plan_bw(p, false);
+    if (!pl.fits)
+        return fail(BF_ERR_UNSUPPORTED, "n = %lld does not fit in LDS for the backward pass",
+                    (long long)((int64_t)1 << p->log_n));
+    if (pl.total > kScratchBytes)
+        return fail(BF_ERR_WORKSPACE,
+                    "this problem needs %zu bytes of scratch, the built-in area holds %zu: use "
+                    "bf_butterfly_multiply_bw with a workspace of the caller's",
+                    pl.total, kScratchBytes);
+    void *area = nullptr;
+    if ((rc = scratch_of_current_device(&area))) return rc;
+    // every partial slice and boundary activation in the area is written by this call's own
+    // launches before anything reads it, so nothing of an earlier call has to be cleared
+    return backward(p, false, twiddle, nullptr, input, grad, d_twiddle, nullptr, d_input, area, kScratchBytes, stream);
+}
 
 int bf_version(void) { return 100; }
 

@@ -194,6 +194,23 @@ int bf_butterfly_multiply_base4_bw(const bf_problem *p, const void *twiddle4,
                                    void *d_twiddle4, void *d_twiddle2, void *d_input,
                                    void *workspace, size_t workspace_bytes, void *stream);
 
+/* bf_butterfly_multiply_bw for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same operands and results,
+ * but the partial sums and intermediate activations live in a fixed area of
+ * BF_NOALLOC_SCRATCH_BYTES that is part of the library's device image (one copy per GPU, held
+ * until the process ends) instead of a workspace argument.  No counterpart in the reference.
+ * The call allocates and frees nothing.  A problem whose backward workspace
+ * (bf_butterfly_multiply_bw_workspace_bytes) exceeds the area is refused with
+ * BF_ERR_WORKSPACE.  The device that is current must be the one `stream` belongs to.  All
+ * calls on one GPU share that GPU's area: calls that overlap in time on one GPU (different
+ * streams or threads) race; calls ordered on one stream are fine.  The first call on a device
+ * looks the area's address up (a host-side query, no allocation); make that call outside a
+ * stream capture.                                                                         */
+#define BF_NOALLOC_SCRATCH_BYTES ((size_t)48 << 20)
+int bf_butterfly_multiply_bw_noalloc(const bf_problem *p, const void *twiddle, const void *input,
+                                     const void *grad, void *d_twiddle, void *d_input,
+                                     void *stream);
+
 #ifdef __cplusplus
 }
 #endif
