@@ -31,9 +31,59 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
+# Kernels whose row pipelines wait for their LDS-direct row fetches with hand-counted
+# `s_waitcnt vmcnt(N)`: N is right only while the compiler adds no memory operation of its own
+# between request and wait, i.e. while nothing spills to scratch memory.
+GATED_KERNELS = ("fast_fw_kernel", "fast_bw_kernel", "wide_fw_kernel", "fast4_fw_kernel", "fast4_bw_kernel",
+                 "fast4g_fw_kernel", "fast4g_bw_kernel")
+RESOURCES = os.path.join(PKG, "kernel_resources.txt")
+
+
+def parse_kernel_resources(text):
+    """{mangled kernel name: {field: int}} from -Rpass-analysis=kernel-resource-usage remarks."""
+    import re
+    kernels, cur = {}, None
+    for line in text.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", line)
+        if m:
+            cur = kernels.setdefault(m.group(1), {})
+            continue
+        m = re.search(r"remark:\s+([A-Za-z ]+?)(?: \[[^\]]*\])?: (\d+)", line)
+        if m and cur is not None:
+            cur[m.group(1).strip()] = int(m.group(2))
+    return kernels
+
+
+def check_kernel_resources(path=RESOURCES):
+    """Names of gated kernels that use scratch memory or spill registers (must be empty), and
+    the number of gated kernels seen."""
+    with open(path) as f:
+        kernels = parse_kernel_resources(f.read())
+    gated = {k: v for k, v in kernels.items() if any(g in k for g in GATED_KERNELS)}
+    bad = [k for k, v in gated.items()
+           if v.get("ScratchSize", 1) != 0 or v.get("VGPRs Spill", 1) != 0 or v.get("SGPRs Spill", 1) != 0]
+    return bad, len(gated)
+
+
 def build_hip():
-    _run(["hipcc", "-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-shared"] + DEVICE_FLAGS +
-         ["-o", LIB_HIP, os.path.join(CSRC, "butterfly_hip.hip")])
+    cmd = (["hipcc", "-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-shared"] + DEVICE_FLAGS +
+           ["-Rpass-analysis=kernel-resource-usage", "-o", LIB_HIP, os.path.join(CSRC, "butterfly_hip.hip")])
+    print("+", " ".join(cmd), flush=True)
+    r = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+    remarks = [l for l in r.stderr.splitlines() if "kernel-resource-usage" in l]
+    other = [l for l in r.stderr.splitlines() if "kernel-resource-usage" not in l]
+    if other:
+        print("\n".join(other), file=sys.stderr, flush=True)
+    if r.returncode != 0:
+        raise subprocess.CalledProcessError(r.returncode, cmd)
+    with open(RESOURCES, "w") as f:
+        f.write("\n".join(remarks) + "\n")
+    bad, seen = check_kernel_resources()
+    if seen == 0:
+        raise RuntimeError("no resource-usage remarks for the register-resident kernels: cannot check for spills")
+    if bad:
+        raise RuntimeError("kernels with hand-counted memory waits use scratch memory or spill: " + ", ".join(bad))
+    print(f"{seen} register-resident kernels: no scratch memory, no spills", flush=True)
     return LIB_HIP
 
 

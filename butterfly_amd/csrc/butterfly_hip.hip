@@ -143,7 +143,32 @@ int ensure_attributes()
     return BF_OK;
 }
 
-constexpr int kNumCU = 256;     // MI355X
+// Compute units of the device that is current, asked once per device.  Grids of the persistent
+// kernels (one workgroup per compute unit), the partial areas and the measured crossovers are
+// sized from it.  Host-only queries on a machine without a device plan for an MI355X (256).
+constexpr int kDefaultNumCU = 256;
+constexpr int kMaxDevices = 64;
+std::mutex g_device_mutex;
+int g_num_cu[kMaxDevices];
+
+int num_cu()
+{
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+        (void)hipGetLastError();
+        return kDefaultNumCU;
+    }
+    std::lock_guard<std::mutex> lock(g_device_mutex);
+    if (g_num_cu[device] == 0) {
+        int count = 0;
+        if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0) {
+            (void)hipGetLastError();
+            count = kDefaultNumCU;
+        }
+        g_num_cu[device] = count;
+    }
+    return g_num_cu[device];
+}
 #ifndef BF_FAST_FW_ROWS
 #define BF_FAST_FW_ROWS 4
 #endif
@@ -337,7 +362,7 @@ FastGrid fast_grid(int64_t batch, int Lk, int64_t lanes, int rows_in_flight, int
     FastGrid g;
     g.slots = 1024 >> Lk;
     g.ngroups = (batch + g.slots - 1) / g.slots;
-    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * wg_per_cu / lanes);
+    const int64_t want = std::max<int64_t>(1, (int64_t)num_cu() * wg_per_cu / lanes);
     const int64_t iters = (g.ngroups + rows_in_flight - 1) / rows_in_flight;
     g.nwg = std::min(want, iters);
     g.groups_per_wg = ((iters + g.nwg - 1) / g.nwg) * rows_in_flight;
@@ -353,7 +378,7 @@ FastGrid wide_grid(int64_t batch, int64_t nstacks)
     FastGrid g;
     g.slots = 1;
     g.ngroups = batch;
-    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU / nstacks);
+    const int64_t want = std::max<int64_t>(1, (int64_t)num_cu() / nstacks);
     g.nwg = std::min(want, batch);
     g.groups_per_wg = (batch + g.nwg - 1) / g.nwg;
     g.nwg = (batch + g.groups_per_wg - 1) / g.groups_per_wg;
@@ -764,7 +789,7 @@ int launch_bias_add(const bf_problem *p, const void *bias, void *output, const V
     a.batch = p->batch;
     a.width = p->output_size;
     const int64_t cols = (p->output_size + kBiasThreads - 1) / kBiasThreads;
-    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * 8 / (cols * p->nstacks));
+    const int64_t want = std::max<int64_t>(1, (int64_t)num_cu() * 8 / (cols * p->nstacks));
     a.nparts = std::min<int64_t>(std::min<int64_t>(want, p->batch), 65535);
     a.rows_per_part = (p->batch + a.nparts - 1) / a.nparts;
     a.nparts = (p->batch + a.rows_per_part - 1) / a.rows_per_part;
@@ -850,7 +875,7 @@ BiasGradPlan plan_bias_grad(const bf_problem *p)
     BiasGradPlan b = {};
     if (p->batch <= 0 || p->nstacks <= 0 || p->output_size <= 0) return b;
     b.cols = (p->output_size + kBiasThreads - 1) / kBiasThreads;
-    const int64_t want = std::max<int64_t>(1, (int64_t)kNumCU * 8 / (b.cols * p->nstacks));
+    const int64_t want = std::max<int64_t>(1, (int64_t)num_cu() * 8 / (b.cols * p->nstacks));
     b.nparts = std::min<int64_t>(std::min<int64_t>(want, p->batch), 65535);
     b.rows_per_part = (p->batch + b.nparts - 1) / b.nparts;
     b.nparts = (p->batch + b.rows_per_part - 1) / b.rows_per_part;
@@ -1156,7 +1181,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                 a.ngroups = g.ngroups;
                 a.groups_per_wg = g.groups_per_wg;
                 nparts = g.nwg;
-                if (k == P - 1 && bias_partial && bias_nparts && q.L == 10 && p->dtype == BF_F32 && g.nwg <= kNumCU) {
+                if (k == P - 1 && bias_partial && bias_nparts && q.L == 10 && p->dtype == BF_F32 && g.nwg <= num_cu()) {
                     a.bias_partial = bias_partial;
                     a.bias_width = p->output_size;
                     *bias_nparts = g.nwg;
@@ -1241,7 +1266,6 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
 constexpr size_t kScratchBytes = (size_t)48 << 20;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
-constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 void *g_scratch_ptr[kMaxDevices];
 
@@ -1377,7 +1401,7 @@ int bf_butterfly_bias_grad(const bf_problem *p, const void *grad, void *d_bias, 
 // stand-alone column sum.
 static size_t bias_area_bytes(const bf_problem *p)
 {
-    const size_t fused = align256((size_t)kNumCU * std::max<int64_t>(p->nstacks, 1) *
+    const size_t fused = align256((size_t)num_cu() * std::max<int64_t>(p->nstacks, 1) *
                                   std::max<int64_t>(p->output_size, 0) * elem_bytes(p->dtype));
     return std::max(fused, plan_bias_grad(p).bytes);
 }

@@ -6,7 +6,10 @@
 // optional output size.  The base-4 operators are new; their argument order follows
 // butterfly_multiply_base4_torch (torch_butterfly/multiply_base4.py:7-8).
 //
-// Device tensors only: there is deliberately no CPU path behind these operators.
+// Device tensors go to the HIP library and nowhere else.  Host tensors are accepted by the three
+// operators the reference has (butterfly_multiply, _fw, _bw), in float, double, complex64 and
+// complex128 as there (csrc/butterfly.cpp:44-52, 84-92), and run on the single-threaded host
+// path of host_path.hpp; the operators that are new here take device tensors only.
 
 #include <ATen/ATen.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
@@ -17,6 +20,7 @@
 #include <tuple>
 
 #include "../../include/butterfly_hip.h"
+#include "host_path.hpp"
 
 namespace {
 
@@ -39,7 +43,86 @@ int dtype_code(const Tensor &t, const char *who)
 
 void require_device(const Tensor &t, const char *who)
 {
-    TORCH_CHECK(t.is_cuda(), who, ": tensors must live on a HIP device; this library has no CPU path");
+    TORCH_CHECK(t.is_cuda(), who, ": tensors must live on a HIP device; this operator has no CPU path");
+}
+
+// ---- host tensors ---------------------------------------------------------------------------
+
+bf_host::Shape host_shape(int64_t batch, int64_t nstacks, int64_t log_n, int64_t nblocks, int64_t input_size,
+                          int64_t output_size, bool increasing_stride)
+{
+    bf_host::Shape sh;
+    sh.batch = batch;
+    sh.nstacks = nstacks;
+    sh.log_n = log_n;
+    sh.nblocks = nblocks;
+    sh.input_size = input_size;
+    sh.output_size = output_size;
+    sh.increasing_stride = increasing_stride;
+    return sh;
+}
+
+void host_strides(int64_t dst[3], const Tensor &t)
+{
+    for (int i = 0; i < 3; ++i) dst[i] = t.stride(i);
+}
+
+// Calls f(T()) with T the host path's scalar type for the tensor's dtype.
+template <typename F>
+void host_dispatch(const Tensor &t, const char *who, F &&f)
+{
+    switch (t.scalar_type()) {
+        case at::kFloat: f(float()); break;
+        case at::kDouble: f(double()); break;
+        case at::kComplexFloat: f(bf_host::Cplx<float>()); break;
+        case at::kComplexDouble: f(bf_host::Cplx<double>()); break;
+        default: TORCH_CHECK(false, who, " not implemented for '", t.scalar_type(), "'");
+    }
+}
+
+Tensor host_multiply_fw(const Tensor &twiddle, const Tensor &input, bool increasing_stride, int64_t log_n,
+                        int64_t output_size, const char *who)
+{
+    const Tensor tw = twiddle.resolve_conj().contiguous();
+    const Tensor x = input.resolve_conj();
+    const int64_t n = (int64_t)1 << log_n;
+    Tensor output = at::empty({x.size(0), x.size(1), n}, x.options());
+    if (output_size < n) output = output.slice(2, 0, output_size);
+    const bf_host::Shape sh = host_shape(x.size(0), x.size(1), log_n, tw.size(1), x.size(2), output_size, increasing_stride);
+    int64_t xs[3], os[3];
+    host_strides(xs, x);
+    host_strides(os, output);
+    host_dispatch(x, who, [&](auto tag) {
+        using T = decltype(tag);
+        bf_host::multiply_fw<T>(sh, static_cast<const T *>(tw.data_ptr()), static_cast<const T *>(x.data_ptr()), xs,
+                                static_cast<T *>(output.data_ptr()), os);
+    });
+    return output;
+}
+
+std::tuple<Tensor, Tensor> host_multiply_bw(const Tensor &twiddle, const Tensor &input, const Tensor &grad,
+                                            bool increasing_stride, int64_t log_n, const char *who)
+{
+    const Tensor tw = twiddle.resolve_conj().contiguous();
+    const Tensor x = input.resolve_conj();
+    const Tensor g = grad.resolve_conj();
+    const int64_t n = (int64_t)1 << log_n;
+    const int64_t input_size = x.size(2);
+    Tensor d_twiddle = at::empty(tw.sizes(), tw.options());
+    Tensor d_input = at::empty({x.size(0), x.size(1), std::max(input_size, n)}, x.options());
+    if (input_size < n) d_input = d_input.slice(2, 0, input_size);
+    const bf_host::Shape sh = host_shape(x.size(0), x.size(1), log_n, tw.size(1), input_size, g.size(2), increasing_stride);
+    int64_t xs[3], gs[3], ds[3];
+    host_strides(xs, x);
+    host_strides(gs, g);
+    host_strides(ds, d_input);
+    host_dispatch(x, who, [&](auto tag) {
+        using T = decltype(tag);
+        bf_host::multiply_bw<T>(sh, static_cast<const T *>(tw.data_ptr()), static_cast<const T *>(x.data_ptr()), xs,
+                                static_cast<const T *>(g.data_ptr()), gs, static_cast<T *>(d_twiddle.data_ptr()),
+                                static_cast<T *>(d_input.data_ptr()), ds);
+    });
+    return std::make_tuple(d_twiddle, d_input);
 }
 
 void set_strides(int64_t dst[3], const Tensor &t)
@@ -118,8 +201,10 @@ Tensor multiply_fw_impl(const Tensor &twiddle, const Tensor &input, const Tensor
     const int64_t output_size_val = output_size.has_value() ? output_size.value() : s.n;
     TORCH_CHECK(output_size_val <= s.n, who, ": output_size must be <= n");
     TORCH_CHECK(output_size_val >= 0, who, ": output_size must be >= 0");
-    require_device(input, who);
     TORCH_CHECK(twiddle.scalar_type() == input.scalar_type(), who, ": twiddle and input must have the same dtype");
+    if (input.is_cpu() && !bias.defined() && !in_perm.defined() && !out_index.defined())
+        return host_multiply_fw(twiddle, input, increasing_stride, s.log_n, output_size_val, who);
+    require_device(input, who);
     Tensor b;
     if (bias.defined()) {
         CHECK_DEVICE(bias); CHECK_SAME_DEVICE(bias, input);
@@ -218,9 +303,13 @@ std::tuple<Tensor, Tensor, Tensor> multiply_bw_impl(const Tensor &twiddle, const
     CHECK_SHAPE(twiddle, s.nstacks, s.nblocks, s.log_n, s.n / 2, 2, 2);
     CHECK_SHAPE(grad, s.batch, s.nstacks, output_size);
     TORCH_CHECK(output_size <= s.n, who, ": grad must have at most n columns");
-    require_device(input, who);
     TORCH_CHECK(twiddle.scalar_type() == input.scalar_type() && grad.scalar_type() == input.scalar_type(), who,
                 ": twiddle, input and grad must have the same dtype");
+    if (input.is_cpu() && !with_bias && !in_perm.defined() && !out_index.defined()) {
+        auto r = host_multiply_bw(twiddle, input, grad, increasing_stride, s.log_n, who);
+        return std::make_tuple(std::get<0>(r), std::get<1>(r), Tensor());
+    }
+    require_device(input, who);
 
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const Tensor tw = dense(twiddle);

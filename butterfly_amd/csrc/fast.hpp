@@ -516,6 +516,42 @@ __device__ __forceinline__ void transpose_rows(T *buf, int wr, int rd, T (&v)[R]
     }
 }
 
+// The hand-counted waits, checked against the order in which the kernels issue their own
+// vector-memory operations.  Counters complete in issue order, so `s_waitcnt vmcnt(N)` waits for
+// everything but the N newest operations; N must be the number of operations issued between the
+// requests for the rows awaited and the wait.
+//
+// Backward kernel: walk from the top of the iteration in which the rows that the next iteration
+// reads are requested (AHEAD - 1 iterations before the one that waits) to the wait in front of
+// the last barrier of the waiting iteration.
+template <typename Q, int R, int AHEAD>
+constexpr int bw_operations_behind_awaited_rows()
+{
+    int younger = 0;
+    for (int j = 1 - AHEAD; j <= 0; ++j) {               // iteration, relative to the waiting one
+        if (j != 1 - AHEAD) younger += 2 * R;            // top: R requests for x, R for the gradient
+        for (int k = 1; k <= Q::K; ++k) {
+            if (k == Q::K && j == 0) return younger;     // the wait, in front of barrier K
+            if (Q::DEFER && k == 1) younger += R;        // deferred stores, right behind barrier 1
+        }
+        if (Q::K == 0 && j == 0) return younger;         // no barriers: the wait precedes the stores
+        if (!Q::DEFER) younger += R;                     // stores closing the iteration
+    }
+    return -1;
+}
+
+// Forward kernel: the rows of the next iteration are requested during the previous one (request
+// r in phase r mod (TT + 1), phase p behind barrier p); behind them come that iteration's R
+// stores and the waiting iteration's requests of the phases in front of its last barrier.
+template <int R, int TT>
+constexpr int fw_operations_behind_awaited_rows()
+{
+    int younger = R;
+    for (int phase = 0; phase < (TT == 0 ? 1 : TT); ++phase)
+        for (int r = 0; r < R; ++r) younger += r % (TT + 1) == phase ? 1 : 0;
+    return younger;
+}
+
 #ifndef BF_FAST_FW_WAVES
 #define BF_FAST_FW_WAVES 4
 #endif
@@ -599,6 +635,7 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     // iteration, requested during the previous one.  Younger than those: the previous
     // iteration's R stores and this iteration's EARLY requests.
     constexpr int YOUNGER = R + EARLY;
+    static_assert(!DIRECT || YOUNGER == fw_operations_behind_awaited_rows<R, TT>(), "wait count of the row fetch");
 
     T nxt[R];
     if constexpr (DIRECT) {
@@ -822,7 +859,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // transpose buffers: [parity][walk][rowwords][R]; where both walks move the same way and
     // R = 1, the two walks share one access as an (x, g) pair: [parity][rowwords] pairs
     __shared__ __align__(16) T lds[Q::K > 0 ? 4 * R * kFastRowWords : 1];
-    __shared__ __align__(16) T lds_carry[Q::DEFER ? R * kFastRowWords : 1];
+    // (two buffers, alternating between iterations: with a single barrier per iteration a fast
+    // wavefront could otherwise write the next iteration's values while a slow one still reads)
+    __shared__ __align__(16) T lds_carry[Q::DEFER ? 2 * R * kFastRowWords : 1];
     __shared__ T lds_tb[TB_LDS ? NS * kFastThreads : 1];
     __shared__ T lds_ta[NTA > 0 ? NTA * kFastThreads : 1];
     // row slots: 4 sets of R for x, then 4 sets of R for the output gradient
@@ -933,13 +972,20 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         // iteration's stores when they come first and, if those requests were made one
         // iteration earlier, that iteration's stores and this iteration's requests.
         constexpr int YOUNGER = ((Q::DEFER && Q::K > 1) ? R : 0) + (AHEAD == 2 ? 3 * R : 0);
+        static_assert(!DIRECT || (Q::K == 0 ? 3 * R : YOUNGER) == bw_operations_behind_awaited_rows<Q, R, AHEAD>(),
+                      "wait count of the row fetch");
         if constexpr (DIRECT) {
             fetch_x(it + 1 + AHEAD);
             fetch_g(it + AHEAD);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const float xv = lds_rows[(((it + 1) & 3) * R + r) * kFastRowWords + (Q::SF ? c.fB : c.fA)];
-                const float gr = lds_rows[((4 + (it & 3)) * R + r) * kFastRowWords + (Q::SB ? c.fB : c.fA)];
+                float gr = lds_rows[((4 + (it & 3)) * R + r) * kFastRowWords + (Q::SB ? c.fB : c.fA)];
+                // A row group past the end of the batch must add nothing to the d_twiddle sums.
+                // Its fetch already asked for zeros (out-of-range offsets), but the sums of the
+                // whole launch should not hang on what a fetch that reads nothing leaves in LDS:
+                // a zero gradient here makes every product of the sweep zero.
+                if (!group_ok(R * it + r)) gr = 0.0f;
                 vF[r] = xv;
                 gv[r] = gr;
                 if constexpr (BIAS_SUM) {
@@ -963,12 +1009,13 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                     if constexpr (hasF) put_rows<T, R>(bufF, wrF, vF);
                     if constexpr (hasB) put_rows<T, R>(bufB, wrB, gv);
                 }
-                if constexpr (Q::DEFER && k == 1) put_rows<T, R>(lds_carry, c.fB, carry);
+                T *carry_buf = lds_carry + (Q::DEFER ? flip * R * kFastRowWords : 0);
+                if constexpr (Q::DEFER && k == 1) put_rows<T, R>(carry_buf, c.fB, carry);
                 if constexpr (DIRECT && k == Q::K) wait_rows_in_lds<YOUNGER>();
                 __syncthreads();
                 if constexpr (Q::DEFER && k == 1) {
                     T done[R];
-                    get_rows<T, R>(lds_carry, c.fA, done);
+                    get_rows<T, R>(carry_buf, c.fA, done);
 #pragma unroll
                     for (int r = 0; r < R; ++r) store_grad(R * (it - 1) + r, done[r]);
                 }

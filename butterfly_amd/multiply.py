@@ -1,7 +1,11 @@
 """Functional entry points of the base-2 butterfly multiply.
 
-``butterfly_multiply{,_fw,_bw}`` call the registered operators (HIP kernels); they are the
-counterparts of the scripted wrappers in the reference's torch_butterfly/multiply.py:8-25.
+``butterfly_multiply{,_fw,_bw}`` call the registered operators (HIP kernels for device tensors;
+host tensors run on the operators' single-threaded host path, as the reference's run on its
+csrc/cpu); they are the counterparts of the scripted wrappers in the reference's
+torch_butterfly/multiply.py:8-25.  The operators that are new here (bias and permutations
+folded in) exist for device tensors only: for host tensors the wrappers below compose them
+from butterfly_multiply and plain tensor operations.
 ``butterfly_multiply_torch`` is a plain-PyTorch restatement of the same product, kept as a
 differentiable cross-check like the reference's (multiply.py:28-51); nothing dispatches to
 it automatically.
@@ -35,6 +39,8 @@ def butterfly_multiply_bias(twiddle: torch.Tensor, input: torch.Tensor, bias: to
     """butterfly_multiply(...) + bias with the addition done by the kernel that writes the
     output; bias (nstacks, output_size or n).  Differentiable in all three tensors.  The
     reference adds the bias as a separate pass (torch_butterfly/butterfly.py:152-169)."""
+    if not input.is_cuda:
+        return butterfly_multiply(twiddle, input, increasing_stride, output_size) + bias
     return torch.ops.torch_butterfly.butterfly_multiply_bias(twiddle, input, bias, increasing_stride,
                                                              output_size)
 
@@ -48,6 +54,18 @@ def butterfly_multiply_perm(twiddle: torch.Tensor, input: torch.Tensor, in_perm:
     FixedPermutation(q) behind the layer is out_index = inverse of q.  Differentiable in
     twiddle, input and bias.  The reference runs each permutation as a separate gather
     (torch_butterfly/permutation.py:55-78)."""
+    if not input.is_cuda:
+        n = 2 * twiddle.shape[3]
+        cols = n if output_size is None else output_size
+        x = input
+        if in_perm is not None:
+            x = fit_last_dim(x, n).index_select(-1, in_perm.long())
+        y = butterfly_multiply(twiddle, x, increasing_stride, None)
+        if bias is not None:
+            y = y + torch.nn.functional.pad(bias, (0, n - cols))
+        if out_index is not None:
+            y = torch.zeros_like(y).index_copy(-1, out_index.long(), y)
+        return y[..., :cols]
     return torch.ops.torch_butterfly.butterfly_multiply_perm(twiddle, input, in_perm, out_index, bias,
                                                              increasing_stride, output_size)
 

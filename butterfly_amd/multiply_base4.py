@@ -28,7 +28,11 @@ def butterfly_multiply_base4_bw(twiddle4, twiddle2, input, grad, increasing_stri
 def butterfly_multiply_base4(twiddle4, twiddle2, input, increasing_stride: bool = True,
                              output_size: Optional[int] = None):
     """twiddle4 (nstacks, nblocks, log_n // 2, n/4, 4, 4); twiddle2 (nstacks, nblocks,
-    log_n % 2, n/2, 2, 2); input (batch, nstacks, input_size).  Differentiable."""
+    log_n % 2, n/2, 2, 2); input (batch, nstacks, input_size).  Differentiable.  Host tensors
+    take the PyTorch formulation below, which is the reference's only base-4 path
+    (torch_butterfly/multiply_base4.py:7-41); the native operators are for device tensors."""
+    if not input.is_cuda:
+        return butterfly_multiply_base4_torch(twiddle4, twiddle2, input, increasing_stride, output_size)
     return torch.ops.torch_butterfly.butterfly_multiply_base4(twiddle4, twiddle2, input,
                                                               increasing_stride, output_size)
 

@@ -71,17 +71,19 @@ def test_operator_schemas_and_host_side_checks():
         ops.butterfly_multiply_fw(tw, x, True, 9)
     with pytest.raises(RuntimeError, match="must have dimension"):
         ops.butterfly_multiply_fw(tw, x[0], True, None)
-    # there is no CPU path: CPU tensors are refused, loudly
+    # host tensors run on the operators' own host path (the reference's three operators only) ...
+    from butterfly_amd.multiply import butterfly_multiply_torch
+    assert torch.allclose(ops.butterfly_multiply_fw(tw, x, True, None), butterfly_multiply_torch(tw, x, True), atol=1e-6)
+    # ... the operators that are new here take device tensors and say so, loudly
     with pytest.raises(RuntimeError, match="no CPU path"):
-        ops.butterfly_multiply_fw(tw, x, True, None)
+        ops.butterfly_multiply_bias_fw(tw, x, torch.randn(1, 8), True, None)
     with pytest.raises(RuntimeError, match="no CPU path"):
-        ops.butterfly_multiply_bw(tw, x, x.clone(), True)
+        ops.butterfly_multiply_base4_fw(torch.randn(1, 1, 1, 2, 4, 4), torch.randn(1, 1, 1, 4, 2, 2), x, True, None)
     # the wrappers are TorchScript-callable like the reference's scripted functions
     @torch.jit.script
     def scripted(t: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
         return torch.ops.torch_butterfly.butterfly_multiply(t, v, True, None)
-    with pytest.raises(RuntimeError, match="no CPU path"):
-        scripted(tw, x)
+    assert torch.equal(scripted(tw, x), ops.butterfly_multiply_fw(tw, x, True, None))
 
 
 @pytest.mark.parametrize("inc", [True, False])
@@ -337,3 +339,102 @@ def test_launch_plans_cover_every_stage_once():
     assert [l.split()[0] for l in _capi.describe_plan(0, 32768, 1, 12, 2, True, True)] == ["low", "span", "low"]
     assert [l.split()[0] for l in _capi.describe_plan(0, 2048, 1, 13, 1, True, True)] == ["low", "span"]
     assert [l.split()[0] for l in _capi.describe_plan(0, 16, 1, 20, 1, True, False)] == ["low", "span", "span"]
+
+
+def test_kernels_with_counted_memory_waits_use_no_scratch_memory():
+    """The register-resident kernels wait for their LDS-direct row fetches with
+    `s_waitcnt vmcnt(N)`, N counted by hand from the kernel's own loads and stores.  A register
+    spill would put scratch loads and stores of the compiler's between request and wait and make
+    N too large: the build records the compiler's resource-usage remarks, and no such kernel may
+    show scratch memory or spills."""
+    from butterfly_amd import build
+    assert os.path.isfile(build.RESOURCES), "run `python -m butterfly_amd.build` first"
+    bad, seen = build.check_kernel_resources()
+    assert seen >= 200, seen     # every fast_* / wide_* / fast4* instantiation reports
+    assert bad == []
+    with open(build.RESOURCES) as f:
+        kernels = build.parse_kernel_resources(f.read())
+    assert max(v["VGPRs"] + v["AGPRs"] for v in kernels.values()) <= 128   # 16 wavefronts per compute unit
+
+
+GOLDEN = os.path.join(ROOT, "tests", "golden", "butterfly_ref_cases.npz")
+
+
+def test_operators_on_host_tensors_match_the_reference_vectors():
+    """Host tensors (float, double, complex64, complex128) run on the operators' own host path:
+    every golden case written from the compiled reference, through
+    torch.ops.torch_butterfly.butterfly_multiply_fw / _bw and through autograd."""
+    import butterfly_amd  # noqa: F401
+    ops = torch.ops.torch_butterfly
+    d = np.load(GOLDEN)
+    ncases = len([k for k in d.files if k.endswith("_meta")])
+    seen, exact = set(), 0
+    for i in range(ncases):
+        tw, x, g = (torch.from_numpy(d[f"c{i}_{k}"]) for k in ("twiddle", "input", "grad"))
+        inc, osz = [int(v) for v in d[f"c{i}_meta"]]
+        osz = None if osz < 0 else osz
+        seen.add(tw.dtype)
+        y = ops.butterfly_multiply_fw(tw, x, bool(inc), osz)
+        dtw, dx = ops.butterfly_multiply_bw(tw, x, g, bool(inc))
+        n = 1 << tw.shape[2]
+        assert y.shape == d[f"c{i}_output"].shape and y.stride() == (x.shape[1] * n, n, 1)
+        tol_fw, tol_bw = (1e-5, 1e-4) if tw.dtype in (torch.float32, torch.complex64) else (1e-12, 1e-11)
+        assert rel_err(y.numpy(), d[f"c{i}_output"]) < tol_fw, i
+        assert rel_err(dx.numpy(), d[f"c{i}_d_input"]) < tol_bw, i
+        assert rel_err(dtw.numpy(), d[f"c{i}_d_twiddle"]) < tol_bw, i
+        exact += int(np.array_equal(y.numpy(), d[f"c{i}_output"]) and np.array_equal(dx.numpy(), d[f"c{i}_d_input"])
+                     and np.array_equal(dtw.numpy(), d[f"c{i}_d_twiddle"]))
+        twr, xr = tw.clone().requires_grad_(), x.clone().requires_grad_()
+        ya = ops.butterfly_multiply(twr, xr, bool(inc), osz)
+        a_dtw, a_dx = torch.autograd.grad(ya, (twr, xr), g)
+        assert torch.equal(ya.detach(), y) and torch.equal(a_dtw, dtw) and torch.equal(a_dx, dx)
+    assert seen == {torch.float32, torch.float64, torch.complex64, torch.complex128}
+    assert exact == ncases      # same operations in the same order as the reference: identical bits
+
+
+@pytest.mark.parametrize("batch,n", [(10, 4096), (300, 512)])
+def test_reference_multiply_test_on_cpu(batch, n):
+    """The reference's own operator test on the 'cpu' device
+    (/root/reference/tests/test_multiply.py:17-59; it skips its large-batch shape there, a smaller
+    batch of the same row length stands in): operator against the PyTorch restatement, forward
+    and both gradients, real and complex, both stride orders, same tolerances."""
+    import math
+    from butterfly_amd.multiply import butterfly_multiply, butterfly_multiply_torch
+    log_n, nstacks, nblocks = int(math.log2(n)), 2, 3
+    torch.manual_seed(n)
+    for cplx in (False, True):
+        for inc in (True, False):
+            dtype = torch.complex64 if cplx else torch.float32
+            twiddle = (torch.randn(nstacks, nblocks, log_n, n // 2, 2, 2, dtype=dtype) / math.sqrt(2)).requires_grad_()
+            x = torch.randn(batch, nstacks, n, dtype=dtype, requires_grad=True)
+            out = butterfly_multiply(twiddle, x, inc)
+            out_t = butterfly_multiply_torch(twiddle, x, inc)
+            assert torch.allclose(out, out_t, rtol=1e-3, atol=1e-5)
+            grad = torch.randn_like(out_t)
+            d_tw, d_x = torch.autograd.grad(out, (twiddle, x), grad)
+            d_tw_t, d_x_t = torch.autograd.grad(out_t, (twiddle, x), grad)
+            assert torch.allclose(d_x, d_x_t, rtol=1e-3, atol=1e-5)
+            assert torch.allclose(d_tw, d_tw_t, rtol=1e-3, atol=1e-5)
+
+
+def test_modules_run_on_host_tensors():
+    """Butterfly / ButterflyBase4 / special.fft on the CPU, as the reference's modules do."""
+    import butterfly_amd
+    from butterfly_amd import special
+    from butterfly_amd.multiply import butterfly_multiply_torch
+    torch.manual_seed(3)
+    layer = butterfly_amd.Butterfly(100, 200, bias=True, nblocks=2)
+    x = torch.randn(5, 100, requires_grad=True)
+    y = layer(x)
+    ref = butterfly_multiply_torch(layer.twiddle, layer.pre_process(x), layer.increasing_stride, None)
+    ref = ref.reshape(5, -1)[:, :200] + layer.bias
+    assert y.shape == (5, 200) and torch.allclose(y, ref, atol=1e-5)
+    y.sum().backward()
+    assert layer.twiddle.grad is not None and x.grad is not None and layer.bias.grad is not None
+    b4 = butterfly_amd.ButterflyBase4(64, 64, bias=False)
+    assert b4(torch.randn(3, 64)).shape == (3, 64)
+    f = special.fft(64, normalized=True)
+    z = torch.randn(4, 64, dtype=torch.complex64)
+    assert torch.allclose(f(z), torch.fft.fft(z, norm="ortho"), atol=1e-5)
+    dbl = butterfly_amd.Butterfly(16, 16, bias=False).double()
+    assert dbl(torch.randn(2, 16, dtype=torch.float64)).dtype == torch.float64
