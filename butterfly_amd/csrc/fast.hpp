@@ -271,10 +271,70 @@ __device__ __forceinline__ float fw_product(float v, float ta, float tb, int bpe
     return fmaf(ta, v, p);
 }
 
+// The same product pinned where it is written, for the backward kernel's replay walk: that
+// kernel issues the stages of its two walks in a chosen order (BwPipe::order), which only holds
+// if the compiler cannot slide one walk's arithmetic past the other's.  DPP kinds only; the
+// plain multiply and the s_nop give the two wait states the DPP read of v needs after a write.
+#define BF_FW_PRODUCT_DPP(CTRL)                                                                       \
+    asm volatile("v_mul_f32_e32 %0, %2, %1\n\t"                                                       \
+                 "s_nop 0\n\t"                                                                        \
+                 "v_fmac_f32_dpp %0, %1, %3 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1"          \
+                 : "=&v"(out)                                                                         \
+                 : "v"(v), "v"(ta), "v"(tb))
+
+template <int K>
+__device__ __forceinline__ float fw_product_pinned(float v, float ta, float tb)
+{
+    static_assert(K >= 0 && K < 4, "DPP exchange kinds only");
+    float out;
+    if constexpr (K == 0) BF_FW_PRODUCT_DPP("quad_perm:[1,0,3,2]");
+    else if constexpr (K == 1) BF_FW_PRODUCT_DPP("quad_perm:[2,3,0,1]");
+    else if constexpr (K == 2) BF_FW_PRODUCT_DPP("row_half_mirror");
+    else BF_FW_PRODUCT_DPP("row_mirror");
+    return out;
+}
+#undef BF_FW_PRODUCT_DPP
+
 template <int K>
 __device__ __forceinline__ float2 fw_product(float2 v, float2 ta, float2 tb, int bperm_addr)
 {
     return mac(mul(ta, v), tb, partner<K>(v, bperm_addr));
+}
+
+// The same stage in two halves, for exchanges that take an LDS round trip: the partner's value is
+// requested first and the arithmetic follows once other work has covered the wait.
+__device__ __forceinline__ float fw_finish(float v, float ta, float tb, float pv)
+{
+    float out;
+    asm volatile("v_mul_f32_e32 %0, %3, %4\n\t"
+                 "v_fmac_f32_e32 %0, %2, %1"
+                 : "=&v"(out)
+                 : "v"(v), "v"(ta), "v"(tb), "v"(pv));
+    return out;
+}
+__device__ __forceinline__ float2 fw_finish(float2 v, float2 ta, float2 tb, float2 pv) { return mac(mul(ta, v), tb, pv); }
+
+template <typename T>
+__device__ __forceinline__ void bw_finish(T &self, T &cross, T &g, T x, T ta, T tc, T gp)
+{
+    fmac_pinned(self, g, x);
+    fmac_pinned(cross, gp, x);
+    g = macc(mul(conj_of(ta), g), tc, gp);
+}
+__device__ __forceinline__ void bw_finish(float &self, float &cross, float &g, float x, float ta, float tc, float gp)
+{
+    fmac_pinned(self, g, x);
+    fmac_pinned(cross, gp, x);
+    g = fmaf(tc, gp, ta * g);
+}
+
+// row form: the partner's x and the partner's conj(tb) * g are both needed
+template <typename T>
+__device__ __forceinline__ void bw_finish_row(T &self, T &cross, T &g, T x, T ta, T px, T pm)
+{
+    fmac_pinned(self, g, x);
+    fmac_pinned(cross, g, px);
+    g = add(mul(conj_of(ta), g), pm);
 }
 
 // Per-thread coordinates in both layouts.
@@ -576,20 +636,43 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     const FastCoords c = fast_coords<L>(t);
     const int col = P::column(chunk, c.eA, a.low_bits);  // column of this thread's element in the full row
 
-    T ta[NS], tb[NS], tc_unused[NS];
-    load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb,
-                       tc_unused, false);
-
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
     const int ng = (int)(g1 - g0);
     const int64_t row_end = g1 * SLOTS < a.batch ? g1 * SLOTS : a.batch;
     const int rows_valid = (int)(row_end - g0 * SLOTS);
     const T *in_base = reinterpret_cast<const T *>(a.in) + g0 * SLOTS * a.in_view.sb + stack * a.in_view.ss;
+    const int in_row = (int)(a.in_view.sb * EB), out_row = (int)(a.out_view.sb * EB);
+
+    // LDS flavour: lane l of wavefront w fetches element 64 w + l of each row group, which lands
+    // at the padded word 65 w + l of the group's slot; `set` alternates between iterations
+    const BufDesc in_desc = make_desc(in_base);
+    const int slot_d = t >> L, col_d = P::column(chunk, t & (n - 1), a.low_bits);
+    const int64_t in_col_d = view_col(a.in_view, col_d);
+    const int in_dma = in_col_d >= 0 ? slot_d * in_row + (int)(in_col_d * a.in_view.se * EB) : kOob;
+    const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
+    auto fetch_row = [&](int grel, int set, int r) {
+        const bool ok = (grel + r) * SLOTS + slot_d < rows_valid;
+        load_row_to_lds(in_desc, rows_addr + (set * R + r) * kFastRowWords * 4, ok ? in_dma : kOob,
+                        (grel + r) * SLOTS * in_row);
+    };
+    // The rows of the first two iterations are requested before anything else: they travel from
+    // HBM while the factors, which mostly come from L2, are loaded.
+    if constexpr (DIRECT) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            fetch_row(0, 0, r);
+            fetch_row(R, 1, r);
+        }
+    }
+
+    T ta[NS], tb[NS], tc_unused[NS];
+    load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb,
+                       tc_unused, false);
+
     const __amdgpu_buffer_rsrc_t in_rs = make_rsrc(in_base);
     const __amdgpu_buffer_rsrc_t out_rs =
         make_rsrc(reinterpret_cast<T *>(a.out) + g0 * SLOTS * a.out_view.sb + stack * a.out_view.ss);
-    const int in_row = (int)(a.in_view.sb * EB), out_row = (int)(a.out_view.sb * EB);
     // thread-constant part of the offsets; the row group adds a wave-uniform part
     const int64_t in_col = view_col(a.in_view, col), out_col = view_col(a.out_view, col);
     const int in_thr = in_col >= 0 ? c.slot * in_row + (int)(in_col * a.in_view.se * EB) : kOob;
@@ -604,18 +687,6 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
             const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
             v[r] = buf_load<T>(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
         }
-    };
-    // LDS flavour: lane l of wavefront w fetches element 64 w + l of each row group, which lands
-    // at the padded word 65 w + l of the group's slot; `set` alternates between iterations
-    const BufDesc in_desc = make_desc(in_base);
-    const int slot_d = t >> L, col_d = P::column(chunk, t & (n - 1), a.low_bits);
-    const int64_t in_col_d = view_col(a.in_view, col_d);
-    const int in_dma = in_col_d >= 0 ? slot_d * in_row + (int)(in_col_d * a.in_view.se * EB) : kOob;
-    const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
-    auto fetch_row = [&](int grel, int set, int r) {
-        const bool ok = (grel + r) * SLOTS + slot_d < rows_valid;
-        load_row_to_lds(in_desc, rows_addr + (set * R + r) * kFastRowWords * 4, ok ? in_dma : kOob,
-                        (grel + r) * SLOTS * in_row);
     };
     // The requests of an iteration are spread over its TT + 1 phases (row r goes out at the
     // start of phase r mod (TT + 1)): sixteen wavefronts asking for R rows each at the same
@@ -639,11 +710,6 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
 
     T nxt[R];
     if constexpr (DIRECT) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            fetch_row(0, 0, r);
-            fetch_row(R, 1, r);
-        }
         wait_rows_in_lds<0>();
         __syncthreads();
     } else {
@@ -792,6 +858,58 @@ struct BwPipe {
             if (bphase(s) == k) return s;
         return -1;
     }
+
+    // Order in which the stages of phase k are issued.  The two walks are independent chains, so
+    // any interleaving is valid; what matters is where the exchanges over lane bits 4 and 5 sit.
+    // Those go through the LDS crossbar (ds_swizzle / ds_bpermute) and take an LDS round trip;
+    // a stage that uses one is issued in two halves (exchange, then the arithmetic on what came
+    // back) with up to two register-exchange stages of the other walk in between, and the walk
+    // that still has such stages ahead keeps enough of the other walk's cheap stages for them.
+    // An entry is walk * 4096 + part * 1024 + (stage's position in its walk's list for the phase);
+    // part 0: whole stage, 1: exchange only, 2: the rest.
+    struct Order {
+        int n;
+        int step[4 * NS + 4];
+    };
+    static constexpr bool f_slow(int k, int i) { return P::kind(f_first(k) + i) >= 4; }
+    static constexpr bool b_slow(int k, int j) { return P::kind(b_first(k) - j) >= 4; }
+    static constexpr Order order(int k)
+    {
+        Order o{};
+        const int nf = f_count(k), nb = b_count(k);
+        int i = 0, j = 0;
+        auto push = [&](int walk, int part, int pos) { o.step[o.n++] = walk * 4096 + part * 1024 + pos; };
+        while (i < nf || j < nb) {
+            const bool lf = i < nf && f_slow(k, i), lb = j < nb && b_slow(k, j);
+            if (lf && lb) {
+                push(0, 1, i); push(1, 1, j); push(0, 2, i); push(1, 2, j);
+                ++i; ++j;
+            } else if (lf) {
+                push(0, 1, i);
+                for (int c = 0; c < 2 && j < nb && !b_slow(k, j); ++c) push(1, 0, j++);
+                push(0, 2, i);
+                ++i;
+            } else if (lb) {
+                push(1, 1, j);
+                for (int c = 0; c < 2 && i < nf && !f_slow(k, i); ++c) push(0, 0, i++);
+                push(1, 2, j);
+                ++j;
+            } else if (j >= nb) {
+                push(0, 0, i++);
+            } else if (i >= nf) {
+                push(1, 0, j++);
+            } else {
+                int need_b = 0, have_b = 0, need_f = 0, have_f = 0;
+                for (int q = i; q < nf; ++q) { need_b += f_slow(k, q) ? 2 : 0; have_f += f_slow(k, q) ? 0 : 1; }
+                for (int q = j; q < nb; ++q) { need_f += b_slow(k, q) ? 2 : 0; have_b += b_slow(k, q) ? 0 : 1; }
+                const bool keep_b = have_b <= need_b, keep_f = have_f <= need_f;
+                if (keep_b && !keep_f) push(0, 0, i++);
+                else if (keep_f && !keep_b) push(1, 0, j++);
+                else { push(1, 0, j++); push(0, 0, i++); }
+            }
+        }
+        return o;
+    }
 };
 
 // (x, g) pair that travels through LDS as one access
@@ -874,23 +992,19 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const int col = P::column(chunk, c.eA, a.low_bits);  // column of this thread's element in the full row
 
     T ta[NS], tb[NS], tc[NS], acc_self[NS], acc_cross[NS];
-    load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb, tc,
-                       COL, [&](auto S) {
-                           if constexpr (TB_LDS) lds_tb[S * kFastThreads + t] = tb[S];
-                           if constexpr (S < NTA) lds_ta[S * kFastThreads + t] = ta[S];
-                       });
-    static_for<0, NS>([&](auto S) {
-        acc_self[S] = zero_of(T());
-        acc_cross[S] = zero_of(T());
-    });
-    auto tb_of = [&](auto S) -> T {
-        if constexpr (TB_LDS) return lds_tb[S * kFastThreads + t];
-        else return tb[S];
+    auto load_all_factors = [&] {
+        load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb,
+                           tc, COL, [&](auto S) {
+                               if constexpr (TB_LDS) lds_tb[S * kFastThreads + t] = tb[S];
+                               if constexpr (S < NTA) lds_ta[S * kFastThreads + t] = ta[S];
+                           });
+        static_for<0, NS>([&](auto S) {
+            acc_self[S] = zero_of(T());
+            acc_cross[S] = zero_of(T());
+        });
     };
-    auto ta_of = [&](auto S) -> T {
-        if constexpr (S < NTA) return lds_ta[S * kFastThreads + t];
-        else return ta[S];
-    };
+    // (rows that arrive in registers: factors first, as the fetch needs no head start in LDS)
+    if constexpr (!DIRECT) load_all_factors();
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
@@ -957,6 +1071,42 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         }
     };
 
+    // The first rows are requested before anything else: they travel from HBM while the factors,
+    // which mostly come from L2, are loaded.
+    if constexpr (DIRECT) {
+        fetch_x(0);
+        fetch_g(-1);  // nothing to sweep yet: rows of zeros
+        if constexpr (AHEAD == 2) {
+            fetch_x(1);
+            fetch_g(0);
+        }
+        load_all_factors();
+    }
+
+    auto tb_of = [&](auto S) -> T {
+        if constexpr (TB_LDS) return lds_tb[S * kFastThreads + t];
+        else return tb[S];
+    };
+    auto ta_of = [&](auto S) -> T {
+        if constexpr (S < NTA) return lds_ta[S * kFastThreads + t];
+        else return ta[S];
+    };
+    // look-ahead ring for the replay walk's off-diagonal entries (float kernels; see the stage loop)
+    constexpr int TB_AHEAD = NS - 1 >= 2 ? 2 : 1;
+    T tb_ring[TB_AHEAD];
+    if constexpr (W == 1 && NS > 1)
+        static_for<0, TB_AHEAD>([&](auto S) { tb_ring[S] = tb_of(std::integral_constant<int, S % (NS - 1)>{}); });
+
+    // rows of iteration `j` out of their LDS slots, in the layouts the two walks start in
+    auto read_rows = [&](int j, T (&xv)[R], T (&gr)[R]) {
+        if constexpr (DIRECT) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                xv[r] = lds_rows[(((j + 1) & 3) * R + r) * kFastRowWords + (Q::SF ? c.fB : c.fA)];
+                gr[r] = lds_rows[((4 + (j & 3)) * R + r) * kFastRowWords + (Q::SB ? c.fB : c.fA)];
+            }
+        }
+    };
     // One pipelined iteration: forward replay of the groups of iteration it + 1 into `nxt`,
     // reverse sweep of the groups of iteration it out of `cur`.  Register flavour: vF / gv
     // enter holding the freshly loaded x and g.  LDS flavour: they are read from the row
@@ -968,6 +1118,11 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // the number of phases is odd.
     auto iteration = [&](auto FLIP, int it, T (&vF)[R], T (&gv)[R], T (&carry)[R], T (&cur)[R][NS], T (&nxt)[R][NS]) {
         constexpr int flip = decltype(FLIP)::value;
+        // The next iteration's rows are read out of LDS a phase ahead of their use, right behind
+        // the barrier that publishes them, where the registers allow (two more live values).
+        constexpr bool PREREAD = DIRECT && Q::K >= 1 && NS * R < 20;
+        T pre_x[R], pre_g[R];
+        T pend_f[R], pend_b[R], pend_b2[R];  // exchanged values on their way (see BwPipe::order)
         // Memory operations issued after the requests the wait is for and before the wait: this
         // iteration's stores when they come first and, if those requests were made one
         // iteration earlier, that iteration's stores and this iteration's requests.
@@ -979,8 +1134,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             fetch_g(it + AHEAD);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const float xv = lds_rows[(((it + 1) & 3) * R + r) * kFastRowWords + (Q::SF ? c.fB : c.fA)];
-                float gr = lds_rows[((4 + (it & 3)) * R + r) * kFastRowWords + (Q::SB ? c.fB : c.fA)];
+                const float xv = vF[r];
+                float gr = gv[r];
                 // A row group past the end of the batch must add nothing to the d_twiddle sums.
                 // Its fetch already asked for zeros (out-of-range offsets), but the sums of the
                 // whole launch should not hang on what a fetch that reads nothing leaves in LDS:
@@ -1013,6 +1168,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 if constexpr (Q::DEFER && k == 1) put_rows<T, R>(carry_buf, c.fB, carry);
                 if constexpr (DIRECT && k == Q::K) wait_rows_in_lds<YOUNGER>();
                 __syncthreads();
+                // the next iteration's rows are in LDS for everybody now: read them here, a
+                // phase of arithmetic ahead of their first use
+                if constexpr (PREREAD && k == Q::K) read_rows(it + 1, pre_x, pre_g);
                 if constexpr (Q::DEFER && k == 1) {
                     T done[R];
                     get_rows<T, R>(carry_buf, c.fA, done);
@@ -1030,30 +1188,89 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             }
             constexpr int cf = Q::f_count(k), cb = Q::b_count(k);
             constexpr int f0 = Q::f_first(k), b0 = Q::b_first(k);
-            static_for<0, (cf > cb ? cf : cb)>([&](auto J) {
-                constexpr int j = J;
-                if constexpr (j < cb) {
-                    // reverse stage: uses the gradient before it passes through the stage
-                    constexpr int s = b0 - j;
-#pragma unroll
-                    for (int r = 0; r < R; ++r) {
+            // complex64: one reverse stage, one forward stage in turn (its exchanges move twice
+            // the words and its register budget has no room for values on their way)
+            if constexpr (W == 2) {
+                static_for<0, (cf > cb ? cf : cb)>([&](auto J) {
+                    constexpr int j = J;
+                    if constexpr (j < cb) {
+                        constexpr int s = b0 - j;
+                        const auto SS = std::integral_constant<int, s>{};
                         if constexpr (COL)
-                            bw_products<P::kind(s)>(acc_self[s], acc_cross[s], gv[r], cur[r][s],
-                                                    ta_of(std::integral_constant<int, s>{}), tc[s], c.bperm_addr);
+                            bw_products<P::kind(s)>(acc_self[s], acc_cross[s], gv[0], cur[0][s], ta_of(SS), tc[s], c.bperm_addr);
                         else
-                            bw_products_row<P::kind(s)>(acc_self[s], acc_cross[s], gv[r], cur[r][s],
-                                                        ta_of(std::integral_constant<int, s>{}),
-                                                        tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
+                            bw_products_row<P::kind(s)>(acc_self[s], acc_cross[s], gv[0], cur[0][s], ta_of(SS), tb_of(SS),
+                                                        c.bperm_addr);
                     }
-                }
-                if constexpr (j < cf) {
-                    constexpr int s = f0 + j;
+                    if constexpr (j < cf) {
+                        constexpr int s = f0 + j;
+                        const auto SS = std::integral_constant<int, s>{};
+                        nxt[0][s] = vF[0];
+                        if constexpr (s + 1 < NS) vF[0] = fw_product<P::kind(s)>(vF[0], ta_of(SS), tb_of(SS), c.bperm_addr);
+                    }
+                });
+            }
+            constexpr auto ord = Q::order(k);
+            static_assert(ord.n >= cf + cb, "every stage of the phase is issued");
+            static_for<0, (W == 1 ? ord.n : 0)>([&](auto I) {
+                constexpr int code = ord.step[I];
+                constexpr int walk = code / 4096, part = (code / 1024) % 4, pos = code % 1024;
+                if constexpr (walk == 1) {
+                    // reverse stage: uses the gradient before it passes through the stage
+                    constexpr int s = b0 - pos;
+                    constexpr int Kd = P::kind(s);
+                    const auto SS = std::integral_constant<int, s>{};
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
-                        nxt[r][s] = vF[r];
-                        if constexpr (s + 1 < NS)
-                            vF[r] = fw_product<P::kind(s)>(vF[r], ta_of(std::integral_constant<int, s>{}),
-                                                           tb_of(std::integral_constant<int, s>{}), c.bperm_addr);
+                        if constexpr (part == 0) {
+                            if constexpr (COL)
+                                bw_products<Kd>(acc_self[s], acc_cross[s], gv[r], cur[r][s], ta_of(SS), tc[s], c.bperm_addr);
+                            else
+                                bw_products_row<Kd>(acc_self[s], acc_cross[s], gv[r], cur[r][s], ta_of(SS), tb_of(SS),
+                                                    c.bperm_addr);
+                        } else if constexpr (part == 1) {
+                            if constexpr (COL) {
+                                pend_b[r] = partner<Kd>(gv[r], c.bperm_addr);
+                            } else {
+                                pend_b[r] = partner<Kd>(cur[r][s], c.bperm_addr);
+                                pend_b2[r] = partner<Kd>(mul(conj_of(tb_of(SS)), gv[r]), c.bperm_addr);
+                            }
+                            // (the request stays in front of the other walk's stages that cover it)
+                            if (r == R - 1) __builtin_amdgcn_sched_barrier(0);
+                        } else {
+                            if constexpr (COL)
+                                bw_finish(acc_self[s], acc_cross[s], gv[r], cur[r][s], ta_of(SS), tc[s], pend_b[r]);
+                            else
+                                bw_finish_row(acc_self[s], acc_cross[s], gv[r], cur[r][s], ta_of(SS), pend_b[r], pend_b2[r]);
+                        }
+                    }
+                } else {
+                    constexpr int s = f0 + pos;
+                    constexpr int Kd = P::kind(s);
+                    const auto SS = std::integral_constant<int, s>{};
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        if constexpr (part != 2) nxt[r][s] = vF[r];
+                        if constexpr (s + 1 < NS) {
+                            if constexpr (part == 1) {
+                                pend_f[r] = partner<Kd>(vF[r], c.bperm_addr);
+                                if (r == R - 1) __builtin_amdgcn_sched_barrier(0);
+                            } else {
+                                // The off-diagonal entry comes out of the look-ahead ring, whose slot is
+                                // refilled at once with the entry TB_AHEAD product stages further on
+                                // (wrapping into the next iteration): the pinned stages keep every LDS read
+                                // where it is written, so the look-ahead has to be spelled out.
+                                // (slot = position in the endless sequence of product stages, modulo
+                                // the ring size: the two unrolled iterations differ when NS - 1 is odd)
+                                constexpr int slot = (s + flip * (NS - 1)) % TB_AHEAD;
+                                const T tbv = tb_ring[slot];
+                                if (r == R - 1)
+                                    tb_ring[slot] = tb_of(std::integral_constant<int, (s + TB_AHEAD) % (NS - 1)>{});
+                                if constexpr (part == 2) vF[r] = fw_finish(vF[r], ta_of(SS), tbv, pend_f[r]);
+                                else if constexpr (Kd < 4) vF[r] = fw_product_pinned<Kd>(vF[r], ta_of(SS), tbv);
+                                else vF[r] = fw_product<Kd>(vF[r], ta_of(SS), tbv, c.bperm_addr);
+                            }
+                        }
                     }
                 }
             });
@@ -1063,6 +1280,13 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         for (int r = 0; r < R; ++r) {
             if constexpr (Q::DEFER) carry[r] = gv[r];
             else store_grad(R * it + r, gv[r]);
+        }
+        if constexpr (DIRECT) {
+            if constexpr (!PREREAD) read_rows(it + 1, vF, gv);
+            else {
+#pragma unroll
+                for (int r = 0; r < R; ++r) { vF[r] = pre_x[r]; gv[r] = pre_g[r]; }
+            }
         }
     };
 
@@ -1077,14 +1301,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // with a deferred closing transpose one more (empty) iteration flushes the last groups
     const int it_end = Q::DEFER ? nit + 1 : nit;
     if constexpr (DIRECT) {
-        fetch_x(0);
-        fetch_g(-1);  // nothing to sweep yet: rows of zeros
-        if constexpr (AHEAD == 2) {
-            fetch_x(1);
-            fetch_g(0);
-        }
         wait_rows_in_lds<0>();
         __syncthreads();
+        read_rows(-1, vF, gv);
         for (int it = -1; it < it_end; it += 2) {
             iteration(std::integral_constant<int, 0>{}, it, vF, gv, carry, actP, actQ);
             iteration(std::integral_constant<int, 1>{}, it + 1, vF, gv, carry, actQ, actP);
