@@ -28,9 +28,39 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per backward call of cfg2 (main kernel + reduce) from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# scaled by a 64 MiB copy; see profiles/butterfly_fw_bw_cfg2_hbm_traffic.md
-CFG2_BW_TRAFFIC_BYTES = 288.9e6
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_all_configs.md")
+KERNEL_SOURCES = os.path.join(ROOT, "butterfly_amd", "csrc")
+
+
+def kernel_source_digest():
+    """Digest of the library's sources: counter readings belong to the build they were taken on."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(KERNEL_SOURCES)):
+        if name.endswith((".hpp", ".hip", ".cpp")):
+            with open(os.path.join(KERNEL_SOURCES, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(config):
+    """HBM bytes per launch set of the dominant call of `config`, from the rocprofv3 FETCH_SIZE /
+    WRITE_SIZE table under profiles/ (a line `| config | digest | bytes | ...`), or None when
+    there is no reading for this configuration or the sources have changed since it was taken."""
+    try:
+        with open(TRAFFIC_TABLE) as f:
+            lines = f.read().splitlines()
+    except OSError:
+        return None
+    digest = kernel_source_digest()
+    for line in lines:
+        cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 3 and cells[0] == config and cells[1] == digest:
+            try:
+                return float(cells[2])
+            except ValueError:
+                return None
+    return None
 
 CONFIGS = {
     # name: batch, nstacks, log_n, nblocks, increasing_stride, complex, base4, backward, cpu sample batch
@@ -45,20 +75,22 @@ CONFIGS = {
                  workload="cfg2: butterfly_multiply fw+bw, input (16384,1,1024) fp32 N(0,1), twiddle "
                           "(1,2,10,512,2,2) N(0,1/2), increasing_stride=False, grad N(0,1)"),
     "cfg3": dict(batch=8192, nstacks=1, log_n=12, nblocks=1, inc=True, cplx=True, base4=False, bw=True,
-                 cpu_batch=256,
+                 cpu_batch=256, autograd=True,
                  metric="butterfly_multiply fwd+bwd GB/s, complex64 FFT twiddles, batch 8192 n=4096",
                  workload="cfg3: butterfly_multiply fw+bw complex64, normalised DFT twiddles (1,1,12,2048,2,2), "
-                          "input (8192,1,4096) bit-reversed outside the op, increasing_stride=True"),
+                          "input (8192,1,4096) bit-reversed outside the op, increasing_stride=True; the "
+                          "butterfly_multiply operator under autograd (forward, then torch.autograd.grad)"),
     "cfg4": dict(batch=16384, nstacks=4, log_n=8, nblocks=1, inc=True, cplx=False, base4=True, bw=True,
                  cpu_batch=2048,
                  metric="butterfly_multiply_base4 fwd+bwd GB/s, batch 16384 nstacks 4 n=256 fp32",
                  workload="cfg4: butterfly_multiply_base4 fw+bw, input (16384,4,256) fp32 N(0,1), twiddle4 "
                           "(4,1,4,64,4,4) N(0,1/4), increasing_stride=True"),
     "cfg5": dict(batch=32768, nstacks=1, log_n=12, nblocks=2, inc=True, cplx=False, base4=False, bw=True,
-                 cpu_batch=1024,
+                 cpu_batch=1024, autograd=True,
                  metric="butterfly_multiply fwd+bwd GB/s (op level), batch 32768 n=4096 fp32 nblocks 2",
                  workload="cfg5 (op level): butterfly_multiply fw+bw of Butterfly(4096, 4096, nblocks=2), input "
-                          "(32768,1,4096) fp32 N(0,1), ortho twiddle (1,2,12,2048,2,2), increasing_stride=True"),
+                          "(32768,1,4096) fp32 N(0,1), ortho twiddle (1,2,12,2048,2,2), increasing_stride=True; the "
+                          "butterfly_multiply operator under autograd (forward, then torch.autograd.grad)"),
     "cfg5m": dict(batch=32768, nstacks=1, log_n=12, nblocks=2, inc=True, cplx=False, base4=False, bw=True,
                   cpu_batch=1024, module="fused",
                   metric="Butterfly(4096,4096,bias) module fwd+bwd GB/s, batch 32768 fp32 nblocks 2",
@@ -290,6 +322,15 @@ def main():
     elif c["base4"]:
         fw_call = lambda: ops.butterfly_multiply_base4_fw(tws[0], tws[1], x, inc, None)
         bw_call = lambda: ops.butterfly_multiply_base4_bw(tws[0], tws[1], x, grad, inc)
+    elif c.get("autograd"):
+        # the differentiable operator, as a training step calls it: its forward keeps what a backward
+        # in several passes would otherwise recompute
+        twg, xg = tws[0].requires_grad_(), x.requires_grad_()
+        state = {}
+
+        def fw_call():
+            state["y"] = ops.butterfly_multiply(twg, xg, inc, None)
+        bw_call = lambda: torch.autograd.grad(state["y"], (twg, xg), grad)
     else:
         fw_call = lambda: ops.butterfly_multiply_fw(tws[0], x, inc, None)
         bw_call = lambda: ops.butterfly_multiply_bw(tws[0], x, grad, inc)
@@ -348,7 +389,7 @@ def main():
         "fw_GBps": fw_b / (fw_ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "kernel": dom_name, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": dom_gbs / HBM_PEAK_GBS,
-                     "traffic": CFG2_BW_TRAFFIC_BYTES if args.config == "cfg2" else None},
+                     "traffic": measured_traffic(args.config)},
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.config, c)

@@ -25,6 +25,8 @@ SYMBOLS = [
     "bf_butterfly_multiply_base4_bw_workspace_bytes",
     "bf_butterfly_multiply_base4_bw",
     "bf_butterfly_multiply_bw_noalloc",
+    "bf_butterfly_multiply_saved_bytes", "bf_butterfly_multiply_fw_saving",
+    "bf_butterfly_multiply_bw_saved_workspace_bytes", "bf_butterfly_multiply_bw_saved",
 ]
 
 NOALLOC_SCRATCH_BYTES = 48 << 20
@@ -86,6 +88,12 @@ def lib():
         L.bf_butterfly_multiply_base4_bw_workspace_bytes.restype = sz
         L.bf_butterfly_multiply_base4_bw.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_bw_noalloc.argtypes = [pp, vp, vp, vp, vp, vp, vp]
+        L.bf_butterfly_multiply_saved_bytes.argtypes = [pp]
+        L.bf_butterfly_multiply_saved_bytes.restype = sz
+        L.bf_butterfly_multiply_fw_saving.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_bw_saved_workspace_bytes.argtypes = [pp, ctypes.c_int]
+        L.bf_butterfly_multiply_bw_saved_workspace_bytes.restype = sz
+        L.bf_butterfly_multiply_bw_saved.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
         _lib = L
     return _lib
 
@@ -326,6 +334,39 @@ def multiply_bw_noalloc(twiddle, input, grad, increasing_stride, d_twiddle=None,
     _check(lib().bf_butterfly_multiply_bw_noalloc(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
                                                   _ptr(d_twiddle), _ptr(d_input), _stream()))
     return d_twiddle, d_input
+
+
+def multiply_fw_bw_saving(twiddle, input, grad, increasing_stride, output_size=None, bias=None, in_perm=None,
+                          out_index=None):
+    """Forward that leaves the backward's intermediate activations behind, then the backward that
+    reads them.  Returns (output, d_twiddle, d_input, d_bias or None), or None when the problem
+    saves nothing."""
+    assert twiddle.is_contiguous() and twiddle.is_cuda and input.is_cuda and grad.is_cuda
+    nb, log_n = twiddle.shape[1], twiddle.shape[2]
+    n = 1 << log_n
+    O = n if output_size is None else output_size
+    p = make_problem(input, log_n, nb, increasing_stride, O)
+    out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
+    p.output_stride = _strides(out)
+    d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
+    p.d_input_stride = _strides(d_input)
+    nsaved = lib().bf_butterfly_multiply_saved_bytes(ctypes.byref(p))
+    if nsaved == 0:
+        return None
+    saved = torch.empty(nsaved, dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_fw_saving(ctypes.byref(p), _ptr(twiddle), _ptr(input),
+                                                 None if bias is None else _ptr(bias), _table(in_perm, n),
+                                                 _table(out_index, n), _ptr(out), _ptr(saved), nsaved, _stream()))
+    assert tuple(grad.shape) == tuple(out.shape)
+    p.output_stride = _strides(grad)
+    d_twiddle = torch.empty_like(twiddle)
+    d_bias = None if bias is None else torch.empty_like(bias)
+    nbytes = lib().bf_butterfly_multiply_bw_saved_workspace_bytes(ctypes.byref(p), int(bias is not None))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_bw_saved(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad), _ptr(saved),
+                                                _table(in_perm, n), _table(out_index, n), _ptr(d_twiddle), _ptr(d_input),
+                                                None if d_bias is None else _ptr(d_bias), _ptr(ws), nbytes, _stream()))
+    return out, d_twiddle, d_input, d_bias
 
 
 def multiply_base4_fw(twiddle4, twiddle2, input, increasing_stride, output_size=None):

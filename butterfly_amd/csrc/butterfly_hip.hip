@@ -920,7 +920,9 @@ struct BwPlan {
     bool fast4;         // base-4 register-resident kernels, one launch per block
 };
 
-BwPlan plan_bw(const bf_problem *p, bool base4)
+// saved_boundaries: the activations entering every pass after the first come from the caller
+// (left behind by the forward call that saves them) instead of being recomputed into the workspace.
+BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false)
 {
     BwPlan pl = {};
     const int64_t n = (int64_t)1 << p->log_n;
@@ -964,7 +966,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4)
         pl.nparts = nparts;
         size_t off = 0;
         pl.off_boundaries = off;
-        off += mp.npass > 1 ? (size_t)(mp.npass - 1) * pl.boundary_bytes : 0;
+        off += mp.npass > 1 && !saved_boundaries ? (size_t)(mp.npass - 1) * pl.boundary_bytes : 0;
         pl.off_gbuf = off;
         off += mp.npass > 1 ? pl.boundary_bytes : 0;
         pl.off_partials = off;
@@ -1049,7 +1051,7 @@ int launch_reduce(const bf_problem *p, const Schedule &sc, int t0, int t1, int64
 int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, const void *input,
              const void *grad, void *d_tw2, void *d_tw4, void *d_input, void *workspace,
              size_t workspace_bytes, void *stream_, void *bias_partial = nullptr, int64_t *bias_nparts = nullptr,
-             const int *in_perm = nullptr, const int *out_index = nullptr)
+             const int *in_perm = nullptr, const int *out_index = nullptr, const void *saved = nullptr)
 {
     if (bias_nparts) *bias_nparts = 0;
     int rc = check_problem(p, true);
@@ -1059,9 +1061,10 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const Schedule sc = make_schedule(p, base4);
     const int64_t n = (int64_t)1 << p->log_n;
-    const BwPlan pl = plan_bw(p, base4);
+    const BwPlan pl = plan_bw(p, base4, saved != nullptr);
     if (!pl.fits)
         return fail(BF_ERR_UNSUPPORTED, "n = %lld does not fit in LDS for the backward pass", (long long)n);
+    if (saved && !pl.fast) return fail(BF_ERR_INVALID, "this problem has no saved activations");
     if (pl.total > 0 && (!workspace || workspace_bytes < pl.total))
         return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", pl.total, workspace_bytes);
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
@@ -1145,9 +1148,10 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     if (pl.fast) {
         const PassPlan mp = build_passes(p, base4);
         const int P = mp.npass;
-        auto boundary = [&](int k) { return ws + pl.off_boundaries + (size_t)(k - 1) * pl.boundary_bytes; };
+        char *bounds = saved ? const_cast<char *>(static_cast<const char *>(saved)) : ws + pl.off_boundaries;
+        auto boundary = [&](int k) { return bounds + (size_t)(k - 1) * pl.boundary_bytes; };
         // forward replay: boundary k = activation entering pass k (k >= 1)
-        for (int k = 0; k + 1 < P; ++k) {
+        for (int k = 0; k + 1 < P && !saved; ++k) {
             rc = multipass_forward(p, mp, tw2, k == 0 ? input : boundary(k), boundary(k + 1), nullptr,
                                    k == 0 ? x_view : dense, dense, k, k + 1, stream);
             if (rc) return rc;
@@ -1414,11 +1418,11 @@ size_t bf_butterfly_multiply_bias_bw_workspace_bytes(const bf_problem *p)
 
 static int bias_backward(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
                          void *d_twiddle, void *d_input, void *d_bias, void *workspace, size_t workspace_bytes,
-                         void *stream, const int *in_perm, const int *out_index)
+                         void *stream, const int *in_perm, const int *out_index, const void *saved = nullptr)
 {
     int rc = check_problem(p, true);
     if (rc) return rc;
-    const size_t main_bytes = align256(plan_bw(p, false).total);
+    const size_t main_bytes = align256(plan_bw(p, false, saved != nullptr).total);
     const size_t need = main_bytes + bias_area_bytes(p);
     if (!workspace || workspace_bytes < need)
         return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
@@ -1426,7 +1430,7 @@ static int bias_backward(const bf_problem *p, const void *twiddle, const void *i
     char *area = static_cast<char *>(workspace) + main_bytes;
     int64_t nparts = 0;
     rc = backward(p, false, twiddle, nullptr, input, grad, d_twiddle, nullptr, d_input, workspace, main_bytes, stream,
-                  area, &nparts, in_perm, out_index);
+                  area, &nparts, in_perm, out_index, saved);
     if (rc) return rc;
     if (p->nstacks <= 0 || p->output_size <= 0) return BF_OK;
     if (nparts > 0) {
@@ -1470,6 +1474,84 @@ int bf_butterfly_multiply_perm_bw(const bf_problem *p, const void *twiddle, cons
                              in_perm, out_index);
     return backward(p, false, twiddle, nullptr, input, grad, d_twiddle, nullptr, d_input, workspace, workspace_bytes,
                     stream, nullptr, nullptr, in_perm, out_index);
+}
+
+// Bytes of activations the saving forward leaves for the backward: one dense (B, S, n) plane per
+// pass of the backward plan after the first; 0 when the backward is a single pass (or runs on
+// kernels that do not use such planes).
+static size_t saved_bytes(const bf_problem *p)
+{
+    const BwPlan pl = plan_bw(p, false, true);
+    if (!pl.fits || !pl.fast || pl.nchunks <= 1) return 0;
+    return (size_t)(pl.nchunks - 1) * pl.boundary_bytes;
+}
+
+size_t bf_butterfly_multiply_saved_bytes(const bf_problem *p)
+{
+    if (check_problem(p, true)) return 0;
+    return saved_bytes(p);
+}
+
+int bf_butterfly_multiply_fw_saving(const bf_problem *p, const void *twiddle, const void *input, const void *bias,
+                                    const int32_t *in_perm, const int32_t *out_index, void *output, void *saved,
+                                    size_t saved_capacity, void *stream_)
+{
+    int rc = check_problem(p, false);
+    if (rc) return rc;
+    if ((rc = check_perms(p, false, in_perm, out_index))) return rc;
+    if ((rc = ensure_attributes())) return rc;
+    const size_t need = saved_bytes(p);
+    if (need == 0) return fail(BF_ERR_INVALID, "this problem has no activations to save: use bf_butterfly_multiply_fw");
+    if (!saved || saved_capacity < need)
+        return fail(BF_ERR_WORKSPACE, "room for %zu bytes of saved activations needed, %zu given", need, saved_capacity);
+    if (!twiddle || !input || !output) return fail(BF_ERR_INVALID, "an operand is NULL");
+    if (((reinterpret_cast<uintptr_t>(saved) | reinterpret_cast<uintptr_t>(twiddle)) & 15) != 0)
+        return fail(BF_ERR_INVALID, "twiddle and the saved area must be 16-byte aligned");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int64_t n = (int64_t)1 << p->log_n;
+    const PassPlan mp = build_passes(p, false);
+    const BwPlan pl = plan_bw(p, false, true);
+    const View in_view = make_view(p->input_stride, std::min(p->input_size, n), in_perm);
+    const View out_view = make_view(p->output_stride, p->output_size, out_index);
+    const View dense = dense_view(p->nstacks, n);
+    char *bounds = static_cast<char *>(saved);
+    auto boundary = [&](int k) { return bounds + (size_t)(k - 1) * pl.boundary_bytes; };
+    const int P = mp.npass;
+    // the passes of the backward plan, each into its own plane: plane k = activation entering pass k
+    for (int k = 0; k + 1 < P; ++k) {
+        rc = multipass_forward(p, mp, twiddle, k == 0 ? input : boundary(k), boundary(k + 1), nullptr,
+                               k == 0 ? in_view : dense, dense, k, k + 1, stream);
+        if (rc) return rc;
+    }
+    bool bias_done = false;
+    rc = multipass_forward(p, mp, twiddle, boundary(P - 1), output, nullptr, dense, out_view, P - 1, P, stream, bias,
+                           &bias_done);
+    if (rc || !bias || bias_done) return rc;
+    return p->dtype == BF_C64 ? launch_bias_add<float2>(p, bias, output, out_view, stream)
+                              : launch_bias_add<float>(p, bias, output, out_view, stream);
+}
+
+size_t bf_butterfly_multiply_bw_saved_workspace_bytes(const bf_problem *p, int with_bias)
+{
+    if (check_problem(p, true)) return 0;
+    const size_t main_bytes = plan_bw(p, false, true).total;
+    return with_bias ? align256(main_bytes) + bias_area_bytes(p) : main_bytes;
+}
+
+int bf_butterfly_multiply_bw_saved(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
+                                   const void *saved, const int32_t *in_perm, const int32_t *out_index,
+                                   void *d_twiddle, void *d_input, void *d_bias, void *workspace,
+                                   size_t workspace_bytes, void *stream)
+{
+    int rc = check_problem(p, true);
+    if (rc) return rc;
+    if (!saved || saved_bytes(p) == 0)
+        return fail(BF_ERR_INVALID, "this problem has no saved activations: use bf_butterfly_multiply_bw");
+    if (d_bias)
+        return bias_backward(p, twiddle, input, grad, d_twiddle, d_input, d_bias, workspace, workspace_bytes, stream,
+                             in_perm, out_index, saved);
+    return backward(p, false, twiddle, nullptr, input, grad, d_twiddle, nullptr, d_input, workspace, workspace_bytes,
+                    stream, nullptr, nullptr, in_perm, out_index, saved);
 }
 
 // One line per launch group of the base-2 schedule, e.g. "low t=0..10 L=10 nb=1 inc=1 chunks=8".

@@ -183,9 +183,11 @@ const int32_t *table_ptr(const Tensor &t, Tensor &keep, const Tensor &like, int6
 }
 
 // Shared body of the forward operators (`bias`, `in_perm`, `out_index` undefined = none).
+// keep (may be NULL): where the call may leave the intermediate activations that a backward in
+// several passes would otherwise recompute; defined on return when it did.
 Tensor multiply_fw_impl(const Tensor &twiddle, const Tensor &input, const Tensor &bias, bool increasing_stride,
                         c10::optional<int64_t> output_size, const char *who, const Tensor &in_perm = Tensor(),
-                        const Tensor &out_index = Tensor())
+                        const Tensor &out_index = Tensor(), Tensor *keep = nullptr)
 {
     CHECK_DEVICE(twiddle); CHECK_DEVICE(input); CHECK_SAME_DEVICE(twiddle, input);
     CHECK_DIM(twiddle, 6); CHECK_DIM(input, 3);
@@ -221,13 +223,29 @@ Tensor multiply_fw_impl(const Tensor &twiddle, const Tensor &input, const Tensor
     if (output_size_val < s.n) output = output.slice(2, 0, output_size_val);
     bf_problem p = make_problem(s, x, increasing_stride, output_size_val, who);
     set_strides(p.output_stride, output);
-    const size_t ws_bytes = bf_butterfly_multiply_fw_workspace_bytes(&p);
-    Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
     Tensor keep_in, keep_out;
     const int32_t *ip = table_ptr(in_perm, keep_in, x, s.n, "in_perm", who);
     const int32_t *oi = table_ptr(out_index, keep_out, x, s.n, "out_index", who);
+    if (ip || oi) TORCH_CHECK(s.input_size <= s.n, who, ": column tables need input_size <= n");
+    if (keep) {
+        // (the backward will make d_input dense over max(input_size, n) columns: same plan)
+        const int64_t dw = std::max(s.input_size, s.n);
+        p.d_input_stride[0] = s.batch > 1 ? s.nstacks * dw : 0;
+        p.d_input_stride[1] = s.nstacks > 1 ? dw : 0;
+        p.d_input_stride[2] = s.input_size > 1 ? 1 : 0;
+        const size_t nsaved = bf_butterfly_multiply_saved_bytes(&p);
+        if (nsaved > 0) {
+            *keep = at::empty({(int64_t)nsaved}, x.options().dtype(at::kByte));
+            check_rc(bf_butterfly_multiply_fw_saving(&p, tw.data_ptr(), x.data_ptr(), b.defined() ? b.data_ptr() : nullptr,
+                                                     ip, oi, output.data_ptr(), keep->data_ptr(), nsaved,
+                                                     current_stream()),
+                     who);
+            return output;
+        }
+    }
+    const size_t ws_bytes = bf_butterfly_multiply_fw_workspace_bytes(&p);
+    Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
     if (ip || oi) {
-        TORCH_CHECK(s.input_size <= s.n, who, ": column tables need input_size <= n");
         check_rc(bf_butterfly_multiply_perm_fw(&p, tw.data_ptr(), x.data_ptr(), ip, oi,
                                                b.defined() ? b.data_ptr() : nullptr, output.data_ptr(),
                                                ws.data_ptr(), ws_bytes, current_stream()),
@@ -283,10 +301,11 @@ Tensor butterfly_bias_grad(const Tensor grad)
 }
 
 // Shared body of the backward operators.
+// kept: what the forward left in its `keep` (undefined: the backward recomputes what it needs)
 std::tuple<Tensor, Tensor, Tensor> multiply_bw_impl(const Tensor &twiddle, const Tensor &input, const Tensor &grad,
                                                     bool increasing_stride, bool with_bias, const char *who,
                                                     const Tensor &in_perm = Tensor(),
-                                                    const Tensor &out_index = Tensor())
+                                                    const Tensor &out_index = Tensor(), const Tensor &kept = Tensor())
 {
     CHECK_DEVICE(twiddle); CHECK_DEVICE(input); CHECK_DEVICE(grad);
     CHECK_SAME_DEVICE(twiddle, input); CHECK_SAME_DEVICE(input, grad);
@@ -325,7 +344,17 @@ std::tuple<Tensor, Tensor, Tensor> multiply_bw_impl(const Tensor &twiddle, const
     Tensor keep_in, keep_out;
     const int32_t *ip = table_ptr(in_perm, keep_in, x, s.n, "in_perm", who);
     const int32_t *oi = table_ptr(out_index, keep_out, x, s.n, "out_index", who);
-    if (ip || oi) {
+    if (kept.defined()) {
+        if (ip || oi) TORCH_CHECK(s.input_size <= s.n, who, ": column tables need input_size <= n");
+        if (with_bias) d_bias = at::empty({s.nstacks, output_size}, g.options());
+        const size_t ws_bytes = bf_butterfly_multiply_bw_saved_workspace_bytes(&p, with_bias ? 1 : 0);
+        Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+        check_rc(bf_butterfly_multiply_bw_saved(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), kept.data_ptr(), ip, oi,
+                                                d_twiddle.data_ptr(), d_input.data_ptr(),
+                                                with_bias ? d_bias.data_ptr() : nullptr, ws.data_ptr(), ws_bytes,
+                                                current_stream()),
+                 who);
+    } else if (ip || oi) {
         TORCH_CHECK(s.input_size <= s.n, who, ": column tables need input_size <= n");
         if (with_bias) d_bias = at::empty({s.nstacks, output_size}, g.options());
         const size_t ws_bytes = with_bias ? bf_butterfly_multiply_bias_bw_workspace_bytes(&p)
@@ -373,52 +402,80 @@ using torch::autograd::variable_list;
 
 class ButterflyMultiply : public torch::autograd::Function<ButterflyMultiply> {
 public:
+    // wants_grad: a gradient will be asked for.  The forward then runs along the backward's pass
+    // plan and keeps the activations between the passes (device tensors whose backward takes
+    // several passes: rows beyond 1024, more than two blocks), which the reference's Function
+    // (csrc/butterfly.cpp:99-118) leaves to its backward to recompute.
     static Tensor forward(AutogradContext *ctx, Tensor twiddle, Tensor input, bool increasing_stride,
-                          c10::optional<int64_t> output_size)
+                          c10::optional<int64_t> output_size, bool wants_grad)
     {
         ctx->saved_data["increasing_stride"] = increasing_stride;
-        ctx->save_for_backward({twiddle, input});
-        return butterfly_multiply_fw(twiddle, input, increasing_stride, output_size);
+        Tensor kept;
+        Tensor out = multiply_fw_impl(twiddle, input, Tensor(), increasing_stride, output_size, "butterfly_multiply",
+                                      Tensor(), Tensor(), wants_grad && input.is_cuda() ? &kept : nullptr);
+        ctx->saved_data["kept"] = kept.defined();
+        if (kept.defined()) ctx->save_for_backward({twiddle, input, kept});
+        else ctx->save_for_backward({twiddle, input});
+        return out;
     }
 
     static variable_list backward(AutogradContext *ctx, variable_list grad_output)
     {
         const auto saved = ctx->get_saved_variables();
         const bool increasing_stride = ctx->saved_data["increasing_stride"].toBool();
-        auto result = butterfly_multiply_bw(saved[0], saved[1], grad_output[0], increasing_stride);
-        return {std::get<0>(result), std::get<1>(result), Tensor(), Tensor()};
+        const Tensor kept = ctx->saved_data["kept"].toBool() ? saved[2] : Tensor();
+        auto result = multiply_bw_impl(saved[0], saved[1], grad_output[0], increasing_stride, false,
+                                       "butterfly_multiply_bw", Tensor(), Tensor(), kept);
+        return {std::get<0>(result), std::get<1>(result), Tensor(), Tensor(), Tensor()};
     }
 };
+
+bool grad_wanted(std::initializer_list<Tensor> ts)
+{
+    if (!at::GradMode::is_enabled()) return false;
+    for (const Tensor &t : ts)
+        if (t.defined() && t.requires_grad()) return true;
+    return false;
+}
 
 Tensor butterfly_multiply(Tensor twiddle, Tensor input, bool increasing_stride,
                           c10::optional<int64_t> output_size)
 {
-    return ButterflyMultiply::apply(twiddle, input, increasing_stride, output_size);
+    return ButterflyMultiply::apply(twiddle, input, increasing_stride, output_size, grad_wanted({twiddle, input}));
 }
 
 class ButterflyMultiplyBias : public torch::autograd::Function<ButterflyMultiplyBias> {
 public:
     static Tensor forward(AutogradContext *ctx, Tensor twiddle, Tensor input, Tensor bias, bool increasing_stride,
-                          c10::optional<int64_t> output_size)
+                          c10::optional<int64_t> output_size, bool wants_grad)
     {
+        TORCH_CHECK(bias.defined(), "butterfly_multiply_bias: bias is undefined");
         ctx->saved_data["increasing_stride"] = increasing_stride;
-        ctx->save_for_backward({twiddle, input});
-        return butterfly_multiply_bias_fw(twiddle, input, bias, increasing_stride, output_size);
+        Tensor kept;
+        Tensor out = multiply_fw_impl(twiddle, input, bias, increasing_stride, output_size, "butterfly_multiply_bias",
+                                      Tensor(), Tensor(), wants_grad && input.is_cuda() ? &kept : nullptr);
+        ctx->saved_data["kept"] = kept.defined();
+        if (kept.defined()) ctx->save_for_backward({twiddle, input, kept});
+        else ctx->save_for_backward({twiddle, input});
+        return out;
     }
 
     static variable_list backward(AutogradContext *ctx, variable_list grad_output)
     {
         const auto saved = ctx->get_saved_variables();
         const bool increasing_stride = ctx->saved_data["increasing_stride"].toBool();
-        auto result = butterfly_multiply_bias_bw(saved[0], saved[1], grad_output[0], increasing_stride);
-        return {std::get<0>(result), std::get<1>(result), std::get<2>(result), Tensor(), Tensor()};
+        const Tensor kept = ctx->saved_data["kept"].toBool() ? saved[2] : Tensor();
+        auto result = multiply_bw_impl(saved[0], saved[1], grad_output[0], increasing_stride, true,
+                                       "butterfly_multiply_bias_bw", Tensor(), Tensor(), kept);
+        return {std::get<0>(result), std::get<1>(result), std::get<2>(result), Tensor(), Tensor(), Tensor()};
     }
 };
 
 Tensor butterfly_multiply_bias(Tensor twiddle, Tensor input, Tensor bias, bool increasing_stride,
                                c10::optional<int64_t> output_size)
 {
-    return ButterflyMultiplyBias::apply(twiddle, input, bias, increasing_stride, output_size);
+    return ButterflyMultiplyBias::apply(twiddle, input, bias, increasing_stride, output_size,
+                                        grad_wanted({twiddle, input, bias}));
 }
 
 // New operators: the multiply between two fixed column permutations, folded into the first
@@ -452,17 +509,23 @@ class ButterflyMultiplyPerm : public torch::autograd::Function<ButterflyMultiply
 public:
     static Tensor forward(AutogradContext *ctx, Tensor twiddle, Tensor input, c10::optional<Tensor> in_perm,
                           c10::optional<Tensor> out_index, c10::optional<Tensor> bias, bool increasing_stride,
-                          c10::optional<int64_t> output_size)
+                          c10::optional<int64_t> output_size, bool wants_grad)
     {
         ctx->saved_data["increasing_stride"] = increasing_stride;
         ctx->saved_data["with_bias"] = bias.has_value();
         ctx->saved_data["has_in"] = in_perm.has_value();
         ctx->saved_data["has_out"] = out_index.has_value();
+        Tensor kept;
+        Tensor out = multiply_fw_impl(twiddle, input, opt(bias), increasing_stride, output_size,
+                                      "butterfly_multiply_perm", opt(in_perm), opt(out_index),
+                                      wants_grad && input.is_cuda() ? &kept : nullptr);
+        ctx->saved_data["kept"] = kept.defined();
         variable_list saved = {twiddle, input};
         if (in_perm.has_value()) saved.push_back(in_perm.value());
         if (out_index.has_value()) saved.push_back(out_index.value());
+        if (kept.defined()) saved.push_back(kept);
         ctx->save_for_backward(saved);
-        return butterfly_multiply_perm_fw(twiddle, input, in_perm, out_index, bias, increasing_stride, output_size);
+        return out;
     }
 
     static variable_list backward(AutogradContext *ctx, variable_list grad_output)
@@ -473,12 +536,12 @@ public:
         size_t next = 2;
         if (has_in) in_perm = saved[next++];
         if (has_out) out_index = saved[next++];
-        auto r = butterfly_multiply_perm_bw(saved[0], saved[1], grad_output[0], in_perm, out_index,
-                                            ctx->saved_data["with_bias"].toBool(),
-                                            ctx->saved_data["increasing_stride"].toBool());
+        const Tensor kept = ctx->saved_data["kept"].toBool() ? saved[next++] : Tensor();
         const bool with_bias = ctx->saved_data["with_bias"].toBool();
+        auto r = multiply_bw_impl(saved[0], saved[1], grad_output[0], ctx->saved_data["increasing_stride"].toBool(),
+                                  with_bias, "butterfly_multiply_perm_bw", opt(in_perm), opt(out_index), kept);
         return {std::get<0>(r), std::get<1>(r), Tensor(), Tensor(), with_bias ? std::get<2>(r) : Tensor(), Tensor(),
-                Tensor()};
+                Tensor(), Tensor()};
     }
 };
 
@@ -486,7 +549,8 @@ Tensor butterfly_multiply_perm(Tensor twiddle, Tensor input, c10::optional<Tenso
                                c10::optional<Tensor> out_index, c10::optional<Tensor> bias, bool increasing_stride,
                                c10::optional<int64_t> output_size)
 {
-    return ButterflyMultiplyPerm::apply(twiddle, input, in_perm, out_index, bias, increasing_stride, output_size);
+    return ButterflyMultiplyPerm::apply(twiddle, input, in_perm, out_index, bias, increasing_stride, output_size,
+                                        grad_wanted({twiddle, input, opt(bias)}));
 }
 
 // ---- diagonals folded into the factors ------------------------------------------------------

@@ -140,6 +140,31 @@ int bf_butterfly_multiply_perm_bw(const bf_problem *p, const void *twiddle, cons
                                   void *d_bias, void *workspace, size_t workspace_bytes,
                                   void *stream);
 
+/* Forward and backward of a pair that share their intermediate activations.  A backward call
+ * that runs in several passes (rows longer than 1024, more than two blocks) needs the activation
+ * entering every pass after the first, and bf_butterfly_multiply_bw recomputes them with forward
+ * launches of its own.  bf_butterfly_multiply_fw_saving runs the forward along the backward's
+ * pass plan and leaves those activations in `saved` (bf_butterfly_multiply_saved_bytes bytes:
+ * one dense (B, S, n) plane per pass after the first; 0 = single pass, nothing to save, use the
+ * plain calls); bf_butterfly_multiply_bw_saved reads them instead of recomputing.  `bias` as in
+ * bf_butterfly_multiply_bias_fw, in_perm / out_index as in bf_butterfly_multiply_perm_fw / _bw
+ * (each may be NULL).  What the reference's autograd Function would
+ * keep between its forward and backward (csrc/butterfly.cpp:99-118 saves twiddle and input only
+ * and its backward recomputes everything, csrc/cuda/butterfly_cuda.cu:534-646).             */
+size_t bf_butterfly_multiply_saved_bytes(const bf_problem *p);
+int bf_butterfly_multiply_fw_saving(const bf_problem *p, const void *twiddle, const void *input,
+                                    const void *bias, const int32_t *in_perm,
+                                    const int32_t *out_index, void *output, void *saved,
+                                    size_t saved_capacity, void *stream);
+size_t bf_butterfly_multiply_bw_saved_workspace_bytes(const bf_problem *p, int with_bias);
+/* d_bias (S, O) may be NULL; when given it receives the column sums of grad as in
+ * bf_butterfly_multiply_bias_bw (size the workspace with with_bias != 0).                   */
+int bf_butterfly_multiply_bw_saved(const bf_problem *p, const void *twiddle, const void *input,
+                                   const void *grad, const void *saved, const int32_t *in_perm,
+                                   const int32_t *out_index, void *d_twiddle, void *d_input,
+                                   void *d_bias, void *workspace, size_t workspace_bytes,
+                                   void *stream);
+
 /* Diagnostic, host only (no device call): how the base-2 forward (backward != 0: backward)
  * call for this problem is cut into launches, one text line per pass in order --
  *   "low t=A..B L=.. nb=.. inc=.. chunks=.."   stages A..B-1 on bits 0..9, 1024-element chunks

@@ -851,3 +851,115 @@ def test_misaligned_twiddle_is_rejected():
     import butterfly_amd  # noqa: F401
     y = torch.ops.torch_butterfly.butterfly_multiply_fw(tw, x, True, None)
     assert rel_err(y.cpu().numpy(), oracle.butterfly_fw(tw.cpu().numpy(), x.cpu().numpy(), True)) < FW_TOL
+
+
+SAVING_CASES = [
+    # dtype, B, S, L, nb, I, O, inc -- backward plans of several passes: the forward keeps what they need
+    (np.float32, 40, 2, 9, 3, None, None, True),
+    (np.float32, 33, 1, 10, 5, 1000, 900, False),
+    (np.float32, 21, 2, 11, 1, None, None, False),
+    (np.float32, 21, 1, 11, 2, 2000, 1500, True),
+    (np.float32, 300, 1, 12, 2, None, None, True),
+    (np.float32, 1500, 1, 12, 1, None, None, False),
+    (np.float32, 10, 2, 12, 3, 2 * 4096 + 7, 4091, False),
+    (np.float32, 3, 1, 14, 1, None, None, True),
+    (np.complex64, 40, 1, 9, 2, None, None, False),
+    (np.complex64, 10, 2, 12, 3, None, None, True),
+    (np.complex64, 600, 1, 12, 1, 4000, None, True),
+]
+
+
+@pytest.mark.parametrize("case", SAVING_CASES, ids=lambda c: f"{np.dtype(c[0]).name}-B{c[1]}-S{c[2]}-L{c[3]}-nb{c[4]}-I{c[5]}-O{c[6]}-inc{int(c[7])}")
+def test_forward_that_saves_for_the_backward(case):
+    """bf_butterfly_multiply_fw_saving + bf_butterfly_multiply_bw_saved (the forward runs along the
+    backward's pass plan and keeps the activations between the passes; the backward reads them
+    instead of recomputing): all results against the oracle, with and without the bias."""
+    from butterfly_amd import _capi
+    dtype, B, S, L, nb, I, O, inc = case
+    say("saving case", case)
+    rng = np.random.default_rng(7000 + L * 17 + nb)
+    tw, x, g = make_case(rng, dtype, B, S, L, nb, I, O)
+    y_ref = oracle.butterfly_fw(tw, x, inc, O)
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+    r = _capi.multiply_fw_bw_saving(dev(tw), dev(x), dev(g), inc, O)
+    assert r is not None
+    y, dtw, dx, _ = r
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+    bias = randn(rng, (S, g.shape[2]), dtype)
+    y, dtw, dx, db = _capi.multiply_fw_bw_saving(dev(tw), dev(x), dev(g), inc, O, bias=dev(bias))
+    assert rel_err(y.cpu().numpy(), y_ref + bias[None]) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+    assert rel_err(db.cpu().numpy(), g.sum(0)) < BW_TOL
+
+
+def test_single_pass_problems_save_nothing():
+    from butterfly_amd import _capi
+    rng = np.random.default_rng(7100)
+    tw, x, g = make_case(rng, np.float32, 50, 1, 10, 2)
+    assert _capi.multiply_fw_bw_saving(dev(tw), dev(x), dev(g), False) is None
+
+
+@pytest.mark.parametrize("dtype,L,nb", [(np.float32, 12, 2), (np.complex64, 12, 1), (np.float32, 10, 3)],
+                         ids=["f32-4096-nb2", "c64-4096", "f32-1024-nb3"])
+def test_autograd_operators_keep_activations_between_passes(dtype, L, nb):
+    """torch.ops.torch_butterfly.butterfly_multiply / _bias under autograd (kept activations) against
+    the oracle and against the operators called one by one (which recompute)."""
+    import butterfly_amd  # noqa: F401
+    ops = torch.ops.torch_butterfly
+    rng = np.random.default_rng(7200 + L + nb)
+    B, S, I, O = 70, 2, (1 << L) - 5, (1 << L) - 9
+    tw, x, g = make_case(rng, dtype, B, S, L, nb, I, O)
+    say("autograd keep", np.dtype(dtype).name, L, nb)
+    y_ref = oracle.butterfly_fw(tw, x, True, O)
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, True)
+    twd, xd = dev(tw).requires_grad_(), dev(x).requires_grad_()
+    y = ops.butterfly_multiply(twd, xd, True, O)
+    assert y.shape == (B, S, O) and y.stride() == (S << L, 1 << L, 1)
+    dtw, dx = torch.autograd.grad(y, (twd, xd), dev(g))
+    assert rel_err(y.detach().cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+    dtw2, dx2 = ops.butterfly_multiply_bw(dev(tw), dev(x), dev(g), True)
+    assert rel_err(dx.cpu().numpy(), dx2.cpu().numpy()) < 1e-6 and rel_err(dtw.cpu().numpy(), dtw2.cpu().numpy()) < 1e-6
+    bias = randn(rng, (S, O), dtype)
+    bd = dev(bias).requires_grad_()
+    yb = ops.butterfly_multiply_bias(twd, xd, bd, True, O)
+    dtw, dx, db = torch.autograd.grad(yb, (twd, xd, bd), dev(g))
+    assert rel_err(yb.detach().cpu().numpy(), y_ref + bias[None]) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+    assert rel_err(db.cpu().numpy(), g.sum(0)) < BW_TOL
+    # no gradient wanted: nothing is kept, the plain forward plan runs
+    with torch.no_grad():
+        y0 = ops.butterfly_multiply(dev(tw), dev(x), True, O)
+    assert rel_err(y0.cpu().numpy(), y_ref) < FW_TOL
+
+
+@pytest.mark.parametrize("dtype,L,nb", [(np.complex64, 12, 1), (np.float32, 11, 2)], ids=["c64-4096", "f32-2048-nb2"])
+def test_saving_forward_between_column_permutations(dtype, L, nb):
+    """The pair that shares its activations with a permutation in front and behind (what
+    special.fft(4096) under autograd runs): against the oracle between explicit gathers."""
+    from butterfly_amd import _capi
+    n = 1 << L
+    rng = np.random.default_rng(7300 + L)
+    B, S = 90, 1
+    tw, x, g = make_case(rng, dtype, B, S, L, nb)
+    in_perm = rng.permutation(n).astype(np.int32)
+    out_index = rng.permutation(n).astype(np.int32)
+    say("saving perm", np.dtype(dtype).name, L, nb)
+    u = x[:, :, in_perm]
+    y_mid = oracle.butterfly_fw(tw, u, False)
+    y_ref = np.empty_like(y_mid)
+    y_ref[:, :, out_index] = y_mid
+    dtw_ref, du_ref = oracle.butterfly_bw(tw, u, g[:, :, out_index], False)
+    dx_ref = np.zeros_like(x)
+    dx_ref[:, :, in_perm] = du_ref
+    y, dtw, dx, _ = _capi.multiply_fw_bw_saving(dev(tw), dev(x), dev(g), False, in_perm=dev(in_perm),
+                                               out_index=dev(out_index))
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
