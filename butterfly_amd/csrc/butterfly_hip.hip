@@ -20,6 +20,7 @@
 #include "wide.hpp"
 #include "fast4.hpp"
 #include "fast4g.hpp"
+#include "stage.hpp"
 #include "bias.hpp"
 
 namespace {
@@ -643,6 +644,7 @@ void launch_fast4g_t(bool backward, const Fast4GArgs &a, dim3 grid, hipStream_t 
     else hipLaunchKernelGGL((fast4g_fw_kernel<T, L, INC, R>), grid, dim3(kFastThreads), 0, stream, a);
 }
 
+// (float L = 10 only runs on the 1024-element chunks of longer rows: whole rows of 1024 take fast4.hpp)
 int launch_fast4g(bool cplx, int L, bool inc, bool backward, const Fast4GArgs &a, dim3 grid, hipStream_t stream)
 {
 #define BF_F4G(LL)                                                                              \
@@ -658,7 +660,7 @@ int launch_fast4g(bool cplx, int L, bool inc, bool backward, const Fast4GArgs &a
         }
     } else {
         switch (L * 2 + (inc ? 1 : 0)) {
-            BF_F4G(3) BF_F4G(5) BF_F4G(7) BF_F4G(9)
+            BF_F4G(3) BF_F4G(5) BF_F4G(7) BF_F4G(9) BF_F4G(10)
             default: return fail(BF_ERR_UNSUPPORTED, "no base-4 kernel for this shape");
         }
     }
@@ -679,6 +681,8 @@ Fast4GArgs fast4g_block_args(const bf_problem *p, const void *tw4, const void *t
     a.tw4_stack_stride = p->nblocks * (L / 2) * (n / 4) * 16;
     a.tw2 = (L & 1) ? static_cast<const char *>(tw2) + (size_t)k * (n / 2) * 4 * e : nullptr;
     a.tw2_stack_stride = p->nblocks * (L & 1) * (n / 2) * 4;
+    a.tw4_stage_stride = (n / 4) * 16;
+    a.n_full = n;
     a.batch = p->batch;
     return a;
 }
@@ -720,6 +724,196 @@ int fast4_forward(const bf_problem *p, const void *tw4, const void *tw2, const v
         a.groups_per_wg = g.groups_per_wg;
         const bool inc = (p->increasing_stride != 0) != ((k & 1) != 0);
         const int rc = launch_fast4(L, inc, false, a, dim3((unsigned)g.nwg, (unsigned)p->nstacks), stream);
+        if (rc) return rc;
+    }
+    return BF_OK;
+}
+
+// ---- base-4 rows beyond the reach of one workgroup's registers ------------------------------------
+//
+// A block of a long base-4 row is cut into passes, one launch each:
+//   * a CHUNK pass: the general base-4 kernels (fast4g.hpp) on independent chunks of 2^LC elements
+//     for the stages that stay inside a chunk -- with increasing stride the first LC / 2 radix-4
+//     stages (LC = 10 float, 8 complex64); with decreasing stride the last ones and, for odd
+//     log_n, the closing 2x2 stage on bit 0 (LC = 9 / 7 then, so that the bit pairs line up);
+//   * one STAGE pass (stage.hpp) per remaining stage: the radix-4 stages on the bits above the
+//     chunk and, with increasing stride and odd log_n, the closing 2x2 stage on the top bit.
+struct Pass4 {
+    bool chunk;
+    int t0, t1;        // global stage range [t0, t1)
+    int LC;            // chunk pass: log2 of the chunk length
+    bool inc;
+    int block, idx0;   // chunk pass: block and index (within the block) of its first radix-4 stage
+};
+
+struct Plan4Long {
+    bool ok = false;
+    int npass = 0;
+    Pass4 pass[kMaxPasses];
+};
+
+Plan4Long plan4_long(const bf_problem *p, bool base4)
+{
+    Plan4Long pl;
+    {
+        // the chunk kernels address their operands with 32-bit offsets from a workgroup's first row
+        const int64_t n = (int64_t)1 << p->log_n;
+        const size_t e = elem_bytes(p->dtype);
+        const int64_t rows = (p->batch + kFast4FwRows + 2) * 8;   // (any workgroup's share, with margin)
+        const int64_t dense[3] = {p->nstacks * n, n, 1};
+        if (!span_ok(p->input_stride, rows, n, e) || !span_ok(p->output_stride, rows, n, e) ||
+            !span_ok(dense, rows, n, e) || !span_ok(p->d_input_stride, rows, n, e))
+            return pl;
+    }
+    const int L = (int)p->log_n;
+    const int reach = p->dtype == BF_C64 ? 8 : 10;
+    if (!base4 || L <= reach || L > kMaxLogN || p->nblocks < 1 || p->batch <= 0 || p->nstacks <= 0 ||
+        p->input_size <= 0 || p->output_size <= 0)
+        return pl;
+    const int per = L / 2 + (L & 1), l4 = L / 2;
+    for (int k = 0; k < p->nblocks; ++k) {
+        const bool inc = (p->increasing_stride != 0) != ((k & 1) != 0);
+        const int LC = (inc || !(L & 1)) ? reach : reach - 1;
+        const int nlow = LC / 2, nhigh = l4 - nlow;
+        auto add = [&](bool chunk, int t0, int t1, int idx0) {
+            if (pl.npass == kMaxPasses) return false;
+            Pass4 &q = pl.pass[pl.npass++];
+            q.chunk = chunk;
+            q.t0 = t0;
+            q.t1 = t1;
+            q.LC = LC;
+            q.inc = inc;
+            q.block = k;
+            q.idx0 = idx0;
+            return true;
+        };
+        if (inc) {
+            if (!add(true, k * per, k * per + nlow, 0)) return pl;
+            for (int j = nlow; j < per; ++j)
+                if (!add(false, k * per + j, k * per + j + 1, j)) return pl;
+        } else {
+            for (int j = 0; j < nhigh; ++j)
+                if (!add(false, k * per + j, k * per + j + 1, j)) return pl;
+            if (!add(true, k * per + nhigh, k * per + per, nhigh)) return pl;
+        }
+    }
+    pl.ok = true;
+    return pl;
+}
+
+struct StageGrid {
+    int64_t tiles, nparts, rows_per_wg;
+};
+
+StageGrid stage_grid(const bf_problem *p, int radix)
+{
+    const int64_t n = (int64_t)1 << p->log_n;
+    StageGrid g;
+    g.tiles = (n / radix + kStageThreads - 1) / kStageThreads;
+    const int64_t want = std::max<int64_t>(1, (int64_t)num_cu() * 8 / (g.tiles * p->nstacks));
+    g.nparts = std::min<int64_t>(std::min<int64_t>(want, p->batch), 65535);
+    g.rows_per_wg = (p->batch + g.nparts - 1) / g.nparts;
+    g.nparts = (p->batch + g.rows_per_wg - 1) / g.rows_per_wg;
+    return g;
+}
+
+FastGrid chunk4_grid(const bf_problem *p, const Pass4 &q, bool backward)
+{
+    const int64_t chunks = (int64_t)1 << (p->log_n - q.LC);
+    return fast_grid(p->batch, q.LC, p->nstacks * chunks, backward ? 1 : fast4_fw_rows(p), 1);
+}
+
+// partial slices (of 4 n scalars per stage) the backward of this pass writes
+int64_t pass4_slices(const bf_problem *p, const Pass4 &q)
+{
+    if (q.chunk) return chunk4_grid(p, q, true).nwg * (q.t1 - q.t0);
+    return stage_grid(p, stage_info(make_schedule(p, true), q.t0).radix4 ? 4 : 2).nparts;
+}
+
+// One pass forward (backward == false: x_in -> x_out) or backward (x_in, g_out -> g_in and the
+// pass's partial slices; *nparts receives their number per stage).
+int run_pass4(const bf_problem *p, const Schedule &sc, const Pass4 &q, bool backward, const void *tw2, const void *tw4,
+              const void *x_in, const View &x_view, void *x_out, const View &xo_view, const void *g_out,
+              const View &g_view, void *g_in, const View &gi_view, void *partial, int64_t *nparts, hipStream_t stream)
+{
+    const int64_t n = (int64_t)1 << p->log_n;
+    const int L = (int)p->log_n;
+    const size_t e = elem_bytes(p->dtype);
+    const bool cplx = p->dtype == BF_C64;
+    if (q.chunk) {
+        const FastGrid g = chunk4_grid(p, q, backward);
+        Fast4GArgs a = {};
+        a.tw4 = static_cast<const char *>(tw4) + ((size_t)q.block * (L / 2) + q.idx0) * (n / 4) * 16 * e;
+        a.tw4_stack_stride = sc.tw4_stack_stride;
+        a.tw4_stage_stride = (n / 4) * 16;
+        a.tw2 = (L & 1) ? static_cast<const char *>(tw2) + (size_t)q.block * (n / 2) * 4 * e : nullptr;
+        a.tw2_stack_stride = sc.tw2_stack_stride;
+        a.n_full = n;
+        a.x_in = x_in;
+        a.x_view = x_view;
+        a.x_out = x_out;
+        a.xo_view = xo_view;
+        a.g_out = g_out;
+        a.g_view = g_view;
+        a.g_in = g_in;
+        a.gi_view = gi_view;
+        a.partial = partial;
+        a.batch = p->batch;
+        a.ngroups = g.ngroups;
+        a.groups_per_wg = g.groups_per_wg;
+        if (nparts) *nparts = g.nwg;
+        return launch_fast4g(cplx, q.LC, q.inc, backward, a,
+                             dim3((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)(n >> q.LC)), stream);
+    }
+    const StageInfo si = stage_info(sc, q.t0);
+    const int radix = si.radix4 ? 4 : 2;
+    const StageGrid g = stage_grid(p, radix);
+    StageArgs a = {};
+    a.tw = static_cast<const char *>(si.radix4 ? tw4 : tw2) + (size_t)si.tw_off * e;
+    a.tw_stack_stride = si.radix4 ? sc.tw4_stack_stride : sc.tw2_stack_stride;
+    a.log_stride = si.log_stride;
+    a.n = n;
+    a.x_in = x_in;
+    a.x_view = x_view;
+    a.x_out = x_out;
+    a.xo_view = xo_view;
+    a.g_out = g_out;
+    a.g_view = g_view;
+    a.g_in = g_in;
+    a.gi_view = gi_view;
+    a.partial = partial;
+    a.slot = 4 * n;
+    a.batch = p->batch;
+    a.rows_per_wg = g.rows_per_wg;
+    if (nparts) *nparts = g.nparts;
+    const dim3 grid((unsigned)g.nparts, (unsigned)p->nstacks, (unsigned)g.tiles), block(kStageThreads);
+    if (!backward) {
+        if (cplx && si.radix4) hipLaunchKernelGGL((stage_fw_kernel<float2, 4>), grid, block, 0, stream, a);
+        else if (cplx) hipLaunchKernelGGL((stage_fw_kernel<float2, 2>), grid, block, 0, stream, a);
+        else if (si.radix4) hipLaunchKernelGGL((stage_fw_kernel<float, 4>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((stage_fw_kernel<float, 2>), grid, block, 0, stream, a);
+    } else {
+        if (cplx && si.radix4) hipLaunchKernelGGL((stage_bw_kernel<float2, 4>), grid, block, 0, stream, a);
+        else if (cplx) hipLaunchKernelGGL((stage_bw_kernel<float2, 2>), grid, block, 0, stream, a);
+        else if (si.radix4) hipLaunchKernelGGL((stage_bw_kernel<float, 4>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((stage_bw_kernel<float, 2>), grid, block, 0, stream, a);
+    }
+    BF_HIP_CHECK(hipGetLastError());
+    return BF_OK;
+}
+
+// passes [first, last) forward; `scratch` holds the activation between passes (in place)
+int long4_forward(const bf_problem *p, const Schedule &sc, const Plan4Long &pl, const void *tw2, const void *tw4,
+                  const void *input, void *output, void *scratch, const View &in_view, const View &out_view,
+                  int first, int last, hipStream_t stream)
+{
+    const int64_t n = (int64_t)1 << p->log_n;
+    const View dense = dense_view(p->nstacks, n);
+    for (int k = first; k < last; ++k) {
+        const int rc = run_pass4(p, sc, pl.pass[k], false, tw2, tw4, k == first ? input : scratch,
+                                 k == first ? in_view : dense, k == last - 1 ? output : scratch,
+                                 k == last - 1 ? out_view : dense, nullptr, dense, nullptr, dense, nullptr, nullptr,
+                                 stream);
         if (rc) return rc;
     }
     return BF_OK;
@@ -771,6 +965,9 @@ size_t forward_workspace(const bf_problem *p, bool base4)
         const int64_t n4 = (int64_t)1 << p->log_n;
         return p->nblocks > 1 ? align256((size_t)p->batch * p->nstacks * n4 * elem_bytes(p->dtype)) : 0;
     }
+    const Plan4Long lp = plan4_long(p, base4);
+    if (lp.ok)
+        return lp.npass > 1 ? align256(((size_t)p->batch * p->nstacks << p->log_n) * elem_bytes(p->dtype)) : 0;
     const PassPlan mp = build_passes(p, base4, true);
     if (!mp.ok || mp.npass <= 1 || !passes_addressable(p, mp, false)) return 0;
     const int64_t n = (int64_t)1 << p->log_n;
@@ -837,6 +1034,16 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
         if (need > 0 && (!workspace || workspace_bytes < need))
             return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
         rc = fast4_forward(p, tw4, tw2, input, output, workspace, in_view, out_view, 0, (int)p->nblocks, stream);
+        if (rc || !bias) return rc;
+        return p->dtype == BF_C64 ? launch_bias_add<float2>(p, bias, output, out_view, stream)
+                                  : launch_bias_add<float>(p, bias, output, out_view, stream);
+    }
+    const Plan4Long lp = plan4_long(p, base4);
+    if (lp.ok) {
+        const size_t need = forward_workspace(p, base4);
+        if (need > 0 && (!workspace || workspace_bytes < need))
+            return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        rc = long4_forward(p, sc, lp, tw2, tw4, input, output, workspace, in_view, out_view, 0, lp.npass, stream);
         if (rc || !bias) return rc;
         return p->dtype == BF_C64 ? launch_bias_add<float2>(p, bias, output, out_view, stream)
                                   : launch_bias_add<float>(p, bias, output, out_view, stream);
@@ -918,6 +1125,7 @@ struct BwPlan {
     bool fits;
     bool fast;          // register-resident pass plan
     bool fast4;         // base-4 register-resident kernels, one launch per block
+    bool long4;         // base-4 rows longer than that: chunk and stage passes
 };
 
 // saved_boundaries: the activations entering every pass after the first come from the caller
@@ -944,6 +1152,25 @@ BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false)
         off += p->nblocks > 1 ? pl.boundary_bytes : 0;
         pl.off_partials = off;
         off += align256((size_t)pl.nparts * p->nstacks * sc.per * pl.slot * e);
+        pl.total = off;
+        return pl;
+    }
+    const Plan4Long lp = plan4_long(p, base4);
+    if (lp.ok) {
+        pl.fits = true;
+        pl.long4 = true;
+        pl.nchunks = lp.npass;
+        pl.slot = 4 * n;
+        pl.boundary_bytes = align256((size_t)p->batch * p->nstacks * row_bytes);
+        int64_t slices = 1;
+        for (int k = 0; k < lp.npass; ++k) slices = std::max(slices, pass4_slices(p, lp.pass[k]));
+        size_t off = 0;
+        pl.off_boundaries = off;
+        off += lp.npass > 1 ? (size_t)(lp.npass - 1) * pl.boundary_bytes : 0;
+        pl.off_gbuf = off;
+        off += lp.npass > 1 ? pl.boundary_bytes : 0;
+        pl.off_partials = off;
+        off += align256((size_t)slices * p->nstacks * pl.slot * e);
         pl.total = off;
         return pl;
     }
@@ -1131,6 +1358,40 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
             if (rc) return rc;
             rc = launch_reduce(p, sc, k * per, (k + 1) * per, g.nwg, ws + pl.off_partials, pl.slot, d_tw2, d_tw4,
                                stream);
+            if (rc) return rc;
+        }
+        if (p->input_size > n) {
+            View tail = di_view;
+            tail.width = p->input_size - n;
+            View none = tail;
+            none.width = 0;
+            char *base = static_cast<char *>(d_input) + (size_t)n * p->d_input_stride[2] * e_bytes;
+            rc = launch_copy_pad(p, base, none, base, tail, stream);
+            if (rc) return rc;
+        }
+        return BF_OK;
+    }
+
+    if (pl.long4) {
+        const Plan4Long lp = plan4_long(p, base4);
+        const int P = lp.npass;
+        auto boundary = [&](int k) { return ws + pl.off_boundaries + (size_t)(k - 1) * pl.boundary_bytes; };
+        // forward replay: boundary k = activation entering pass k (k >= 1)
+        for (int k = 0; k + 1 < P; ++k) {
+            rc = long4_forward(p, sc, lp, tw2, tw4, k == 0 ? input : boundary(k), boundary(k + 1), nullptr,
+                               k == 0 ? x_view : dense, dense, k, k + 1, stream);
+            if (rc) return rc;
+        }
+        const View dn_view = make_view(p->d_input_stride, std::min(p->input_size, n), in_perm);
+        for (int k = P - 1; k >= 0; --k) {
+            const Pass4 &q = lp.pass[k];
+            int64_t nparts = 0;
+            rc = run_pass4(p, sc, q, true, tw2, tw4, k == 0 ? input : boundary(k), k == 0 ? x_view : dense, nullptr,
+                           dense, k == P - 1 ? grad : ws + pl.off_gbuf, k == P - 1 ? g_view : dense,
+                           k == 0 ? d_input : ws + pl.off_gbuf, k == 0 ? dn_view : dense, ws + pl.off_partials, &nparts,
+                           stream);
+            if (rc) return rc;
+            rc = launch_reduce(p, sc, q.t0, q.t1, nparts, ws + pl.off_partials, pl.slot, d_tw2, d_tw4, stream);
             if (rc) return rc;
         }
         if (p->input_size > n) {

@@ -46,11 +46,16 @@ struct Plan4G {
     static constexpr int kind(int bit) { return bit >= 6 ? bit - 6 : bit; }
 };
 
+// Rows longer than 2^L run these kernels on their 2^L-element chunks (blockIdx.z) for the stages
+// that stay inside a chunk: chunk c uses the factor quads (pairs) c * 2^L / 4 (/ 2) onward of
+// every stage, and its sums land at the same place in the partial slice.
 struct Fast4GArgs {
-    const void *tw4;           // radix-4 factors of this block, stack 0: (L/2, n/4, 4, 4)
+    const void *tw4;           // radix-4 factors of the first stage run here, stack 0: (stages, n_full/4, 4, 4)
     int64_t tw4_stack_stride;  // scalars
-    const void *tw2;           // the block's 2x2 factors, stack 0: (n/2, 2, 2); odd L only
+    int64_t tw4_stage_stride;  // scalars between consecutive stages: (n_full / 4) * 16
+    const void *tw2;           // the block's 2x2 factors, stack 0: (n_full/2, 2, 2); odd L only
     int64_t tw2_stack_stride;
+    int64_t n_full;            // length of the whole row (2^L when the row is one chunk)
     const void *x_in;
     View x_view;
     void *x_out;               // forward output
@@ -73,17 +78,17 @@ struct Factors4G {
     T colm[WITH_COLUMN ? NS4 : 1][4];      // colm[s][m] = T[r ^ m][r]
     T ta, tb, tc;                          // 2x2 stage: T[r][r], T[r][1 - r], T[1 - r][r]
 
-    __device__ __forceinline__ void load(const Fast4GArgs &a, int stack, const FastCoords &c)
+    __device__ __forceinline__ void load(const Fast4GArgs &a, int stack, int chunk, const FastCoords &c)
     {
         constexpr int n = 1 << L;
-        const T *tw4 = reinterpret_cast<const T *>(a.tw4) + stack * a.tw4_stack_stride;
+        const T *tw4 = reinterpret_cast<const T *>(a.tw4) + stack * a.tw4_stack_stride + (int64_t)chunk * (n / 4) * 16;
         static_for<0, NS4>([&](auto S) {
             constexpr int s = S;
             constexpr int b = P::lo(s);
             const int e = P::layout(s) ? c.eB : c.eA;
             const int r = (e >> b) & 3;
             const int q = ((e >> (b + 2)) << b) | (e & ((1 << b) - 1));
-            const T *F = tw4 + ((int64_t)s * (n / 4) + q) * 16;
+            const T *F = tw4 + (int64_t)s * a.tw4_stage_stride + q * 16;
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
                 row[s][m] = F[r * 4 + (r ^ m)];
@@ -96,7 +101,8 @@ struct Factors4G {
             const int e = P::layout(NS4) ? c.eB : c.eA;
             const int r = (e >> b) & 1;
             const int i = ((e >> (b + 1)) << b) | (e & ((1 << b) - 1));
-            const T *F = reinterpret_cast<const T *>(a.tw2) + stack * a.tw2_stack_stride + (int64_t)i * 4;
+            const T *F = reinterpret_cast<const T *>(a.tw2) + stack * a.tw2_stack_stride +
+                         ((int64_t)chunk * (n / 2) + i) * 4;
             ta = F[3 * r];
             tb = F[r + 1];
             tc = F[2 - r];
@@ -122,10 +128,12 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_fw_kernel(Fast4GArgs a)
     __shared__ T lds[P::NSWAP > 0 ? 2 * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
+    const int chunk = blockIdx.z;
     const FastCoords c = fast_coords<L>(t);
+    const int col = (chunk << L) + c.eA;   // column of this thread's element in the whole row
 
     Factors4G<T, L, INC, false> f;
-    f.load(a, stack, c);
+    f.load(a, stack, chunk, c);
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
@@ -137,7 +145,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_fw_kernel(Fast4GArgs a)
     const __amdgpu_buffer_rsrc_t out_rs =
         make_rsrc(reinterpret_cast<T *>(a.x_out) + g0 * SLOTS * a.xo_view.sb + stack * a.xo_view.ss);
     const int in_row = (int)(a.x_view.sb * EB), out_row = (int)(a.xo_view.sb * EB);
-    const int64_t in_col = view_col(a.x_view, c.eA), out_col = view_col(a.xo_view, c.eA);
+    const int64_t in_col = view_col(a.x_view, col), out_col = view_col(a.xo_view, col);
     const int in_thr = in_col >= 0 ? c.slot * in_row + (int)(in_col * a.x_view.se * EB) : kOob;
     const int out_thr = out_col >= 0 ? c.slot * out_row + (int)(out_col * a.xo_view.se * EB) : kOob;
 
@@ -214,10 +222,12 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_bw_kernel(Fast4GArgs a)
     __shared__ T lds[kLdsWords];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
+    const int chunk = blockIdx.z;
     const FastCoords c = fast_coords<L>(t);
+    const int col = (chunk << L) + c.eA;   // column of this thread's element in the whole row
 
     Factors4G<T, L, INC, true> f;
-    f.load(a, stack, c);
+    f.load(a, stack, chunk, c);
     T acc[NS4][4];   // acc[s][m] = dT[r ^ m][r]
     static_for<0, NS4>([&](auto S) {
 #pragma unroll
@@ -237,7 +247,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_bw_kernel(Fast4GArgs a)
     const __amdgpu_buffer_rsrc_t gi_rs =
         make_rsrc(reinterpret_cast<T *>(a.g_in) + g0 * SLOTS * a.gi_view.sb + stack * a.gi_view.ss);
     const int x_row = (int)(a.x_view.sb * EB), g_row = (int)(a.g_view.sb * EB), gi_row = (int)(a.gi_view.sb * EB);
-    const int64_t x_col = view_col(a.x_view, c.eA), g_col = view_col(a.g_view, c.eA), gi_col = view_col(a.gi_view, c.eA);
+    const int64_t x_col = view_col(a.x_view, col), g_col = view_col(a.g_view, col), gi_col = view_col(a.gi_view, col);
     const int x_thr = x_col >= 0 ? c.slot * x_row + (int)(x_col * a.x_view.se * EB) : kOob;
     const int g_thr = g_col >= 0 ? c.slot * g_row + (int)(g_col * a.g_view.se * EB) : kOob;
     const int gi_thr = gi_col >= 0 ? c.slot * gi_row + (int)(gi_col * a.gi_view.se * EB) : kOob;
@@ -326,7 +336,8 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_bw_kernel(Fast4GArgs a)
     int t2 = t;
     asm volatile("" : "+v"(t2));   // (recompute the coordinates instead of keeping them alive)
     const FastCoords c2 = fast_coords<L>(t2);
-    T *part = reinterpret_cast<T *>(a.partial) + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * (4 * n);
+    const int64_t slot = 4 * a.n_full;   // scalars per stage in a partial slice
+    T *part = reinterpret_cast<T *>(a.partial) + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * slot;
     static_for<0, NS>([&](auto S) {
         constexpr int s = S;
         constexpr int b = P::lo(s);
@@ -353,7 +364,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_bw_kernel(Fast4GArgs a)
                 return i * 4 + (m == 0 ? 3 * r : 2 - r);
             }
         };
-        T *d = part + (int64_t)s * (4 * n);
+        T *d = part + (int64_t)s * slot + (s < NS4 ? (int64_t)chunk * (n / 4) * 16 : (int64_t)chunk * (n / 2) * 4);
         if constexpr (SLOTS == 1) {
 #pragma unroll
             for (int m = 0; m < M; ++m) d[dest(e, m)] = vals[m];

@@ -963,3 +963,45 @@ def test_saving_forward_between_column_permutations(dtype, L, nb):
     assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
     assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
     assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
+LONG_BASE4_CASES = [
+    # dtype, B, S, L, nb, I, O, inc -- base-4 rows beyond one workgroup's registers: chunk + stage passes
+    (np.float32, 37, 2, 11, 1, None, None, True),
+    (np.float32, 37, 2, 11, 1, None, None, False),
+    (np.float32, 300, 1, 12, 2, None, None, True),
+    (np.float32, 300, 1, 12, 2, 4000, 4090, False),
+    (np.float32, 21, 1, 13, 3, None, None, True),
+    (np.float32, 21, 2, 13, 1, 2 * 8192 + 3, 8000, False),
+    (np.float32, 9, 1, 14, 2, None, None, False),
+    (np.float32, 2100, 1, 12, 1, None, None, True),
+    (np.complex64, 41, 2, 9, 2, None, None, True),
+    (np.complex64, 41, 1, 9, 3, 500, 490, False),
+    (np.complex64, 600, 1, 10, 2, None, None, False),
+    (np.complex64, 13, 2, 11, 1, None, None, True),
+    (np.complex64, 13, 1, 12, 2, None, None, False),
+]
+
+
+@pytest.mark.parametrize("case", LONG_BASE4_CASES, ids=lambda c: f"{np.dtype(c[0]).name}-B{c[1]}-S{c[2]}-L{c[3]}-nb{c[4]}-I{c[5]}-O{c[6]}-inc{int(c[7])}")
+def test_base4_long_rows(case):
+    from butterfly_amd import _capi
+    dtype, B, S, L, nb, I, O, inc = case
+    say("long base4 case", case)
+    rng = np.random.default_rng(8000 + L * 7 + nb)
+    n = 1 << L
+    I_ = n if I is None else I
+    tw4 = (randn(rng, (S, nb, L // 2, n // 4, 4, 4), dtype) / 2).astype(dtype)
+    tw2 = (randn(rng, (S, nb, L % 2, n // 2, 2, 2), dtype) / np.sqrt(2)).astype(dtype)
+    x = randn(rng, (B, S, I_), dtype)
+    g = randn(rng, (B, S, n if O is None else O), dtype)
+    y_ref = oracle.butterfly_base4_fw(tw4, tw2, x, inc, O)
+    d4_ref, d2_ref, dx_ref = oracle.butterfly_base4_bw(tw4, tw2, x, g, inc)
+    y = _capi.multiply_base4_fw(dev(tw4), dev(tw2), dev(x), inc, O)
+    d4, d2, dx = _capi.multiply_base4_bw(dev(tw4), dev(tw2), dev(x), dev(g), inc)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(d4.cpu().numpy(), d4_ref) < BW_TOL
+    if L % 2:
+        assert rel_err(d2.cpu().numpy(), d2_ref) < BW_TOL

@@ -354,7 +354,8 @@ def test_kernels_with_counted_memory_waits_use_no_scratch_memory():
     assert bad == []
     with open(build.RESOURCES) as f:
         kernels = build.parse_kernel_resources(f.read())
-    assert max(v["VGPRs"] + v["AGPRs"] for v in kernels.values()) <= 128   # 16 wavefronts per compute unit
+    # 1024 threads per workgroup = 16 wavefronts per compute unit: 128 registers each
+    assert max(v["VGPRs"] + v["AGPRs"] for k, v in kernels.items() if any(g in k for g in build.GATED_KERNELS)) <= 128
 
 
 GOLDEN = os.path.join(ROOT, "tests", "golden", "butterfly_ref_cases.npz")
