@@ -544,6 +544,65 @@ __device__ __forceinline__ void load_factors(const void *tw, int64_t stack_off, 
     load_factors<T, P>(tw, stack_off, stage_stride, tw_stage, chunk, low_bits, c, ta, tb, tc, want_tc, [](auto) {});
 }
 
+// float factors, loaded so that every request of a wavefront covers consecutive pairs.  A stage
+// that runs in layout B spreads a wavefront's elements 16 apart, so asking for "my element's
+// factor row" there touches 32 different cache lines per request, sixteen wavefronts after one
+// another (measured: the factor loads of a two-block kernel took 13 thousand cycles).  Instead
+// every thread asks, for every stage, for the factor row of its layout-A element -- consecutive
+// lanes, consecutive pairs, 512 contiguous bytes per request -- and the rows of the layout-B stages
+// then travel through LDS to the threads that hold those elements in layout B (the same
+// transposition the rows themselves take; `batch` stages share a barrier).  The third entry the
+// backward kernel keeps, T[1 - r][r], is the partner's off-diagonal entry: one register exchange.
+// `scratch`: LDS, `batch` buffers of kFastRowWords float2; the caller may alias it with memory
+// that `loaded` writes (a barrier separates the two).
+template <typename P, typename F>
+__device__ __forceinline__ void load_factors_coalesced(const void *tw, int64_t stack_off, int64_t stage_stride,
+                                                       const int (&tw_stage)[kFastMaxStages], int chunk, int low_bits,
+                                                       const FastCoords &c, float (&ta)[P::NS], float (&tb)[P::NS],
+                                                       float (&tc)[P::NS], bool want_tc, float2 *scratch, int batch,
+                                                       F &&loaded)
+{
+    constexpr int NS = P::NS;
+    const float *twp = reinterpret_cast<const float *>(tw) + stack_off + P::pair_base(chunk) * 4;
+    float2 row[NS];   // (T[r][r], T[r][1 - r]) of the element this thread holds in layout A
+    static_for<0, NS>([&](auto S) {
+        constexpr int s = S;
+        constexpr int bit = P::bit(s);
+        const int r = (c.eA >> bit) & 1;
+        const int i = P::pair_index(chunk, c.eA, bit, low_bits);
+        const float2 v = *reinterpret_cast<const float2 *>(twp + tw_stage[s] * stage_stride + i * 4 + 2 * r);
+        row[s] = r ? make_float2(v.y, v.x) : v;
+    });
+    // stages that run in layout B, in order
+    struct Late { int n; int s[NS]; };
+    constexpr Late late = [] {
+        Late l{};
+        for (int s = 0; s < NS; ++s)
+            if (P::layout(s) != 0) l.s[l.n++] = s;
+        return l;
+    }();
+    if constexpr (late.n > 0) {
+        for (int j0 = 0; j0 < late.n; j0 += batch) {
+            if (j0 > 0) __syncthreads();   // the previous batch has been read
+            static_for<0, late.n>([&](auto J) {
+                if (J >= j0 && J < j0 + batch) scratch[(J - j0) * kFastRowWords + c.fA] = row[late.s[J]];
+            });
+            __syncthreads();
+            static_for<0, late.n>([&](auto J) {
+                if (J >= j0 && J < j0 + batch) row[late.s[J]] = scratch[(J - j0) * kFastRowWords + c.fB];
+            });
+        }
+        __syncthreads();   // `loaded` may write where the scratch buffers are
+    }
+    static_for<0, NS>([&](auto S) {
+        constexpr int s = S;
+        ta[s] = row[s].x;
+        tb[s] = row[s].y;
+        if (want_tc) tc[s] = partner<P::kind(s)>(tb[s], c.bperm_addr);
+        loaded(S);
+    });
+}
+
 // Moves the R values a thread holds (one per row in flight) through LDS: written at word
 // `wr`, read back at word `rd` after a barrier.  Four float rows travel as one 128-bit access.
 // WAIT: the wavefront first waits for the rows it has requested into LDS (all but the YOUNGER
@@ -667,8 +726,13 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     }
 
     T ta[NS], tb[NS], tc_unused[NS];
-    load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb,
-                       tc_unused, false);
+    if constexpr (DIRECT)
+        // (the transpose buffers are idle until the loop starts: R float2 buffers)
+        load_factors_coalesced<P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c,
+                                  ta, tb, tc_unused, false, reinterpret_cast<float2 *>(lds), R, [](auto) {});
+    else
+        load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb,
+                           tc_unused, false);
 
     const __amdgpu_buffer_rsrc_t in_rs = make_rsrc(in_base);
     const __amdgpu_buffer_rsrc_t out_rs =
@@ -993,11 +1057,23 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 
     T ta[NS], tb[NS], tc[NS], acc_self[NS], acc_cross[NS];
     auto load_all_factors = [&] {
-        load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta, tb,
-                           tc, COL, [&](auto S) {
-                               if constexpr (TB_LDS) lds_tb[S * kFastThreads + t] = tb[S];
-                               if constexpr (S < NTA) lds_ta[S * kFastThreads + t] = ta[S];
-                           });
+        auto park = [&](auto S) {
+            if constexpr (TB_LDS) lds_tb[S * kFastThreads + t] = tb[S];
+            if constexpr (S < NTA) lds_ta[S * kFastThreads + t] = ta[S];
+        };
+        if constexpr (DIRECT) {
+            // scratch for the layout-B stages' factors: the parking area of the off-diagonal
+            // entries where there is one (it is filled afterwards), else the transpose buffers
+            float2 *scratch = reinterpret_cast<float2 *>(TB_LDS ? reinterpret_cast<float *>(lds_tb)
+                                                                : reinterpret_cast<float *>(lds));
+            constexpr int room = TB_LDS ? NS * kFastThreads / (2 * kFastRowWords) : 2 * R;   // float2 buffers that fit
+            constexpr int batch = room < 5 ? room : 5;
+            load_factors_coalesced<P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits,
+                                      c, ta, tb, tc, COL, scratch, batch, park);
+        } else {
+            load_factors<T, P>(a.tw, stack * a.tw_stack_stride, a.tw_stage_stride, a.tw_stage, chunk, a.low_bits, c, ta,
+                               tb, tc, COL, park);
+        }
         static_for<0, NS>([&](auto S) {
             acc_self[S] = zero_of(T());
             acc_cross[S] = zero_of(T());
