@@ -30,6 +30,7 @@ from .multiply import butterfly_multiply  # noqa: E402
 from .multiply_base4 import butterfly_multiply_base4  # noqa: E402
 from .butterfly import Butterfly, ButterflyBmm, ButterflyUnitary  # noqa: E402
 from .butterfly_base4 import ButterflyBase4  # noqa: E402
+from .graphed import GraphedStep  # noqa: E402
 from . import combine, complex_utils, diagonal, kops, legacy, multiply, multiply_base4, permutation, special  # noqa: E402,F401
 
 __all__ = [
@@ -37,6 +38,7 @@ __all__ = [
     "ButterflyBase4",
     "ButterflyBmm",
     "ButterflyUnitary",
+    "GraphedStep",
     "butterfly_multiply",
     "butterfly_multiply_base4",
     "__version__",
