@@ -711,6 +711,8 @@ int fast4_forward(const bf_problem *p, const void *tw4, const void *tw2, const v
         }
         return BF_OK;
     }
+    if ((reinterpret_cast<uintptr_t>(tw4) & 15) != 0)
+        return fail(BF_ERR_INVALID, "twiddle4 must be 16-byte aligned");
     for (int k = first; k < last; ++k) {
         Fast4Args a = {};
         a.tw4 = static_cast<const float *>(tw4) + (int64_t)k * (L / 2) * (n / 4) * 16;
@@ -1339,6 +1341,8 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                                stream);
             if (rc) return rc;
         }
+        if (!general && (reinterpret_cast<uintptr_t>(tw4) & 15) != 0)
+            return fail(BF_ERR_INVALID, "twiddle4 must be 16-byte aligned");
         for (int k = P - 1; k >= 0 && !general; --k) {
             Fast4Args a = {};
             a.tw4 = static_cast<const float *>(tw4) + (int64_t)k * per * (n / 4) * 16;

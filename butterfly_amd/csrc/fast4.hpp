@@ -142,7 +142,11 @@ struct Factors4 {
     float row[NS][4];  // row[s][m] = T[r][r ^ m]
     float colm[WITH_COLUMN ? NS : 1][4];  // colm[s][m] = T[r ^ m][r]
 
-    __device__ __forceinline__ void load(const float *tw, const FastCoords &c)
+    // One 16-byte load per stage: the thread's row T[r][0..3] (the four lanes of a quad cover
+    // its 64 bytes), put into partner order by two conditional swaps (an xor permutation
+    // decomposes by bits).  The column comes from the partners: the thread at r ^ m holds
+    // T[r ^ m][(r ^ m) ^ m] = T[r ^ m][r] as its own entry m.  tw: 16-byte aligned.
+    __device__ __forceinline__ void load(const float *tw, const FastCoords &c, int lane)
     {
         using P = Plan4<L, INC>;
         constexpr int n = 1 << L;
@@ -153,11 +157,19 @@ struct Factors4 {
             const int e = lay ? c.eB : c.eA;
             const int r = (e >> b) & 3;
             const int q = ((e >> (b + 2)) << b) | (e & ((1 << b) - 1));
-            const float *T = tw + ((int64_t)s * (n / 4) + q) * 16;
-#pragma unroll
-            for (int m = 0; m < 4; ++m) {
-                row[s][m] = T[r * 4 + (r ^ m)];
-                if constexpr (WITH_COLUMN) colm[s][m] = T[(r ^ m) * 4 + r];
+            const float4 v = *reinterpret_cast<const float4 *>(tw + ((int64_t)s * (n / 4) + q) * 16 + r * 4);
+            const bool o1 = (r & 1) != 0, o2 = (r & 2) != 0;
+            const float a0 = o1 ? v.y : v.x, a1 = o1 ? v.x : v.y, a2 = o1 ? v.w : v.z, a3 = o1 ? v.z : v.w;
+            row[s][0] = o2 ? a2 : a0;
+            row[s][1] = o2 ? a3 : a1;
+            row[s][2] = o2 ? a0 : a2;
+            row[s][3] = o2 ? a1 : a3;
+            if constexpr (WITH_COLUMN) {
+                constexpr int KQ = P::kind(s);
+                colm[s][0] = row[s][0];
+                colm[s][1] = partner4<KQ, 1>(row[s][1], lane);
+                colm[s][2] = partner4<KQ, 2>(row[s][2], lane);
+                colm[s][3] = partner4<KQ, 3>(row[s][3], lane);
             }
         });
     }
@@ -175,7 +187,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4_fw_kernel(Fast4Args a)
     const FastCoords c = fast_coords<L>(t);
 
     Factors4<L, INC, false> f;
-    f.load(a.tw4 + stack * a.tw_stack_stride, c);
+    f.load(a.tw4 + stack * a.tw_stack_stride, c, lane);
 
     const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
     const int64_t g1 = g0 + a.groups_per_wg < a.ngroups ? g0 + a.groups_per_wg : a.ngroups;
@@ -258,7 +270,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
     const FastCoords c = fast_coords<L>(t);
 
     Factors4<L, INC, true> f;
-    f.load(a.tw4 + stack * a.tw_stack_stride, c);
+    f.load(a.tw4 + stack * a.tw_stack_stride, c, lane);
     float acc[NS][4];  // acc[s][m] = sum (g of the partner at mask m) * x = dT[r ^ m][r]
     static_for<0, NS>([&](auto S) {
 #pragma unroll

@@ -61,7 +61,8 @@ const char *bf_last_error(void);
  * Replaces butterfly_multiply_fw_cuda / butterfly_multiply_fw_cpu behind
  * torch_butterfly::butterfly_multiply_fw (csrc/butterfly.cpp:20-53,
  * csrc/cpu/butterfly_cpu.cpp:17-66, csrc/cuda/butterfly_cuda.cu:349-416).
- *   twiddle (S, nb, log_n, n/2, 2, 2) dense.                                          */
+ *   twiddle (S, nb, log_n, n/2, 2, 2) dense and 16-byte aligned (every entry point that
+ *   takes factors or writes their gradients requires that of them).                  */
 int bf_butterfly_multiply_fw(const bf_problem *p, const void *twiddle, const void *input,
                              void *output, void *workspace, size_t workspace_bytes, void *stream);
 
@@ -201,7 +202,8 @@ int bf_butterfly_scale_twiddle_bw(int dtype, int64_t nstacks, int64_t nblocks, i
 
 /* Base-4 forward: per block log_n/2 radix-4 stages from twiddle4
  * (S, nb, log_n/2, n/4, 4, 4), then one 2x2 stage from twiddle2 (S, nb, 1, n/2, 2, 2)
- * when log_n is odd (twiddle2 may be NULL when log_n is even).
+ * when log_n is odd (twiddle2 may be NULL when log_n is even).  twiddle4 (and, backward,
+ * d_twiddle4 / d_twiddle2) dense and 16-byte aligned.
  * Native counterpart of butterfly_multiply_base4_torch
  * (torch_butterfly/multiply_base4.py:7-41), which the reference runs as PyTorch ops. */
 int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4,

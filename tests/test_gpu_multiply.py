@@ -851,6 +851,18 @@ def test_misaligned_twiddle_is_rejected():
     import butterfly_amd  # noqa: F401
     y = torch.ops.torch_butterfly.butterfly_multiply_fw(tw, x, True, None)
     assert rel_err(y.cpu().numpy(), oracle.butterfly_fw(tw.cpu().numpy(), x.cpu().numpy(), True)) < FW_TOL
+    # the aligned base-4 kernels read a thread's factor row with one 16-byte load
+    numel4 = (L // 2) * (n // 4) * 16
+    big4 = torch.randn(numel4 + 4, device="cuda")
+    tw4 = big4[1:1 + numel4].view(1, 1, L // 2, n // 4, 4, 4)
+    tw2 = torch.zeros(1, 1, 0, n // 2, 2, 2, device="cuda")
+    assert tw4.is_contiguous() and tw4.data_ptr() % 16 == 4
+    with pytest.raises(_capi.ButterflyError, match="16-byte aligned"):
+        _capi.multiply_base4_fw(tw4, tw2, x, True)
+    with pytest.raises(_capi.ButterflyError, match="16-byte aligned"):
+        _capi.multiply_base4_bw(tw4, tw2, x, torch.randn_like(x), True)
+    y4 = torch.ops.torch_butterfly.butterfly_multiply_base4_fw(tw4, tw2, x, True, None)
+    assert rel_err(y4.cpu().numpy(), oracle.butterfly_base4_fw(tw4.cpu().numpy(), tw2.cpu().numpy(), x.cpu().numpy(), True)) < FW_TOL
 
 
 SAVING_CASES = [
