@@ -27,6 +27,8 @@ SYMBOLS = [
     "bf_butterfly_multiply_bw_noalloc",
     "bf_butterfly_multiply_saved_bytes", "bf_butterfly_multiply_fw_saving",
     "bf_butterfly_multiply_bw_saved_workspace_bytes", "bf_butterfly_multiply_bw_saved",
+    "bf_butterfly_multiply_base4_saved_bytes", "bf_butterfly_multiply_base4_fw_saving",
+    "bf_butterfly_multiply_base4_bw_saved_workspace_bytes", "bf_butterfly_multiply_base4_bw_saved",
 ]
 
 NOALLOC_SCRATCH_BYTES = 48 << 20
@@ -94,6 +96,12 @@ def lib():
         L.bf_butterfly_multiply_bw_saved_workspace_bytes.argtypes = [pp, ctypes.c_int]
         L.bf_butterfly_multiply_bw_saved_workspace_bytes.restype = sz
         L.bf_butterfly_multiply_bw_saved.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_base4_saved_bytes.argtypes = [pp]
+        L.bf_butterfly_multiply_base4_saved_bytes.restype = sz
+        L.bf_butterfly_multiply_base4_fw_saving.argtypes = [pp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_base4_bw_saved_workspace_bytes.argtypes = [pp]
+        L.bf_butterfly_multiply_base4_bw_saved_workspace_bytes.restype = sz
+        L.bf_butterfly_multiply_base4_bw_saved.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
         _lib = L
     return _lib
 
@@ -400,3 +408,34 @@ def multiply_base4_bw(twiddle4, twiddle2, input, grad, increasing_stride):
                                                 _ptr(grad), _ptr(d4), _ptr(d2), _ptr(d_input), _ptr(ws),
                                                 nbytes, _stream()))
     return d4, d2, d_input
+
+
+def multiply_base4_fw_bw_saving(twiddle4, twiddle2, input, grad, increasing_stride, output_size=None):
+    """Base-4 forward that leaves the backward's intermediate activations behind, then the
+    backward that reads them.  Returns (output, d_twiddle4, d_twiddle2, d_input), or None when
+    the problem saves nothing."""
+    assert twiddle4.is_contiguous() and twiddle2.is_contiguous()
+    nb = twiddle4.shape[1]
+    log_n = twiddle4.shape[2] * 2 + twiddle2.shape[2]
+    n = 1 << log_n
+    O = n if output_size is None else output_size
+    p = make_problem(input, log_n, nb, increasing_stride, O)
+    out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
+    p.output_stride = _strides(out)
+    d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
+    p.d_input_stride = _strides(d_input)
+    nsaved = lib().bf_butterfly_multiply_base4_saved_bytes(ctypes.byref(p))
+    if nsaved == 0:
+        return None
+    saved = torch.empty(nsaved, dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_base4_fw_saving(ctypes.byref(p), _ptr(twiddle4), _ptr(twiddle2), _ptr(input),
+                                                       _ptr(out), _ptr(saved), nsaved, _stream()))
+    assert tuple(grad.shape) == tuple(out.shape)
+    p.output_stride = _strides(grad)
+    d4, d2 = torch.empty_like(twiddle4), torch.empty_like(twiddle2)
+    nbytes = lib().bf_butterfly_multiply_base4_bw_saved_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
+    _check(lib().bf_butterfly_multiply_base4_bw_saved(ctypes.byref(p), _ptr(twiddle4), _ptr(twiddle2), _ptr(input),
+                                                      _ptr(grad), _ptr(saved), _ptr(d4), _ptr(d2), _ptr(d_input),
+                                                      _ptr(ws), nbytes, _stream()))
+    return out, d4, d2, d_input

@@ -1149,7 +1149,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false)
         pl.nparts = fast_grid(p->batch, (int)p->log_n, p->nstacks, 1, 1).nwg;
         size_t off = 0;
         pl.off_boundaries = off;
-        off += p->nblocks > 1 ? (size_t)(p->nblocks - 1) * pl.boundary_bytes : 0;
+        off += p->nblocks > 1 && !saved_boundaries ? (size_t)(p->nblocks - 1) * pl.boundary_bytes : 0;
         pl.off_gbuf = off;
         off += p->nblocks > 1 ? pl.boundary_bytes : 0;
         pl.off_partials = off;
@@ -1168,7 +1168,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false)
         for (int k = 0; k < lp.npass; ++k) slices = std::max(slices, pass4_slices(p, lp.pass[k]));
         size_t off = 0;
         pl.off_boundaries = off;
-        off += lp.npass > 1 ? (size_t)(lp.npass - 1) * pl.boundary_bytes : 0;
+        off += lp.npass > 1 && !saved_boundaries ? (size_t)(lp.npass - 1) * pl.boundary_bytes : 0;
         pl.off_gbuf = off;
         off += lp.npass > 1 ? pl.boundary_bytes : 0;
         pl.off_partials = off;
@@ -1293,7 +1293,8 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     const BwPlan pl = plan_bw(p, base4, saved != nullptr);
     if (!pl.fits)
         return fail(BF_ERR_UNSUPPORTED, "n = %lld does not fit in LDS for the backward pass", (long long)n);
-    if (saved && !pl.fast) return fail(BF_ERR_INVALID, "this problem has no saved activations");
+    if (saved && !(pl.fast || pl.fast4 || pl.long4)) return fail(BF_ERR_INVALID, "this problem has no saved activations");
+    const char *saved_planes = static_cast<const char *>(saved);
     if (pl.total > 0 && (!workspace || workspace_bytes < pl.total))
         return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", pl.total, workspace_bytes);
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
@@ -1315,9 +1316,13 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
         const int P = (int)p->nblocks;
         const int per = sc.per;
         const bool general = fast4_general(p);
-        auto boundary = [&](int k) { return ws + pl.off_boundaries + (size_t)(k - 1) * pl.boundary_bytes; };
-        for (int k = 0; k + 1 < P; ++k) {
-            rc = fast4_forward(p, tw4, tw2, k == 0 ? input : boundary(k), boundary(k + 1), nullptr,
+        // boundary k = activation entering block k (k >= 1): recomputed here, or kept by the forward
+        auto boundary = [&](int k) -> const char * {
+            return saved ? saved_planes + (size_t)(k - 1) * pl.boundary_bytes
+                         : ws + pl.off_boundaries + (size_t)(k - 1) * pl.boundary_bytes;
+        };
+        for (int k = 0; k + 1 < P && !saved; ++k) {
+            rc = fast4_forward(p, tw4, tw2, k == 0 ? input : boundary(k), const_cast<char *>(boundary(k + 1)), nullptr,
                                k == 0 ? x_view : dense, dense, k, k + 1, stream);
             if (rc) return rc;
         }
@@ -1379,11 +1384,14 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     if (pl.long4) {
         const Plan4Long lp = plan4_long(p, base4);
         const int P = lp.npass;
-        auto boundary = [&](int k) { return ws + pl.off_boundaries + (size_t)(k - 1) * pl.boundary_bytes; };
-        // forward replay: boundary k = activation entering pass k (k >= 1)
-        for (int k = 0; k + 1 < P; ++k) {
-            rc = long4_forward(p, sc, lp, tw2, tw4, k == 0 ? input : boundary(k), boundary(k + 1), nullptr,
-                               k == 0 ? x_view : dense, dense, k, k + 1, stream);
+        auto boundary = [&](int k) -> const char * {
+            return saved ? saved_planes + (size_t)(k - 1) * pl.boundary_bytes
+                         : ws + pl.off_boundaries + (size_t)(k - 1) * pl.boundary_bytes;
+        };
+        // forward replay: boundary k = activation entering pass k (k >= 1), unless the forward kept them
+        for (int k = 0; k + 1 < P && !saved; ++k) {
+            rc = long4_forward(p, sc, lp, tw2, tw4, k == 0 ? input : boundary(k), const_cast<char *>(boundary(k + 1)),
+                               nullptr, k == 0 ? x_view : dense, dense, k, k + 1, stream);
             if (rc) return rc;
         }
         const View dn_view = make_view(p->d_input_stride, std::min(p->input_size, n), in_perm);
@@ -1869,6 +1877,78 @@ int bf_butterfly_multiply_base4_bw(const bf_problem *p, const void *twiddle4, co
 {
     return backward(p, true, twiddle2, twiddle4, input, grad, d_twiddle2, d_twiddle4, d_input,
                     workspace, workspace_bytes, stream);
+}
+
+// Base-4 counterpart of the activation-keeping pair: the planes are the activations entering
+// every pass of the backward plan after the first (blocks for rows up to 1024, chunk and stage
+// passes beyond).
+static size_t saved4_bytes(const bf_problem *p)
+{
+    const BwPlan pl = plan_bw(p, true, true);
+    if (!pl.fits || pl.nchunks <= 1) return 0;
+    if (!(pl.fast4 && fast4_ok(p, true, false)) && !pl.long4) return 0;
+    return (size_t)(pl.nchunks - 1) * pl.boundary_bytes;
+}
+
+size_t bf_butterfly_multiply_base4_saved_bytes(const bf_problem *p)
+{
+    if (check_problem(p, true)) return 0;
+    return saved4_bytes(p);
+}
+
+int bf_butterfly_multiply_base4_fw_saving(const bf_problem *p, const void *twiddle4, const void *twiddle2,
+                                          const void *input, void *output, void *saved, size_t saved_capacity,
+                                          void *stream_)
+{
+    int rc = check_problem(p, false);
+    if (rc) return rc;
+    if ((rc = ensure_attributes())) return rc;
+    const size_t need = saved4_bytes(p);
+    if (need == 0)
+        return fail(BF_ERR_INVALID, "this problem has no activations to save: use bf_butterfly_multiply_base4_fw");
+    if (!saved || saved_capacity < need)
+        return fail(BF_ERR_WORKSPACE, "room for %zu bytes of saved activations needed, %zu given", need, saved_capacity);
+    if (!twiddle4 || !input || !output || ((p->log_n & 1) && !twiddle2)) return fail(BF_ERR_INVALID, "an operand is NULL");
+    if ((reinterpret_cast<uintptr_t>(saved) & 15) != 0) return fail(BF_ERR_INVALID, "the saved area must be 16-byte aligned");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int64_t n = (int64_t)1 << p->log_n;
+    const BwPlan pl = plan_bw(p, true, true);
+    const Schedule sc = make_schedule(p, true);
+    const View in_view = make_view(p->input_stride, std::min(p->input_size, n), nullptr);
+    const View out_view = make_view(p->output_stride, p->output_size, nullptr);
+    const View dense = dense_view(p->nstacks, n);
+    char *planes = static_cast<char *>(saved);
+    auto boundary = [&](int k) { return planes + (size_t)(k - 1) * pl.boundary_bytes; };
+    const int P = pl.nchunks;
+    const Plan4Long lp = pl.long4 ? plan4_long(p, true) : Plan4Long();
+    for (int k = 0; k < P; ++k) {
+        const void *in = k == 0 ? input : boundary(k);
+        void *out = k == P - 1 ? output : boundary(k + 1);
+        const View &iv = k == 0 ? in_view : dense, &ov = k == P - 1 ? out_view : dense;
+        rc = pl.long4 ? long4_forward(p, sc, lp, twiddle2, twiddle4, in, out, nullptr, iv, ov, k, k + 1, stream)
+                      : fast4_forward(p, twiddle4, twiddle2, in, out, nullptr, iv, ov, k, k + 1, stream);
+        if (rc) return rc;
+    }
+    return BF_OK;
+}
+
+size_t bf_butterfly_multiply_base4_bw_saved_workspace_bytes(const bf_problem *p)
+{
+    if (check_problem(p, true)) return 0;
+    return plan_bw(p, true, true).total;
+}
+
+int bf_butterfly_multiply_base4_bw_saved(const bf_problem *p, const void *twiddle4, const void *twiddle2,
+                                         const void *input, const void *grad, const void *saved, void *d_twiddle4,
+                                         void *d_twiddle2, void *d_input, void *workspace, size_t workspace_bytes,
+                                         void *stream)
+{
+    int rc = check_problem(p, true);
+    if (rc) return rc;
+    if (!saved || saved4_bytes(p) == 0)
+        return fail(BF_ERR_INVALID, "this problem has no saved activations: use bf_butterfly_multiply_base4_bw");
+    return backward(p, true, twiddle2, twiddle4, input, grad, d_twiddle2, d_twiddle4, d_input, workspace,
+                    workspace_bytes, stream, nullptr, nullptr, nullptr, nullptr, saved);
 }
 
 static int scale_twiddle(bool bw, int dtype, int64_t nstacks, int64_t nblocks, int64_t log_n, int increasing_stride,

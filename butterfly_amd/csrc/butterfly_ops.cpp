@@ -688,8 +688,10 @@ Shapes base4_shapes(const Tensor &twiddle4, const Tensor &twiddle2, const Tensor
     return s;
 }
 
-Tensor butterfly_multiply_base4_fw(const Tensor twiddle4, const Tensor twiddle2, const Tensor input,
-                                   bool increasing_stride, c10::optional<int64_t> output_size)
+// keep: when given and the backward of this problem runs in several passes, the forward runs
+// along the backward's plan and leaves the activations between its passes there
+Tensor base4_fw_impl(const Tensor &twiddle4, const Tensor &twiddle2, const Tensor &input, bool increasing_stride,
+                     c10::optional<int64_t> output_size, Tensor *keep)
 {
     const Shapes s = base4_shapes(twiddle4, twiddle2, input, "butterfly_multiply_base4_fw");
     const int64_t output_size_val = output_size.has_value() ? output_size.value() : s.n;
@@ -702,6 +704,22 @@ Tensor butterfly_multiply_base4_fw(const Tensor twiddle4, const Tensor twiddle2,
     if (output_size_val < s.n) output = output.slice(2, 0, output_size_val);
     bf_problem p = make_problem(s, x, increasing_stride, output_size_val, "butterfly_multiply_base4_fw");
     set_strides(p.output_stride, output);
+    if (keep) {
+        // (the backward will make d_input dense over max(input_size, n) columns: same plan)
+        const int64_t dw = std::max(s.input_size, s.n);
+        p.d_input_stride[0] = s.batch > 1 ? s.nstacks * dw : 0;
+        p.d_input_stride[1] = s.nstacks > 1 ? dw : 0;
+        p.d_input_stride[2] = s.input_size > 1 ? 1 : 0;
+        const size_t nsaved = bf_butterfly_multiply_base4_saved_bytes(&p);
+        if (nsaved > 0) {
+            *keep = at::empty({(int64_t)nsaved}, x.options().dtype(at::kByte));
+            check_rc(bf_butterfly_multiply_base4_fw_saving(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(),
+                                                           output.data_ptr(), keep->data_ptr(), nsaved,
+                                                           current_stream()),
+                     "butterfly_multiply_base4");
+            return output;
+        }
+    }
     const size_t ws_bytes = bf_butterfly_multiply_base4_fw_workspace_bytes(&p);
     Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
     check_rc(bf_butterfly_multiply_base4_fw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(), output.data_ptr(),
@@ -710,9 +728,15 @@ Tensor butterfly_multiply_base4_fw(const Tensor twiddle4, const Tensor twiddle2,
     return output;
 }
 
-std::tuple<Tensor, Tensor, Tensor> butterfly_multiply_base4_bw(const Tensor twiddle4, const Tensor twiddle2,
-                                                               const Tensor input, const Tensor grad,
-                                                               bool increasing_stride)
+Tensor butterfly_multiply_base4_fw(const Tensor twiddle4, const Tensor twiddle2, const Tensor input,
+                                   bool increasing_stride, c10::optional<int64_t> output_size)
+{
+    return base4_fw_impl(twiddle4, twiddle2, input, increasing_stride, output_size, nullptr);
+}
+
+// kept: the activations a forward with `keep` left behind (undefined: recompute them)
+std::tuple<Tensor, Tensor, Tensor> base4_bw_impl(const Tensor &twiddle4, const Tensor &twiddle2, const Tensor &input,
+                                                 const Tensor &grad, bool increasing_stride, const Tensor &kept)
 {
     const Shapes s = base4_shapes(twiddle4, twiddle2, input, "butterfly_multiply_base4_bw");
     CHECK_DEVICE(grad); CHECK_SAME_DEVICE(input, grad); CHECK_DIM(grad, 3);
@@ -732,6 +756,15 @@ std::tuple<Tensor, Tensor, Tensor> butterfly_multiply_base4_bw(const Tensor twid
     bf_problem p = make_problem(s, x, increasing_stride, output_size, "butterfly_multiply_base4_bw");
     set_strides(p.output_stride, g);
     set_strides(p.d_input_stride, d_input);
+    if (kept.defined()) {
+        const size_t ws_bytes = bf_butterfly_multiply_base4_bw_saved_workspace_bytes(&p);
+        Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+        check_rc(bf_butterfly_multiply_base4_bw_saved(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(), g.data_ptr(),
+                                                      kept.data_ptr(), d4.data_ptr(), d2.data_ptr(), d_input.data_ptr(),
+                                                      ws.data_ptr(), ws_bytes, current_stream()),
+                 "butterfly_multiply_base4_bw");
+        return std::make_tuple(d4, d2, d_input);
+    }
     const size_t ws_bytes = bf_butterfly_multiply_base4_bw_workspace_bytes(&p);
     Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
     check_rc(bf_butterfly_multiply_base4_bw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(), g.data_ptr(),
@@ -741,29 +774,45 @@ std::tuple<Tensor, Tensor, Tensor> butterfly_multiply_base4_bw(const Tensor twid
     return std::make_tuple(d4, d2, d_input);
 }
 
+std::tuple<Tensor, Tensor, Tensor> butterfly_multiply_base4_bw(const Tensor twiddle4, const Tensor twiddle2,
+                                                               const Tensor input, const Tensor grad,
+                                                               bool increasing_stride)
+{
+    return base4_bw_impl(twiddle4, twiddle2, input, grad, increasing_stride, Tensor());
+}
+
 class ButterflyMultiplyBase4 : public torch::autograd::Function<ButterflyMultiplyBase4> {
 public:
+    // wants_grad: as in ButterflyMultiply, the forward keeps the activations between the passes of
+    // a backward that runs in several (more than one block, or rows beyond one workgroup's reach)
     static Tensor forward(AutogradContext *ctx, Tensor twiddle4, Tensor twiddle2, Tensor input,
-                          bool increasing_stride, c10::optional<int64_t> output_size)
+                          bool increasing_stride, c10::optional<int64_t> output_size, bool wants_grad)
     {
         ctx->saved_data["increasing_stride"] = increasing_stride;
-        ctx->save_for_backward({twiddle4, twiddle2, input});
-        return butterfly_multiply_base4_fw(twiddle4, twiddle2, input, increasing_stride, output_size);
+        Tensor kept;
+        Tensor out = base4_fw_impl(twiddle4, twiddle2, input, increasing_stride, output_size,
+                                   wants_grad ? &kept : nullptr);
+        ctx->saved_data["kept"] = kept.defined();
+        if (kept.defined()) ctx->save_for_backward({twiddle4, twiddle2, input, kept});
+        else ctx->save_for_backward({twiddle4, twiddle2, input});
+        return out;
     }
 
     static variable_list backward(AutogradContext *ctx, variable_list grad_output)
     {
         const auto saved = ctx->get_saved_variables();
         const bool increasing_stride = ctx->saved_data["increasing_stride"].toBool();
-        auto r = butterfly_multiply_base4_bw(saved[0], saved[1], saved[2], grad_output[0], increasing_stride);
-        return {std::get<0>(r), std::get<1>(r), std::get<2>(r), Tensor(), Tensor()};
+        const Tensor kept = ctx->saved_data["kept"].toBool() ? saved[3] : Tensor();
+        auto r = base4_bw_impl(saved[0], saved[1], saved[2], grad_output[0], increasing_stride, kept);
+        return {std::get<0>(r), std::get<1>(r), std::get<2>(r), Tensor(), Tensor(), Tensor()};
     }
 };
 
 Tensor butterfly_multiply_base4(Tensor twiddle4, Tensor twiddle2, Tensor input, bool increasing_stride,
                                 c10::optional<int64_t> output_size)
 {
-    return ButterflyMultiplyBase4::apply(twiddle4, twiddle2, input, increasing_stride, output_size);
+    return ButterflyMultiplyBase4::apply(twiddle4, twiddle2, input, increasing_stride, output_size,
+                                         grad_wanted({twiddle4, twiddle2, input}));
 }
 
 int64_t hip_version() { return bf_hip_version(); }

@@ -221,6 +221,24 @@ int bf_butterfly_multiply_base4_bw(const bf_problem *p, const void *twiddle4,
                                    void *d_twiddle4, void *d_twiddle2, void *d_input,
                                    void *workspace, size_t workspace_bytes, void *stream);
 
+/* The base-4 pair that shares its intermediate activations, as bf_butterfly_multiply_fw_saving /
+ * _bw_saved do for base 2: several blocks (rows up to 1024) or several passes (longer rows) make
+ * bf_butterfly_multiply_base4_bw recompute the activation entering each after the first; the
+ * saving forward leaves them in `saved` (bf_butterfly_multiply_base4_saved_bytes; 0 = nothing to
+ * save, use the plain calls) and the backward reads them.  What autograd keeps for
+ * butterfly_multiply_base4_torch (torch_butterfly/multiply_base4.py:7-41) is every stage's
+ * expanded temporaries; this keeps one (B, S, n) plane per pass.                             */
+size_t bf_butterfly_multiply_base4_saved_bytes(const bf_problem *p);
+int bf_butterfly_multiply_base4_fw_saving(const bf_problem *p, const void *twiddle4,
+                                          const void *twiddle2, const void *input, void *output,
+                                          void *saved, size_t saved_capacity, void *stream);
+size_t bf_butterfly_multiply_base4_bw_saved_workspace_bytes(const bf_problem *p);
+int bf_butterfly_multiply_base4_bw_saved(const bf_problem *p, const void *twiddle4,
+                                         const void *twiddle2, const void *input,
+                                         const void *grad, const void *saved, void *d_twiddle4,
+                                         void *d_twiddle2, void *d_input, void *workspace,
+                                         size_t workspace_bytes, void *stream);
+
 /* bf_butterfly_multiply_bw for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): same operands and results,
  * but the partial sums and intermediate activations live in a fixed area of

@@ -1017,3 +1017,62 @@ def test_base4_long_rows(case):
     assert rel_err(d4.cpu().numpy(), d4_ref) < BW_TOL
     if L % 2:
         assert rel_err(d2.cpu().numpy(), d2_ref) < BW_TOL
+
+
+SAVING4_CASES = [
+    # dtype, B, S, L, nb, I, O, inc -- base-4 backward plans of several passes
+    (np.float32, 700, 2, 8, 2, None, None, True),
+    (np.float32, 90, 1, 10, 3, 1000, 900, False),
+    (np.float32, 50, 2, 7, 2, None, None, False),
+    (np.complex64, 60, 1, 6, 3, None, 50, True),
+    (np.float32, 37, 1, 12, 1, None, None, True),
+    (np.float32, 21, 2, 11, 2, 2000, 1500, False),
+    (np.complex64, 13, 1, 10, 2, None, None, False),
+]
+
+
+@pytest.mark.parametrize("case", SAVING4_CASES, ids=lambda c: f"{np.dtype(c[0]).name}-B{c[1]}-S{c[2]}-L{c[3]}-nb{c[4]}-I{c[5]}-O{c[6]}-inc{int(c[7])}")
+def test_base4_forward_that_keeps_activations(case):
+    """The base-4 saving pair against the oracle and, bit for bit, against the plain calls (same
+    kernels, the backward only skips its replay launches); the autograd operator uses it."""
+    from butterfly_amd import _capi
+    import butterfly_amd  # noqa: F401
+    dtype, B, S, L, nb, I, O, inc = case
+    say("base-4 saving case", case)
+    rng = np.random.default_rng(8100 + L * 7 + nb)
+    n = 1 << L
+    tw4 = (randn(rng, (S, nb, L // 2, n // 4, 4, 4), dtype) / 2).astype(dtype)
+    tw2 = (randn(rng, (S, nb, L % 2, n // 2, 2, 2), dtype) / np.sqrt(2)).astype(dtype)
+    x = randn(rng, (B, S, n if I is None else I), dtype)
+    g = randn(rng, (B, S, n if O is None else O), dtype)
+    t4, t2, xd, gd = dev(tw4), dev(tw2), dev(x), dev(g)
+    res = _capi.multiply_base4_fw_bw_saving(t4, t2, xd, gd, inc, O)
+    assert res is not None, "a plan of several passes keeps activations"
+    y, d4, d2, dx = res
+    y_p = _capi.multiply_base4_fw(t4, t2, xd, inc, O)
+    d4_p, d2_p, dx_p = _capi.multiply_base4_bw(t4, t2, xd, gd, inc)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_p) and torch.equal(dx, dx_p) and torch.equal(d4, d4_p) and torch.equal(d2, d2_p)
+    y_ref = oracle.butterfly_base4_fw(tw4, tw2, x, inc, O)
+    d4_ref, d2_ref, dx_ref = oracle.butterfly_base4_bw(tw4, tw2, x, g, inc)
+    assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(d4.cpu().numpy(), d4_ref) < BW_TOL
+    if L % 2:
+        assert rel_err(d2.cpu().numpy(), d2_ref) < BW_TOL
+    # the operator under autograd gives the same bits
+    a4, a2, ax = t4.clone().requires_grad_(), t2.clone().requires_grad_(), xd.clone().requires_grad_()
+    ya = torch.ops.torch_butterfly.butterfly_multiply_base4(a4, a2, ax, inc, O)
+    wrt = (a4, ax) + ((a2,) if L % 2 else ())
+    grads = torch.autograd.grad(ya, wrt, gd)
+    assert torch.equal(ya.detach(), y) and torch.equal(grads[0], d4) and torch.equal(grads[1], dx)
+    if L % 2:
+        assert torch.equal(grads[2], d2)
+
+
+def test_base4_single_pass_saves_nothing():
+    from butterfly_amd import _capi
+    t4 = torch.randn(1, 1, 4, 64, 4, 4).cuda()
+    t2 = torch.zeros(1, 1, 0, 128, 2, 2).cuda()
+    x = torch.randn(10, 1, 256).cuda()
+    assert _capi.multiply_base4_fw_bw_saving(t4, t2, x, torch.randn_like(x), True) is None

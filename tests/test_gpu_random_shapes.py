@@ -93,7 +93,8 @@ def test_random_base4_problems(chunk):
     for i in range(30):
         dtype, B, S, L, nb, I, O, inc, layout = draw_case(rng, True)
         n = 1 << L
-        say(f"random base-4 case {chunk}.{i}:", np.dtype(dtype).name, (B, S, L, nb, I, O, inc, layout))
+        saving = bool(rng.random() < 0.4)
+        say(f"random base-4 case {chunk}.{i}:", np.dtype(dtype).name, (B, S, L, nb, I, O, inc, layout), "saving" if saving else "")
         tw4 = (randn(rng, (S, nb, L // 2, n // 4, 4, 4), dtype) / 2).astype(dtype)
         tw2 = (randn(rng, (S, nb, L % 2, n // 2, 2, 2), dtype) / np.sqrt(2)).astype(dtype)
         x, xd = strided_input(rng, dtype, B, S, I, layout)
@@ -101,8 +102,12 @@ def test_random_base4_problems(chunk):
         t4, t2, gd = torch.from_numpy(tw4).cuda(), torch.from_numpy(tw2).cuda(), torch.from_numpy(g).cuda()
         y_ref = oracle.butterfly_base4_fw(tw4, tw2, x, inc, O)
         d4_ref, d2_ref, dx_ref = oracle.butterfly_base4_bw(tw4, tw2, x, g, inc)
-        y = _capi.multiply_base4_fw(t4, t2, xd, inc, O)
-        d4, d2, dx = _capi.multiply_base4_bw(t4, t2, xd, gd, inc)
+        res = _capi.multiply_base4_fw_bw_saving(t4, t2, xd, gd, inc, O) if saving else None
+        if res is not None:
+            y, d4, d2, dx = res
+        else:
+            y = _capi.multiply_base4_fw(t4, t2, xd, inc, O)
+            d4, d2, dx = _capi.multiply_base4_bw(t4, t2, xd, gd, inc)
         torch.cuda.synchronize()
         assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
         assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
