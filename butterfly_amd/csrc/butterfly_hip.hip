@@ -203,7 +203,11 @@ bool span_ok(const int64_t stride[3], int64_t rows, int64_t width, size_t elem)
 }
 
 constexpr int kMaxPasses = 96;
-constexpr int kSpanMaxBits = 5;    // widest span: tiles of 32 consecutive elements per setting of the span's bits
+// widest span: tiles of 32 consecutive floats (16 consecutive complex64: the same 128 bytes) per
+// setting of the span's bits
+constexpr int kSpanMaxBits = 5;
+constexpr int kSpanMaxBitsComplex = 6;
+constexpr int kSpanMaxStagesComplex = 10;  // stages one complex64 span pass can hold (registers + parked factors)
 constexpr int kMaxLogN = 24;  // the chunk index of the register-resident kernels travels in blockIdx.z
 
 struct Pass {
@@ -220,8 +224,16 @@ struct PassPlan {
     bool ok = false;
     int npass = 0;
     Pass pass[kMaxPasses];
-    int64_t chunks = 1;  // 1024-element chunks per row (LOW passes)
+    int low = 10;        // bits below the spans: LOW passes run on chunks of 2^low elements
 };
+
+// independent columns of work per row and stack of a pass: chunks of a LOW pass, tiles of a span
+int64_t pass_lanes(const bf_problem *p, const Pass &q)
+{
+    if (q.wide) return 1;
+    const int reach = q.span ? 10 : q.L;
+    return (int64_t)1 << (p->log_n > reach ? p->log_n - reach : 0);
+}
 
 int stage_bit(const bf_problem *p, int t)
 {
@@ -241,7 +253,8 @@ int64_t wide_min_rows(const bf_problem *p)
     return p->nblocks == 1 ? 0 : 4096;
 }
 
-PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false)
+// permuted: the call reads or writes its rows through column tables (see the low width below)
+PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false, bool permuted = false)
 {
     PassPlan pl;
     const int L = (int)p->log_n;
@@ -275,20 +288,32 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             q.inc = (p->increasing_stride != 0) != ((k & 1) != 0);
         }
     } else {
-        // bits 0..9: the kernels on 1024-element chunks; the bits above them: spans of up to
-        // kSpanMaxBits adjacent bits, as equal as possible, each one pass of the same kernels over
-        // tiles (SpanPlan) -- n = 4096: [10,11]; n = 2^20: [10..14] [15..19].
-        pl.chunks = (int64_t)1 << (L - 10);
-        const int hbits = L - 10;
-        const int nspans = (hbits + kSpanMaxBits - 1) / kSpanMaxBits;
+        // bits 0..low-1: the kernels on chunks of 2^low elements; the bits above them: spans of up
+        // to kSpanMaxBits adjacent bits, as equal as possible, each one pass of the same kernels
+        // over tiles (SpanPlan) -- float n = 4096: [10,11]; n = 2^20: [10..14] [15..19].
+        // float: low = 10.  complex64 holds one block per LOW pass and ten complex stages fill the
+        // registers (one row in flight, factors parked in LDS), so its low width is the smallest
+        // one (not below 6: then a LOW pass needs no transposition) that keeps the number of
+        // spans: n = 4096: LOW on bits 0..5, one span [6..11]; n = 8192: bits 0..6, [7..12].
+        const bool cplx = p->dtype == BF_C64;
+        const int span_max = cplx ? kSpanMaxBitsComplex : kSpanMaxBits;
+        const int nspans = (L - 10 + span_max - 1) / span_max;
+        // (rows up to 2^16 only: shorter chunks mean more rows per workgroup, and beyond that the
+        // rows a workgroup must reach with 32-bit offsets run out)
+        // Not through column tables either: a gather or scatter touches one element per 128-byte
+        // line and short chunk, where chunks of 1024 still find several (measured on the bit
+        // reversal of special.fft: 1.30 ms against 0.92 ms per step).
+        const int low = cplx && L <= 16 && !permuted ? std::max(6, L - span_max * nspans) : 10;
+        pl.low = low;
+        const int hbits = L - low;
         int group_lb[16], group_bits[16], ngroups = 0;
-        for (int b = 10; b < L; ++ngroups) {
+        for (int b = low; b < L; ++ngroups) {
             group_lb[ngroups] = b;
             group_bits[ngroups] = hbits / nspans + (ngroups < hbits % nspans ? 1 : 0);
             b += group_bits[ngroups];
         }
         auto group_of = [&](int bit) {
-            if (bit < 10) return -1;
+            if (bit < low) return -1;
             int g = 0;
             while (bit >= group_lb[g] + group_bits[g]) ++g;
             return g;
@@ -304,7 +329,8 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
             // a group also takes the way back down where two blocks meet in the row's top bits
             const int lb = high ? group_lb[grp] : 0;
             const int H = high ? group_bits[grp] : 0;
-            const int cap = high ? 2 * H : 10 * max_nb;
+            // (a complex64 span takes the way back down only if both sweeps fit one pass)
+            const int cap = high ? (cplx && 2 * H > kSpanMaxStagesComplex ? H : 2 * H) : low * max_nb;
             int u = t;
             while (u < NS && group_of(stage_bit(p, u)) == grp && u - t < cap) ++u;
             q.t1 = u;
@@ -318,9 +344,9 @@ PassPlan build_passes(const bf_problem *p, bool base4, bool forward_only = false
                 q.mode = u - t == 2 * H ? 2 : (stage_bit(p, t) == lb ? 0 : 1);
                 q.inc = q.mode != 1;
             } else {
-                q.L = 10;
-                if ((u - t) != 10 && (u - t) != 20) return pl;
-                q.NB = (u - t) / 10;
+                q.L = low;
+                if ((u - t) != low && (u - t) != 2 * low) return pl;
+                q.NB = (u - t) / low;
                 q.inc = stage_bit(p, t) == 0;
             }
             t = u;
@@ -395,7 +421,7 @@ bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
     for (int k = 0; k < pl.npass; ++k) {
         const Pass &q = pl.pass[k];
         const FastGrid g = q.wide ? wide_grid(p->batch, p->nstacks)
-                                  : fast_grid(p->batch, q.L, p->nstacks * pl.chunks, backward ? 1 : fw_rows(p),
+                                  : fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), backward ? 1 : fw_rows(p),
                                               backward ? 1 : kFastFwWgPerCu, cap);
         rows = std::max(rows, (g.groups_per_wg + kFastFwRows + 2) * g.slots);
     }
@@ -440,35 +466,46 @@ void launch_fast_bw_t(bool cplx, bool two_rows, const FastBwArgs &a, dim3 grid, 
 
 // SpanPlan passes: the LOW kernels on the tiles of a span of q.H high bits.
 template <int H, int MODE>
-void launch_span_t(bool cplx, bool backward, bool two_rows, const FastFwArgs *fw, const FastBwArgs *bw, dim3 grid,
+bool launch_span_t(bool cplx, bool backward, bool two_rows, const FastFwArgs *fw, const FastBwArgs *bw, dim3 grid,
                    hipStream_t stream)
 {
     using P = SpanPlan<H, MODE>;
     const dim3 block(kFastThreads);
-    if (!backward) {
-        if (cplx) hipLaunchKernelGGL((fast_fw_kernel<float2, P, kFastFwRowsComplex>), grid, block, 0, stream, *fw);
-        else hipLaunchKernelGGL((fast_fw_kernel<float, P, kFastFwRows>), grid, block, 0, stream, *fw);
-    } else if (cplx) {
-        hipLaunchKernelGGL((fast_bw_kernel<float2, P>), grid, block, 0, stream, *bw);
-    } else if (two_rows) {
-        hipLaunchKernelGGL((fast_bw_kernel<float, P, 2>), grid, block, 0, stream, *bw);
-    } else {
-        hipLaunchKernelGGL((fast_bw_kernel<float, P>), grid, block, 0, stream, *bw);
+    // which combinations the host plans: float spans of up to kSpanMaxBits bits, complex64 ones of
+    // up to kSpanMaxBitsComplex bits and kSpanMaxStagesComplex stages
+    constexpr bool for_float = H <= kSpanMaxBits;
+    constexpr bool for_complex = H * (MODE == 2 ? 2 : 1) <= kSpanMaxStagesComplex;
+    if (cplx) {
+        if constexpr (for_complex) {
+            if (!backward) hipLaunchKernelGGL((fast_fw_kernel<float2, P, kFastFwRowsComplex>), grid, block, 0, stream, *fw);
+            else hipLaunchKernelGGL((fast_bw_kernel<float2, P>), grid, block, 0, stream, *bw);
+            return true;
+        }
+        return false;
     }
+    if constexpr (for_float) {
+        if (!backward) hipLaunchKernelGGL((fast_fw_kernel<float, P, kFastFwRows>), grid, block, 0, stream, *fw);
+        else if (two_rows) hipLaunchKernelGGL((fast_bw_kernel<float, P, 2>), grid, block, 0, stream, *bw);
+        else hipLaunchKernelGGL((fast_bw_kernel<float, P>), grid, block, 0, stream, *bw);
+        return true;
+    }
+    return false;
 }
 
 int launch_span(bool cplx, const Pass &q, bool backward, bool two_rows, const FastFwArgs *fw, const FastBwArgs *bw,
                 dim3 grid, hipStream_t stream)
 {
 #define BF_SPAN_CASES(HH)                                                                          \
-    case HH * 3 + 0: launch_span_t<HH, 0>(cplx, backward, two_rows, fw, bw, grid, stream); break;   \
-    case HH * 3 + 1: launch_span_t<HH, 1>(cplx, backward, two_rows, fw, bw, grid, stream); break;   \
-    case HH * 3 + 2: launch_span_t<HH, 2>(cplx, backward, two_rows, fw, bw, grid, stream); break;
+    case HH * 3 + 0: ok = launch_span_t<HH, 0>(cplx, backward, two_rows, fw, bw, grid, stream); break;   \
+    case HH * 3 + 1: ok = launch_span_t<HH, 1>(cplx, backward, two_rows, fw, bw, grid, stream); break;   \
+    case HH * 3 + 2: ok = launch_span_t<HH, 2>(cplx, backward, two_rows, fw, bw, grid, stream); break;
+    bool ok = false;
     switch (q.H * 3 + q.mode) {
-        BF_SPAN_CASES(1) BF_SPAN_CASES(2) BF_SPAN_CASES(3) BF_SPAN_CASES(4) BF_SPAN_CASES(5)
-        default: return fail(BF_ERR_UNSUPPORTED, "no kernel for a span of %d bits", q.H);
+        BF_SPAN_CASES(1) BF_SPAN_CASES(2) BF_SPAN_CASES(3) BF_SPAN_CASES(4) BF_SPAN_CASES(5) BF_SPAN_CASES(6)
+        default: break;
     }
 #undef BF_SPAN_CASES
+    if (!ok) return fail(BF_ERR_UNSUPPORTED, "no kernel for a span of %d bits in mode %d", q.H, q.mode);
     return BF_OK;
 }
 
@@ -541,7 +578,7 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
             else hipLaunchKernelGGL((wide_fw_kernel<float, 11, false>), grid, block, 0, stream, a);
             BF_HIP_CHECK(hipGetLastError());
         } else {
-            const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pl.chunks, fw_rows(p), kFastFwWgPerCu,
+            const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), fw_rows(p), kFastFwWgPerCu,
                                          row_cap(p, false));
             FastFwArgs a = {};
             a.tw = tw;
@@ -559,7 +596,7 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
                 a.bias = bias;
                 if (bias_done) *bias_done = true;
             }
-            const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)pl.chunks);
+            const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)pass_lanes(p, q));
             if (q.span) {
                 a.low_bits = q.lb;
                 const int rc = launch_span(p->dtype == BF_C64, q, false, false, &a, nullptr, grid, stream);
@@ -1050,7 +1087,7 @@ int forward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, c
         return p->dtype == BF_C64 ? launch_bias_add<float2>(p, bias, output, out_view, stream)
                                   : launch_bias_add<float>(p, bias, output, out_view, stream);
     }
-    const PassPlan mp = build_passes(p, base4, true);
+    const PassPlan mp = build_passes(p, base4, true, in_perm || out_index);
     if (mp.ok && passes_addressable(p, mp, false)) {
         const size_t need = forward_workspace(p, base4);
         if (need > 0 && (!workspace || workspace_bytes < need))
@@ -1132,7 +1169,7 @@ struct BwPlan {
 
 // saved_boundaries: the activations entering every pass after the first come from the caller
 // (left behind by the forward call that saves them) instead of being recomputed into the workspace.
-BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false)
+BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false, bool permuted = false)
 {
     BwPlan pl = {};
     const int64_t n = (int64_t)1 << p->log_n;
@@ -1176,7 +1213,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false)
         pl.total = off;
         return pl;
     }
-    const PassPlan mp = build_passes(p, base4);
+    const PassPlan mp = build_passes(p, base4, false, permuted);
     if (mp.ok && passes_addressable(p, mp, true)) {
         // boundaries: the activation entering every pass after the first; one gradient plane
         // that the passes update in place; partial slices sized for the widest pass.
@@ -1188,7 +1225,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false)
         int64_t nparts = 1, slices = 1;  // slices: partial (stage, 2n) slices of the pass that needs most
         for (int k = 0; k < mp.npass; ++k) {
             const Pass &q = mp.pass[k];
-            const int64_t np = fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1, row_cap(p, true)).nwg;
+            const int64_t np = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), 1, 1, row_cap(p, true)).nwg;
             nparts = std::max(nparts, np);
             slices = std::max(slices, np * (q.t1 - q.t0));
         }
@@ -1290,7 +1327,8 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const Schedule sc = make_schedule(p, base4);
     const int64_t n = (int64_t)1 << p->log_n;
-    const BwPlan pl = plan_bw(p, base4, saved != nullptr);
+    const bool permuted = in_perm || out_index;
+    const BwPlan pl = plan_bw(p, base4, saved != nullptr, permuted);
     if (!pl.fits)
         return fail(BF_ERR_UNSUPPORTED, "n = %lld does not fit in LDS for the backward pass", (long long)n);
     if (saved && !(pl.fast || pl.fast4 || pl.long4)) return fail(BF_ERR_INVALID, "this problem has no saved activations");
@@ -1419,7 +1457,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     }
 
     if (pl.fast) {
-        const PassPlan mp = build_passes(p, base4);
+        const PassPlan mp = build_passes(p, base4, false, permuted);
         const int P = mp.npass;
         char *bounds = saved ? const_cast<char *>(static_cast<const char *>(saved)) : ws + pl.off_boundaries;
         auto boundary = [&](int k) { return bounds + (size_t)(k - 1) * pl.boundary_bytes; };
@@ -1440,7 +1478,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
             const View giv = k == 0 ? dn_view : dense;
             int64_t nparts = 0;
             {
-                const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * mp.chunks, 1, 1, row_cap(p, true));
+                const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), 1, 1, row_cap(p, true));
                 FastBwArgs a = {};
                 a.tw = tw2;
                 a.tw_stack_stride = sc.tw2_stack_stride;
@@ -1463,7 +1501,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
                     a.bias_width = p->output_size;
                     *bias_nparts = g.nwg;
                 }
-                const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)mp.chunks);
+                const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, (unsigned)pass_lanes(p, q));
                 // two row groups in flight once a workgroup has enough of them to fill the pipeline
                 if (q.span) {
                     a.low_bits = q.lb;
@@ -1564,6 +1602,12 @@ int scratch_of_current_device(void **ptr)
     return BF_OK;
 }
 
+// Workspace of a base-2 backward call whatever its column tables: the plan may differ with them.
+size_t bw_workspace_total(const bf_problem *p, bool saved_boundaries)
+{
+    return std::max(plan_bw(p, false, saved_boundaries, false).total, plan_bw(p, false, saved_boundaries, true).total);
+}
+
 }  // namespace
 
 extern "C" {
@@ -1610,7 +1654,7 @@ int bf_butterfly_multiply_fw(const bf_problem *p, const void *twiddle, const voi
 size_t bf_butterfly_multiply_bw_workspace_bytes(const bf_problem *p)
 {
     if (check_problem(p, true)) return 0;
-    return plan_bw(p, false).total;
+    return bw_workspace_total(p, false);
 }
 
 int bf_butterfly_multiply_bw(const bf_problem *p, const void *twiddle, const void *input,
@@ -1686,7 +1730,7 @@ static size_t bias_area_bytes(const bf_problem *p)
 size_t bf_butterfly_multiply_bias_bw_workspace_bytes(const bf_problem *p)
 {
     if (check_problem(p, true)) return 0;
-    return align256(plan_bw(p, false).total) + bias_area_bytes(p);
+    return align256(bw_workspace_total(p, false)) + bias_area_bytes(p);
 }
 
 static int bias_backward(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
@@ -1695,7 +1739,7 @@ static int bias_backward(const bf_problem *p, const void *twiddle, const void *i
 {
     int rc = check_problem(p, true);
     if (rc) return rc;
-    const size_t main_bytes = align256(plan_bw(p, false, saved != nullptr).total);
+    const size_t main_bytes = align256(plan_bw(p, false, saved != nullptr, in_perm || out_index).total);
     const size_t need = main_bytes + bias_area_bytes(p);
     if (!workspace || workspace_bytes < need)
         return fail(BF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
@@ -1752,11 +1796,17 @@ int bf_butterfly_multiply_perm_bw(const bf_problem *p, const void *twiddle, cons
 // Bytes of activations the saving forward leaves for the backward: one dense (B, S, n) plane per
 // pass of the backward plan after the first; 0 when the backward is a single pass (or runs on
 // kernels that do not use such planes).
-static size_t saved_bytes(const bf_problem *p)
+static size_t saved_bytes_of_plan(const bf_problem *p, bool permuted)
 {
-    const BwPlan pl = plan_bw(p, false, true);
+    const BwPlan pl = plan_bw(p, false, true, permuted);
     if (!pl.fits || !pl.fast || pl.nchunks <= 1) return 0;
     return (size_t)(pl.nchunks - 1) * pl.boundary_bytes;
+}
+
+// room for the saved activations of a call with or without column tables (the plans may differ)
+static size_t saved_bytes(const bf_problem *p)
+{
+    return std::max(saved_bytes_of_plan(p, false), saved_bytes_of_plan(p, true));
 }
 
 size_t bf_butterfly_multiply_saved_bytes(const bf_problem *p)
@@ -1782,8 +1832,10 @@ int bf_butterfly_multiply_fw_saving(const bf_problem *p, const void *twiddle, co
         return fail(BF_ERR_INVALID, "twiddle and the saved area must be 16-byte aligned");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const int64_t n = (int64_t)1 << p->log_n;
-    const PassPlan mp = build_passes(p, false);
-    const BwPlan pl = plan_bw(p, false, true);
+    const bool permuted = in_perm || out_index;
+    const PassPlan mp = build_passes(p, false, false, permuted);
+    const BwPlan pl = plan_bw(p, false, true, permuted);
+    if (mp.npass < 2 || !pl.fast) return fail(BF_ERR_INVALID, "this problem has no activations to save");
     const View in_view = make_view(p->input_stride, std::min(p->input_size, n), in_perm);
     const View out_view = make_view(p->output_stride, p->output_size, out_index);
     const View dense = dense_view(p->nstacks, n);
@@ -1807,7 +1859,7 @@ int bf_butterfly_multiply_fw_saving(const bf_problem *p, const void *twiddle, co
 size_t bf_butterfly_multiply_bw_saved_workspace_bytes(const bf_problem *p, int with_bias)
 {
     if (check_problem(p, true)) return 0;
-    const size_t main_bytes = plan_bw(p, false, true).total;
+    const size_t main_bytes = bw_workspace_total(p, true);
     return with_bias ? align256(main_bytes) + bias_area_bytes(p) : main_bytes;
 }
 
@@ -1845,10 +1897,10 @@ int bf_describe_plan(const bf_problem *p, int backward, char *text, size_t capac
                 snprintf(line, sizeof line, "wide t=%d..%d L=%d inc=%d\n", q.t0, q.t1, q.L, (int)q.inc);
             else if (q.span)
                 snprintf(line, sizeof line, "span t=%d..%d lb=%d bits=%d mode=%d tiles=%lld\n", q.t0, q.t1, q.lb, q.H,
-                         q.mode, (long long)mp.chunks);
+                         q.mode, (long long)pass_lanes(p, q));
             else
                 snprintf(line, sizeof line, "low t=%d..%d L=%d nb=%d inc=%d chunks=%lld\n", q.t0, q.t1, q.L, q.NB,
-                         (int)q.inc, (long long)mp.chunks);
+                         (int)q.inc, (long long)pass_lanes(p, q));
             out += line;
         }
     }

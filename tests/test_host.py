@@ -290,11 +290,16 @@ def _parse_plan(lines):
 def test_launch_plans_cover_every_stage_once():
     """bf_describe_plan (host only): for every row length up to 2^24, both dtypes, both stride
     orders, forward and backward, the passes cover the stage list exactly once in order; low
-    passes hold whole blocks of ten low bits; a span pass works on at most five adjacent bits
-    from bit 10 up in one sweep up, one sweep down or both; the spans tile bits 10..L-1."""
+    passes hold whole blocks of the `low` lowest bits (10 for float; for complex64 rows of 2048
+    to 65536 the smallest width from 6 up that does not add a span); a span pass works on at most five
+    (complex64: six) adjacent bits from bit `low` up in one sweep up, one sweep down or both (a
+    complex64 pass holds at most ten stages); the spans tile bits low..L-1."""
     from butterfly_amd import _capi
     for cplx in (0, 1):
         for L in range(1, 25):
+            span_max = 6 if cplx else 5
+            nspans = (max(L, 10) - 10 + span_max - 1) // span_max
+            low = max(6, L - span_max * nspans) if cplx and 10 < L <= 16 else min(L, 10)
             for nb in (1, 2, 3):
                 for inc in (True, False):
                     for backward in (False, True):
@@ -314,16 +319,17 @@ def test_launch_plans_cover_every_stage_once():
                             t = b
                             stage_bits = bits[a:b]
                             if q["kind"] == "low":
-                                assert q["L"] == min(L, 10) and b - a == q["L"] * q["nb"], key
-                                assert all(x < 10 for x in stage_bits), key
-                                assert q["chunks"] == (1 << max(0, L - 10)), key
+                                assert q["L"] == low and b - a == q["L"] * q["nb"], key
+                                assert all(x < low for x in stage_bits), key
+                                assert q["chunks"] == (1 << (L - low)), key
                                 assert q["nb"] <= (1 if cplx else 2), key
                                 assert q["inc"] == int(stage_bits[0] == 0 and q["L"] > 1 or (q["L"] == 1 and inc != ((a // L) % 2 == 1))), key
                             elif q["kind"] == "wide":
                                 assert not backward and L in (11, 12) and b - a == L, key
                             elif q["kind"] == "span":
                                 lb, h = q["lb"], q["bits"]
-                                assert lb >= 10 and 1 <= h <= 5 and q["tiles"] == (1 << (L - 10)), key
+                                assert lb >= low and 1 <= h <= span_max and q["tiles"] == (1 << (L - 10)), key
+                                assert not cplx or b - a <= 10, key
                                 up, down = list(range(lb, lb + h)), list(range(lb + h - 1, lb - 1, -1))
                                 assert stage_bits == [up, down, up + down][q["mode"]], key
                                 groups.add((lb, h))
@@ -332,13 +338,15 @@ def test_launch_plans_cover_every_stage_once():
                         assert t == len(bits), key
                         if groups:
                             covered = sorted(x for lb, h in groups for x in range(lb, lb + h))
-                            assert covered == list(range(10, L)), key
+                            assert covered == list(range(low, L)), key
     # the configurations the benchmark is quoted on
     assert _capi.describe_plan(0, 16384, 1, 10, 2, False, True) == ["low t=0..20 L=10 nb=2 inc=0 chunks=1"]
     assert [l.split()[0] for l in _capi.describe_plan(0, 32768, 1, 12, 2, True, False)] == ["wide", "wide"]
     assert [l.split()[0] for l in _capi.describe_plan(0, 32768, 1, 12, 2, True, True)] == ["low", "span", "low"]
     assert [l.split()[0] for l in _capi.describe_plan(0, 2048, 1, 13, 1, True, True)] == ["low", "span"]
     assert [l.split()[0] for l in _capi.describe_plan(0, 16, 1, 20, 1, True, False)] == ["low", "span", "span"]
+    assert _capi.describe_plan(1, 8192, 1, 12, 1, True, True) == ["low t=0..6 L=6 nb=1 inc=1 chunks=64",
+                                                                  "span t=6..12 lb=6 bits=6 mode=0 tiles=4"]
 
 
 def test_kernels_with_counted_memory_waits_use_no_scratch_memory():
