@@ -205,7 +205,7 @@ def make_operands(c, torch, dev):
     elif c["cplx"] and S == 1 and nb == 1:
         from butterfly_amd import special
         tws = (special.fft(n, normalized=True, with_br_perm=False).twiddle.detach().to(dev),)
-    elif nb == 2 and L == 12:
+    elif nb == 2 and L == 12 and not c["cplx"]:
         import butterfly_amd
         tws = (butterfly_amd.Butterfly(n, n, bias=True, init="ortho", nblocks=2).twiddle.detach().to(dev),)
     else:
