@@ -146,3 +146,16 @@ def test_base4_shape_at_full_size():
     rng = np.random.default_rng(4300)
     tw4, tw2, x, g = base4_operands(rng, 16384, 4, 8, 1)
     check_base4(tw4, tw2, x, g, True, what="base-4 shape at full size")
+
+
+@pytest.mark.parametrize("shape", [(200003, 1, 5, 1), (300001, 1, 4, 2), (120007, 2, 6, 1), (70001, 1, 6, 3)],
+                         ids=lambda s: f"B{s[0]}-S{s[1]}-L{s[2]}-nb{s[3]}")
+@pytest.mark.parametrize("inc", [True, False], ids=["inc", "dec"])
+def test_complex_short_rows_many_row_groups_per_workgroup(shape, inc):
+    """complex64 rows of 16 to 64 elements (what the low passes of longer complex rows and the
+    small butterflies of KOP2d run on) and enough of them that every workgroup walks its row
+    loop many times, with a ragged last group."""
+    B, S, L, nb = shape
+    rng = np.random.default_rng(4400 + L * 10 + nb + int(inc))
+    tw, x, g = base2_operands(rng, np.complex64, B, S, L, nb)
+    check_base2(tw, x, g, inc, what="complex short rows")
