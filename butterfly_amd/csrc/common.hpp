@@ -17,9 +17,12 @@ __device__ __forceinline__ float conj_of(float a) { return a; }
 __device__ __forceinline__ float2 conj_of(float2 a) { return make_float2(a.x, -a.y); }
 
 __device__ __forceinline__ float mul(float a, float b) { return a * b; }
+// (the fused multiply-adds are spelled out: left to the compiler, which of the two products of a
+// component gets fused depends on the code around the call, and the same stage would round
+// differently in different kernels)
 __device__ __forceinline__ float2 mul(float2 a, float2 b)
 {
-    return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x);
+    return make_float2(fmaf(a.x, b.x, -(a.y * b.y)), fmaf(a.x, b.y, a.y * b.x));
 }
 
 // acc + a * b

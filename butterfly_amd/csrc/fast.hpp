@@ -709,9 +709,12 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     const int slot_d = t >> L, col_d = P::column(chunk, t & (n - 1), a.low_bits);
     const int64_t in_col_d = view_col(a.in_view, col_d);
     const int in_dma = in_col_d >= 0 ? slot_d * in_row + (int)(in_col_d * a.in_view.se * EB) : kOob;
-    const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
-    auto fetch_row = [&](int grel, int set, int r) {
-        const bool ok = (grel + r) * SLOTS + slot_d < rows_valid;
+    // (wave-uniform: kept in a scalar register, so the per-row slot offsets are scalar additions)
+    const unsigned rows_addr = __builtin_amdgcn_readfirstlane(
+        (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4);
+    // (`full`: the caller knows that the row group exists for every row slot of the workgroup)
+    auto fetch_row = [&](int grel, int set, int r, bool full = false) {
+        const bool ok = full || (grel + r) * SLOTS + slot_d < rows_valid;
         load_row_to_lds(in_desc, rows_addr + (set * R + r) * kFastRowWords * 4, ok ? in_dma : kOob,
                         (grel + r) * SLOTS * in_row);
     };
@@ -755,9 +758,9 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     // The requests of an iteration are spread over its TT + 1 phases (row r goes out at the
     // start of phase r mod (TT + 1)): sixteen wavefronts asking for R rows each at the same
     // moment, right behind the previous iteration's stores, queue up at the memory pipeline.
-    auto fetch_phase = [&](int grel, int set, auto PHASE) {
+    auto fetch_phase = [&](int grel, int set, auto PHASE, bool full) {
         static_for<0, R>([&](auto RR) {
-            if constexpr (RR % (TT + 1) == decltype(PHASE)::value) fetch_row(grel, set, RR);
+            if constexpr (RR % (TT + 1) == decltype(PHASE)::value) fetch_row(grel, set, RR, full);
         });
     };
     // requests of an iteration that go out before its last barrier (all of them when there is none)
@@ -786,11 +789,14 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
 #pragma unroll
         for (int r = 0; r < R; ++r) buf_store(out_rs, kOob, EB * r, zero_of(T()));
     }
-    for (int grel = 0; grel < ng; grel += R) {
+    // FULL: the rows this iteration requests (two iterations ahead) and stores exist for every
+    // row slot, so neither needs its range mask: all but the last iterations of a workgroup.
+    auto iteration = [&](int grel, auto FULL) {
+        constexpr bool full = decltype(FULL)::value;
         T v[R];
         if constexpr (DIRECT) {
             const int set = (grel / R) & 3;
-            fetch_phase(grel + 2 * R, (set + 2) & 3, std::integral_constant<int, 0>{});
+            fetch_phase(grel + 2 * R, (set + 2) & 3, std::integral_constant<int, 0>{}, full);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const float x = lds_rows[(set * R + r) * kFastRowWords + (SF ? c.fB : c.fA)];
@@ -812,7 +818,7 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
                 const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
                 transpose_rows<T, R, DIRECT && nth + 1 == TT, YOUNGER>(buf, wr, rd, v);
                 if constexpr (DIRECT)
-                    fetch_phase(grel + 2 * R, (((grel / R) & 3) + 2) & 3, std::integral_constant<int, nth + 1>{});
+                    fetch_phase(grel + 2 * R, (((grel / R) & 3) + 2) & 3, std::integral_constant<int, nth + 1>{}, full);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) v[r] = fw_product<K>(v[r], ta[s], tb[s], c.bperm_addr);
@@ -822,15 +828,20 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
             T *buf = lds + (nth & 1) * R * kFastRowWords;
             transpose_rows<T, R, DIRECT, YOUNGER>(buf, c.fB, c.fA, v);
             if constexpr (DIRECT)
-                fetch_phase(grel + 2 * R, (((grel / R) & 3) + 2) & 3, std::integral_constant<int, nth + 1>{});
+                fetch_phase(grel + 2 * R, (((grel / R) & 3) + 2) & 3, std::integral_constant<int, nth + 1>{}, full);
         }
         if constexpr (DIRECT && TT == 0) wait_rows_in_lds<YOUNGER>();
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const bool ok = (grel + r) * SLOTS + c.slot < rows_valid;
+            const bool ok = full || (grel + r) * SLOTS + c.slot < rows_valid;
             buf_store(out_rs, ok ? out_thr : kOob, (grel + r) * SLOTS * out_row, add(v[r], bias));
         }
+    };
+    int grel = 0;
+    if constexpr (DIRECT) {
+        for (; grel < ng && (grel + 3 * R) * SLOTS <= rows_valid; grel += R) iteration(grel, std::true_type{});
     }
+    for (; grel < ng; grel += R) iteration(grel, std::false_type{});
     if constexpr (DIRECT) wait_rows_in_lds<0>();  // requests past the last group (they fetch nothing)
 }
 
@@ -1095,8 +1106,10 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const int64_t gi_col = view_col(a.gi_view, col);
     const int gi_thr = gi_col >= 0 ? c.slot * gi_row + (int)(gi_col * a.gi_view.se * EB) : kOob;
     auto group_ok = [&](int grp) { return grp >= 0 && grp * SLOTS + c.slot < rows_valid; };
-    auto store_grad = [&](int grp, T gval) {
-        buf_store(gi_rs, group_ok(grp) ? gi_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * gi_row, gval);
+    // (`full`: the caller knows that the group exists for every row slot of the workgroup)
+    auto store_grad = [&](int grp, T gval, bool full = false) {
+        if (full) buf_store(gi_rs, gi_thr, grp * SLOTS * gi_row, gval);
+        else buf_store(gi_rs, group_ok(grp) ? gi_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * gi_row, gval);
     };
 
     // --- operand fetch, register flavour: thread t holds its layout-A element
@@ -1117,7 +1130,9 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const int64_t x_col_d = view_col(a.x_view, col_d), g_col_d = view_col(a.g_view, col_d);
     const int x_dma = x_col_d >= 0 ? slot_d * x_row + (int)(x_col_d * a.x_view.se * EB) : kOob;
     const int g_dma = g_col_d >= 0 ? slot_d * g_row + (int)(g_col_d * a.g_view.se * EB) : kOob;
-    const unsigned rows_addr = (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4;
+    // (wave-uniform: kept in a scalar register, so the per-row slot offsets are scalar additions)
+    const unsigned rows_addr = __builtin_amdgcn_readfirstlane(
+        (unsigned)(unsigned long long)(LdsFloat *)lds_rows + (unsigned)(t >> 6) * 65 * 4);
     auto group_ok_d = [&](int grp) { return grp >= 0 && grp * SLOTS + slot_d < rows_valid; };
     // Iteration j replays the R groups R j .. R j + R - 1 (they sit in x set j & 3) and sweeps
     // them one iteration later (output-gradient set j & 3).  Rows are requested AHEAD
@@ -1130,20 +1145,27 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     constexpr bool BIAS_SUM = DIRECT && SLOTS == 1;
     const bool bias_on = BIAS_SUM && a.bias_partial != nullptr;
     if constexpr (BIAS_SUM) lds_bias[t] = 0.0f;
-    auto fetch_x = [&](int j) {
+    auto fetch_x = [&](int j, bool full = false) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int grp = R * j + r;
-            load_row_to_lds(x_desc, rows_addr + ((j & 3) * R + r) * kFastRowWords * 4,
-                            group_ok_d(grp) ? x_dma : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row);
+            if (full)
+                load_row_to_lds(x_desc, rows_addr + ((j & 3) * R + r) * kFastRowWords * 4, x_dma, grp * SLOTS * x_row);
+            else
+                load_row_to_lds(x_desc, rows_addr + ((j & 3) * R + r) * kFastRowWords * 4,
+                                group_ok_d(grp) ? x_dma : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row);
         }
     };
-    auto fetch_g = [&](int j) {
+    auto fetch_g = [&](int j, bool full = false) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int grp = R * j + r;
-            load_row_to_lds(g_desc, rows_addr + ((4 + (j & 3)) * R + r) * kFastRowWords * 4,
-                            group_ok_d(grp) ? g_dma : kOob, (grp < 0 ? 0 : grp) * SLOTS * g_row);
+            if (full)
+                load_row_to_lds(g_desc, rows_addr + ((4 + (j & 3)) * R + r) * kFastRowWords * 4, g_dma,
+                                grp * SLOTS * g_row);
+            else
+                load_row_to_lds(g_desc, rows_addr + ((4 + (j & 3)) * R + r) * kFastRowWords * 4,
+                                group_ok_d(grp) ? g_dma : kOob, (grp < 0 ? 0 : grp) * SLOTS * g_row);
         }
     };
 
@@ -1192,8 +1214,13 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     // the previous iteration's input gradients still in layout B (DEFER only).  FLIP
     // alternates between the two unrolled calls and keeps the LDS buffers alternating when
     // the number of phases is odd.
-    auto iteration = [&](auto FLIP, int it, T (&vF)[R], T (&gv)[R], T (&carry)[R], T (&cur)[R][NS], T (&nxt)[R][NS]) {
+    // FULL: every group this iteration touches (the rows it requests, the gradient it sweeps, the
+    // gradient it stores) exists for every row slot, so no access needs its range mask: true for
+    // all but the first two and the last few iterations of a workgroup.
+    auto iteration = [&](auto FLIP, auto FULL, int it, T (&vF)[R], T (&gv)[R], T (&carry)[R], T (&cur)[R][NS],
+                         T (&nxt)[R][NS]) {
         constexpr int flip = decltype(FLIP)::value;
+        constexpr bool full = decltype(FULL)::value;
         // The next iteration's rows are read out of LDS a phase ahead of their use, right behind
         // the barrier that publishes them, where the registers allow (two more live values).
         constexpr bool PREREAD = DIRECT && Q::K >= 1 && NS * R < 20;
@@ -1206,8 +1233,8 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         static_assert(!DIRECT || (Q::K == 0 ? 3 * R : YOUNGER) == bw_operations_behind_awaited_rows<Q, R, AHEAD>(),
                       "wait count of the row fetch");
         if constexpr (DIRECT) {
-            fetch_x(it + 1 + AHEAD);
-            fetch_g(it + AHEAD);
+            fetch_x(it + 1 + AHEAD, full);
+            fetch_g(it + AHEAD, full);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const float xv = vF[r];
@@ -1216,7 +1243,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                 // Its fetch already asked for zeros (out-of-range offsets), but the sums of the
                 // whole launch should not hang on what a fetch that reads nothing leaves in LDS:
                 // a zero gradient here makes every product of the sweep zero.
-                if (!group_ok(R * it + r)) gr = 0.0f;
+                if (!full && !group_ok(R * it + r)) gr = 0.0f;
                 vF[r] = xv;
                 gv[r] = gr;
                 if constexpr (BIAS_SUM) {
@@ -1251,7 +1278,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
                     T done[R];
                     get_rows<T, R>(carry_buf, c.fA, done);
 #pragma unroll
-                    for (int r = 0; r < R; ++r) store_grad(R * (it - 1) + r, done[r]);
+                    for (int r = 0; r < R; ++r) store_grad(R * (it - 1) + r, done[r], full);
                 }
                 if constexpr (paired) {
                     const Pair v2 = buf[rdF];
@@ -1355,7 +1382,7 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if constexpr (Q::DEFER) carry[r] = gv[r];
-            else store_grad(R * it + r, gv[r]);
+            else store_grad(R * it + r, gv[r], full);
         }
         if constexpr (DIRECT) {
             if constexpr (!PREREAD) read_rows(it + 1, vF, gv);
@@ -1380,9 +1407,19 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         wait_rows_in_lds<0>();
         __syncthreads();
         read_rows(-1, vF, gv);
-        for (int it = -1; it < it_end; it += 2) {
-            iteration(std::integral_constant<int, 0>{}, it, vF, gv, carry, actP, actQ);
-            iteration(std::integral_constant<int, 1>{}, it + 1, vF, gv, carry, actQ, actP);
+        const std::false_type masked{};
+        const std::true_type unmasked{};
+        int it = -1;
+        iteration(std::integral_constant<int, 0>{}, masked, it, vF, gv, carry, actP, actQ);
+        iteration(std::integral_constant<int, 1>{}, masked, it + 1, vF, gv, carry, actQ, actP);
+        // iterations it, it + 1 are FULL when the furthest group they request exists in every slot
+        for (it = 1; it < it_end && (R * (it + 2 + AHEAD) + R) * SLOTS <= rows_valid; it += 2) {
+            iteration(std::integral_constant<int, 0>{}, unmasked, it, vF, gv, carry, actP, actQ);
+            iteration(std::integral_constant<int, 1>{}, unmasked, it + 1, vF, gv, carry, actQ, actP);
+        }
+        for (; it < it_end; it += 2) {
+            iteration(std::integral_constant<int, 0>{}, masked, it, vF, gv, carry, actP, actQ);
+            iteration(std::integral_constant<int, 1>{}, masked, it + 1, vF, gv, carry, actQ, actP);
         }
         wait_rows_in_lds<0>();  // requests past the last group (they fetch nothing)
     } else {
@@ -1393,12 +1430,12 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
             vF[0] = x0;
             gv[0] = gm;
             const T x1 = load_x(it + 2), gp = load_g(it + 1);
-            iteration(std::integral_constant<int, 0>{}, it, vF, gv, carry, actP, actQ);
+            iteration(std::integral_constant<int, 0>{}, std::false_type{}, it, vF, gv, carry, actP, actQ);
             x0 = load_x(it + 3);
             gm = load_g(it + 2);
             vF[0] = x1;
             gv[0] = gp;
-            iteration(std::integral_constant<int, 1>{}, it + 1, vF, gv, carry, actQ, actP);
+            iteration(std::integral_constant<int, 1>{}, std::false_type{}, it + 1, vF, gv, carry, actQ, actP);
         }
     }
 
