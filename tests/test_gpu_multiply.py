@@ -992,6 +992,9 @@ LONG_BASE4_CASES = [
     (np.complex64, 600, 1, 10, 2, None, None, False),
     (np.complex64, 13, 2, 11, 1, None, None, True),
     (np.complex64, 13, 1, 12, 2, None, None, False),
+    (np.float32, 5, 1, 16, 1, None, None, True),
+    (np.float32, 2, 1, 19, 1, None, None, True),
+    (np.complex64, 3, 1, 15, 1, None, None, False),
 ]
 
 
