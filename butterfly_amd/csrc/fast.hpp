@@ -1117,10 +1117,12 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     const int64_t x_col = view_col(a.x_view, col), g_col = view_col(a.g_view, col);
     const int x_thr = x_col >= 0 ? c.slot * x_row + (int)(x_col * a.x_view.se * EB) : kOob;
     const int g_thr = g_col >= 0 ? c.slot * g_row + (int)(g_col * a.g_view.se * EB) : kOob;
-    auto load_x = [&](int grp) {
+    auto load_x = [&](int grp, bool full = false) {
+        if (full) return buf_load<T>(x_rs, x_thr, grp * SLOTS * x_row);
         return buf_load<T>(x_rs, group_ok(grp) ? x_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * x_row);
     };
-    auto load_g = [&](int grp) {
+    auto load_g = [&](int grp, bool full = false) {
+        if (full) return buf_load<T>(g_rs, g_thr, grp * SLOTS * g_row);
         return buf_load<T>(g_rs, group_ok(grp) ? g_thr : kOob, (grp < 0 ? 0 : grp) * SLOTS * g_row);
     };
     // --- operand fetch, LDS flavour: lane l of wavefront w fetches element 64 w + l of the row
@@ -1426,16 +1428,38 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         // complex64: an iteration is long enough to cover the fetch, and four more registers
         // held across a whole iteration would not fit
         T x0 = load_x(0), gm = load_g(-1);
-        for (int it = -1; it < it_end; it += 2) {
+        if constexpr (NS >= 9) {
+            // (no second copy of the body for the passes that fill the register file)
+            for (int it = -1; it < it_end; it += 2) {
+                vF[0] = x0;
+                gv[0] = gm;
+                const T x1 = load_x(it + 2), gp = load_g(it + 1);
+                iteration(std::integral_constant<int, 0>{}, std::false_type{}, it, vF, gv, carry, actP, actQ);
+                x0 = load_x(it + 3);
+                gm = load_g(it + 2);
+                vF[0] = x1;
+                gv[0] = gp;
+                iteration(std::integral_constant<int, 1>{}, std::false_type{}, it + 1, vF, gv, carry, actQ, actP);
+            }
+        } else {
+        // a pair of iterations: FULL when every group it loads (up to it + 3) and stores exists in
+        // every row slot
+        auto pair = [&](int it, auto FULL) {
+            constexpr bool full = decltype(FULL)::value;
             vF[0] = x0;
             gv[0] = gm;
-            const T x1 = load_x(it + 2), gp = load_g(it + 1);
-            iteration(std::integral_constant<int, 0>{}, std::false_type{}, it, vF, gv, carry, actP, actQ);
-            x0 = load_x(it + 3);
-            gm = load_g(it + 2);
+            const T x1 = load_x(it + 2, full), gp = load_g(it + 1, full);
+            iteration(std::integral_constant<int, 0>{}, FULL, it, vF, gv, carry, actP, actQ);
+            x0 = load_x(it + 3, full);
+            gm = load_g(it + 2, full);
             vF[0] = x1;
             gv[0] = gp;
-            iteration(std::integral_constant<int, 1>{}, std::false_type{}, it + 1, vF, gv, carry, actQ, actP);
+            iteration(std::integral_constant<int, 1>{}, FULL, it + 1, vF, gv, carry, actQ, actP);
+        };
+        int it = -1;
+        pair(it, std::false_type{});
+        for (it = 1; it < it_end && (it + 4) * SLOTS <= rows_valid; it += 2) pair(it, std::true_type{});
+        for (; it < it_end; it += 2) pair(it, std::false_type{});
         }
     }
 

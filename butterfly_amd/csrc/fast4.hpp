@@ -225,6 +225,8 @@ __global__ __launch_bounds__(kFastThreads) void fast4_fw_kernel(Fast4Args a)
 
     float nxt[R];
     load_rows(0, nxt);
+    // (this loop keeps its range masks: it is bound by HBM, and a second, unmasked copy of the
+    // body measured slower)
     for (int grel = 0; grel < ng; grel += R) {
         float v[R];
 #pragma unroll
@@ -303,24 +305,28 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
         par ^= 1;
     };
     auto row_ok = [&](int grp) { return grp * SLOTS + c.slot < rows_valid; };
-    auto load_rows = [&](int grel, float (&x)[R], float (&g)[R]) {
+    auto load_rows = [&](int grel, float (&x)[R], float (&g)[R], bool full = false) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            x[r] = buf_load<float>(x_rs, row_ok(grel + r) ? x_thr : kOob, (grel + r) * SLOTS * x_row);
-            g[r] = buf_load<float>(g_rs, row_ok(grel + r) ? g_thr : kOob, (grel + r) * SLOTS * g_row);
+            const bool ok = full || row_ok(grel + r);
+            x[r] = buf_load<float>(x_rs, ok ? x_thr : kOob, (grel + r) * SLOTS * x_row);
+            g[r] = buf_load<float>(g_rs, ok ? g_thr : kOob, (grel + r) * SLOTS * g_row);
         }
     };
 
     float nx[R], ngr[R];
     load_rows(0, nx, ngr);
-    for (int grel = 0; grel < ng; grel += R) {
+    // FULL: the groups this iteration stores and the ones it prefetches exist for every row slot,
+    // so no access needs its range mask: all but the last iterations of a workgroup.
+    auto iteration = [&](int grel, auto FULL) {
+        constexpr bool full = decltype(FULL)::value;
         float v[R], gv[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             v[r] = nx[r];
             gv[r] = ngr[r];
         }
-        load_rows(grel + R, nx, ngr);
+        load_rows(grel + R, nx, ngr, full);
         float act[NS][R];
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
@@ -356,8 +362,7 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
                 const float xs = act[s][r];
                 if constexpr (KQ < 2) {
                     bw4_dpp<KQ>(acc[s], gv[r], xs, f.colm[s]);
-                    continue;
-                }
+                } else {
                 const float g1 = partner4<KQ, 1>(gv[r], lane);
                 const float g2 = partner4<KQ, 2>(gv[r], lane);
                 const float g3 = partner4<KQ, 3>(gv[r], lane);
@@ -370,13 +375,17 @@ __global__ __launch_bounds__(kFastThreads) void fast4_bw_kernel(Fast4Args a)
                 d = fmaf(f.colm[s][2], g2, d);
                 d = fmaf(f.colm[s][3], g3, d);
                 gv[r] = d;
+                }
             }
         });
         if constexpr (P::layout(0) != 0) transpose(gv, 0);
 #pragma unroll
         for (int r = 0; r < R; ++r)
-            buf_store(gi_rs, row_ok(grel + r) ? gi_thr : kOob, (grel + r) * SLOTS * gi_row, gv[r]);
-    }
+            buf_store(gi_rs, full || row_ok(grel + r) ? gi_thr : kOob, (grel + r) * SLOTS * gi_row, gv[r]);
+    };
+    int grel = 0;
+    for (; grel < ng && (grel + 2 * R) * SLOTS <= rows_valid; grel += R) iteration(grel, std::true_type{});
+    for (; grel < ng; grel += R) iteration(grel, std::false_type{});
 
     int t2 = t;
     asm volatile("" : "+v"(t2));
