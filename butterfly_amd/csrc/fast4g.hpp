@@ -264,24 +264,29 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_bw_kernel(Fast4GArgs a)
         par ^= 1;
     };
     auto row_ok = [&](int grp) { return grp * SLOTS + c.slot < rows_valid; };
-    auto load_rows = [&](int grel, T (&x)[R], T (&g)[R]) {
+    // (`full`: the caller knows that these row groups exist for every row slot of the workgroup)
+    auto load_rows = [&](int grel, T (&x)[R], T (&g)[R], bool full = false) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            x[r] = buf_load<T>(x_rs, row_ok(grel + r) ? x_thr : kOob, (grel + r) * SLOTS * x_row);
-            g[r] = buf_load<T>(g_rs, row_ok(grel + r) ? g_thr : kOob, (grel + r) * SLOTS * g_row);
+            const bool ok = full || row_ok(grel + r);
+            x[r] = buf_load<T>(x_rs, ok ? x_thr : kOob, (grel + r) * SLOTS * x_row);
+            g[r] = buf_load<T>(g_rs, ok ? g_thr : kOob, (grel + r) * SLOTS * g_row);
         }
     };
 
     T nx[R], ngr[R];
     load_rows(0, nx, ngr);
-    for (int grel = 0; grel < ng; grel += R) {
+    // FULL: the groups this iteration stores and the ones it prefetches exist for every row slot,
+    // so no access needs its range mask: all but the last iterations of a workgroup.
+    auto iteration = [&](int grel, auto FULL) {
+        constexpr bool full = decltype(FULL)::value;
         T v[R], gv[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             v[r] = nx[r];
             gv[r] = ngr[r];
         }
-        load_rows(grel + R, nx, ngr);
+        load_rows(grel + R, nx, ngr, full);
         T act[NS][R];
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
@@ -329,8 +334,11 @@ __global__ __launch_bounds__(kFastThreads) void fast4g_bw_kernel(Fast4GArgs a)
         if constexpr (P::layout(0) != 0) transpose(gv, 0);
 #pragma unroll
         for (int r = 0; r < R; ++r)
-            buf_store(gi_rs, row_ok(grel + r) ? gi_thr : kOob, (grel + r) * SLOTS * gi_row, gv[r]);
-    }
+            buf_store(gi_rs, full || row_ok(grel + r) ? gi_thr : kOob, (grel + r) * SLOTS * gi_row, gv[r]);
+    };
+    int grel = 0;
+    for (; grel < ng && (grel + 2 * R) * SLOTS <= rows_valid; grel += R) iteration(grel, std::true_type{});
+    for (; grel < ng; grel += R) iteration(grel, std::false_type{});
 
     // ---- partial sums of this workgroup, in the layout of the twiddle tensors
     int t2 = t;
