@@ -31,7 +31,7 @@ from .multiply_base4 import butterfly_multiply_base4  # noqa: E402
 from .butterfly import Butterfly, ButterflyBmm, ButterflyUnitary  # noqa: E402
 from .butterfly_base4 import ButterflyBase4  # noqa: E402
 from .graphed import GraphedStep  # noqa: E402
-from . import combine, complex_utils, diagonal, kops, legacy, multiply, multiply_base4, permutation, special  # noqa: E402,F401
+from . import combine, complex_utils, diagonal, kops, legacy, legacy_permutation, multiply, multiply_base4, permutation, special  # noqa: E402,F401
 
 __all__ = [
     "Butterfly",

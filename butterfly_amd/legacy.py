@@ -123,6 +123,40 @@ def _as_complex(t):
         return torch.view_as_complex(t.contiguous())
 
 
+# ---- helpers of butterfly/complex_utils.py and butterfly/utils.py on (..., 2) real pairs ------------
+
+def real_to_complex(X):
+    """(...) -> (..., 2) with zero imaginary parts (butterfly/complex_utils.py:40-47)."""
+    return torch.stack((X, torch.zeros_like(X)), dim=-1)
+
+
+def conjugate(X):
+    """(butterfly/complex_utils.py:50-75)"""
+    return torch.view_as_real(_as_complex(X).conj().resolve_conj())
+
+
+def complex_mul(X, Y):
+    """Elementwise product with broadcasting (butterfly/complex_utils.py:78-131)."""
+    shape = torch.broadcast_shapes(X.shape, Y.shape)
+    return torch.view_as_real(_as_complex(X.expand(shape)) * _as_complex(Y.expand(shape)))
+
+
+def complex_matmul(X, Y):
+    """(..., n, m, 2) x (..., m, p, 2) -> (..., n, p, 2) (butterfly/complex_utils.py:162-201)."""
+    return torch.view_as_real(_as_complex(X) @ _as_complex(Y))
+
+
+conjugate_torch = conjugate
+complex_mul_torch = complex_mul
+complex_matmul_torch = complex_matmul
+
+
+def bitreversal_permutation(n):
+    """numpy array: perm[i] = i with its log2(n) bits reversed (butterfly/utils.py:8-21)."""
+    from .permutation import bitreversal_permutation as table
+    return table(n)
+
+
 def _multiply(twiddle, input, increasing_stride):
     """twiddle (nstack, nblocks, log n, n / 2, 2, 2) in order of application (pairs of reals
     appended for complex), input (batch, nstack, n[, 2])."""
@@ -247,6 +281,65 @@ def butterfly_mult_factors(twiddle, input, increasing_stride=True, return_interm
         values.append(torch.einsum("srp,bgps->bgrs", f, pairs).reshape(-1, n))
     out = torch.stack(values)
     return torch.view_as_real(out) if cplx else out
+
+
+def butterfly_mult_dyadic_torch(twiddle, input, log_strides, return_intermediates=False):
+    """k factors with arbitrary strides, applied in the order given: twiddle
+    (nstack, k, n / 2, 2, 2[, 2]), factor i has stride 2^log_strides[i]; input
+    (batch, nstack, n[, 2]) (butterfly_multiply.py:733-772).  A debugging aid in the reference
+    and here: one PyTorch contraction per factor; with ``return_intermediates`` the input and
+    the value after every factor, stacked."""
+    cplx = input.dim() == 4
+    batch, nstack, n = input.shape[:3]
+    _log2(n)
+    if twiddle.shape[:5] != (nstack, len(log_strides), n // 2, 2, 2):
+        raise ValueError("twiddle must be (nstack, len(log_strides), n / 2, 2, 2) [+ (2,) if complex]")
+    x = _as_complex(input) if cplx else input
+    t = _as_complex(twiddle) if cplx else twiddle
+    values = [x]
+    for i, log_stride in enumerate(log_strides):
+        stride = 1 << log_stride
+        f = t[:, i].reshape(nstack, n // (2 * stride), stride, 2, 2)
+        pairs = values[-1].reshape(batch, nstack, n // (2 * stride), 2, stride)
+        values.append(torch.einsum("sglrp,bsgpl->bsgrl", f, pairs).reshape(batch, nstack, n))
+    out = torch.stack(values) if return_intermediates else values[-1]
+    return torch.view_as_real(out) if cplx else out
+
+
+def butterfly_mult_untied_torch(twiddle, input, increasing_stride=True, return_intermediates=False):
+    """``butterfly_mult_untied`` under the name of the reference's plain-PyTorch version
+    (butterfly_multiply.py:126-165); ``return_intermediates`` walks the factors one by one."""
+    if not return_intermediates:
+        return butterfly_mult_untied(twiddle, input, increasing_stride)
+    m = _log2(input.shape[2])
+    order = list(range(m)) if increasing_stride else list(range(m - 1, -1, -1))
+    return butterfly_mult_dyadic_torch(twiddle[:, order], input, order, True)
+
+
+def butterfly_mult_torch(twiddle, input, increasing_stride=True, return_intermediates=False):
+    """Tied weights (butterfly_multiply.py:43-81)."""
+    m = _log2(input.shape[2])
+    return butterfly_mult_untied_torch(twiddle[:, _tied_index(m, twiddle.device)], input, increasing_stride,
+                                       return_intermediates)
+
+
+def butterfly_mult_conv2d_torch(twiddle, input, kernel_size, padding, increasing_stride=True,
+                                return_intermediates=False):
+    """(butterfly_multiply.py:491-521)"""
+    return butterfly_mult_untied_torch(twiddle, _conv2d_patches(twiddle, input, kernel_size, padding),
+                                       increasing_stride, return_intermediates)
+
+
+def bbt_mult_untied_torch(twiddle, input):
+    """(butterfly_multiply.py:377-386)"""
+    return bbt_mult_untied(twiddle, input, fast=False)
+
+
+# The remaining plain-PyTorch twins of the reference compute what the functions above compute.
+butterfly_ortho_mult_tied_torch = butterfly_ortho_mult_tied
+butterfly_ortho_mult_untied_torch = butterfly_ortho_mult_untied
+bbt_ortho_mult_untied_torch = bbt_ortho_mult_untied
+bbt_mult_conv2d_torch = bbt_mult_conv2d
 
 
 def _tied_blocks(factors, m):

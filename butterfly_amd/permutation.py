@@ -42,6 +42,10 @@ class FixedPermutation(nn.Module):
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         return index_last_dim(input, self.permutation)
 
+    def to_butterfly(self, complex=False, increasing_stride=False):
+        """A two-block Butterfly with the same effect (torch_butterfly/permutation.py:77-78)."""
+        return perm2butterfly(self.permutation, complex, increasing_stride)
+
     def column_table(self, n: int, scatter: bool) -> torch.Tensor:
         """The permutation as the int32 table of n entries that the multiply operators fold
         into their first read (scatter False: entry c = permutation[c]) or their last write
@@ -142,18 +146,19 @@ def wavelet_permutation(n, pytorch_format=False):
 
 
 def perm_vec_to_mat(p, left=False):
-    """0/1 matrix of the permutation vector p: (M x)[i] = x[p[i]] (left=False), i.e.
-    M[i, p[i]] = 1; left=True gives the transpose (x M convention)."""
+    """0/1 matrix M of the permutation vector p.  left=False (right-multiplication format):
+    M[p[i], i] = 1, so the row vector x M equals x[p]; left=True gives the transpose, for which
+    M x equals x[p] (reference: torch_butterfly/permutation.py:98-108)."""
     p = np.asarray(p)
     m = np.zeros((p.size, p.size), dtype=np.int64)
-    m[np.arange(p.size), p] = 1
+    m[p, np.arange(p.size)] = 1
     return m.T if left else m
 
 
 def perm_mat_to_vec(m, left=False):
-    """Inverse of perm_vec_to_mat."""
+    """Inverse of perm_vec_to_mat (reference: torch_butterfly/permutation.py:111-118)."""
     m = np.asarray(m)
-    return np.argmax(m.T if left else m, axis=1)
+    return np.argmax(m if left else m.T, axis=1)
 
 
 def is_2x2_block_diag(mat):
@@ -193,6 +198,204 @@ def matrix_to_butterfly_factor(mat, log_k, pytorch_format=False, check_input=Fal
     rows = np.stack((pos, pos + half), -1)                       # (n/2, 2)
     tw = mat[rows[:, :, None], rows[:, None, :]]                 # tw[i, r, c] = mat[rows[i, r], rows[i, c]]
     return torch.from_numpy(np.ascontiguousarray(tw)) if pytorch_format else tw
+
+
+def half_balance(v, return_swap_locations=False):
+    """Swaps between positions i and i + n/2 after which the first half of the vector v (values
+    distinct modulo n, n even) holds every residue modulo n/2 once, and so does the second half.
+    Returns ``(perm, v[perm])`` with perm the product of the swaps, or ``(low positions of
+    the swapped pairs, v[perm])``.
+
+    Two positions that hold the same residue must end in different halves, and so must the
+    two positions of a pair (i, i + n/2): following "same residue" and "same pair" alternately
+    from any position walks a closed loop of even length, and keeping the first element where
+    it is fixes every other choice on the loop.  (The reference builds the same loops as an
+    edge-oriented graph, torch_butterfly/permutation.py:176-228; which of the two valid
+    settings a loop gets is not part of the contract.)"""
+    v = np.asarray(v)
+    n = v.size
+    if n % 2:
+        raise ValueError("the vector must have even length")
+    nh = n // 2
+    residue = v % nh
+    order = np.argsort(residue, kind="stable")          # positions by residue: two per residue
+    if not np.array_equal(residue[order], np.repeat(np.arange(nh), 2)):
+        raise ValueError("every residue modulo n/2 must occur exactly twice")
+    rival = np.empty(n, dtype=np.int64)
+    rival[order[0::2]] = order[1::2]
+    rival[order[1::2]] = order[0::2]
+    swapped = np.zeros(nh, dtype=bool)
+    seen = np.zeros(n, dtype=bool)
+    for start in range(n):
+        if seen[start]:
+            continue
+        pos = start
+        half = int(pos >= nh)                           # the half this element ends in: it stays put
+        while not seen[pos]:
+            seen[pos] = True
+            other = rival[pos]                          # same residue: must end in the other half
+            seen[other] = True
+            swapped[other % nh] = (int(other >= nh) == half)
+            pos = (other + nh) % n                      # its pair partner ends in `half` again
+    low = np.flatnonzero(swapped)
+    perm = np.arange(n)
+    perm[low], perm[low + nh] = low + nh, low
+    return (low.tolist() if return_swap_locations else perm), v[perm]
+
+
+def modular_balance(v):
+    """The swaps that make the permutation vector v modular-balanced, level by level: blocks of
+    n, n/2, ..., 2 consecutive positions are half-balanced in turn.  Returns ``(perms, w)`` with
+    ``w = v[perms[0]][perms[1]]...`` and w modular-balanced
+    (reference: torch_butterfly/permutation.py:231-252)."""
+    v = np.asarray(v)
+    n = v.size
+    perms = []
+    t = n
+    while t >= 2:
+        level = np.concatenate([half_balance(v[base:base + t])[0] + base for base in range(0, n, t)])
+        v = v[level]
+        perms.append(level)
+        t //= 2
+    return perms, v
+
+
+def is_modular_balanced(perm):
+    """True when every aligned block of j = 2, 4, ..., n consecutive entries of the permutation
+    (vector, or matrix in right-multiplication format) holds j different residues modulo j
+    (reference: torch_butterfly/permutation.py:255-269)."""
+    perm = np.asarray(perm)
+    if perm.ndim > 1:
+        perm = perm_mat_to_vec(perm)
+    n = perm.size
+    log_n = int(n).bit_length() - 1
+    if n != 1 << log_n:
+        raise ValueError("the size must be a power of 2")
+    for k in range(1, log_n + 1):
+        j = 1 << k
+        residues = np.sort((perm % j).reshape(n // j, j), axis=1)
+        if not np.array_equal(residues, np.broadcast_to(np.arange(j), (n // j, j))):
+            return False
+    return True
+
+
+def _balanced_factor_vectors(w):
+    """w modular-balanced (right-multiplication vector, x L = x[w]): vectors f_n, f_{n/2}, ...,
+    f_2 with w = f_n[f_{n/2}[...[f_2]]], f_k moving entries by 0 or +-k/2 inside blocks of k."""
+    n = w.size
+    if n == 2:
+        return [w.copy()]
+    nh = n // 2
+    inner = np.concatenate((w[:nh] % nh, w[nh:] % nh + nh))    # what is left inside the two halves
+    outer = w[invert(inner)]                                   # w = outer[inner]
+    first = _balanced_factor_vectors(inner[:nh])
+    second = _balanced_factor_vectors(inner[nh:] - nh)
+    return [outer] + [np.concatenate((a, b + nh)) for a, b in zip(first, second)]
+
+
+def modular_balanced_to_butterfly_factor(L):
+    """Butterfly factors (permutation matrices in right-multiplication format, block sizes
+    n, n/2, ..., 2) whose product in that order is the modular-balanced permutation L (vector or
+    matrix in right-multiplication format; reference: torch_butterfly/permutation.py:272-301)."""
+    L = np.asarray(L)
+    w = L if L.ndim == 1 else perm_mat_to_vec(L)
+    if not is_modular_balanced(w):
+        raise ValueError("the permutation is not modular-balanced")
+    return [perm_vec_to_mat(f) for f in _balanced_factor_vectors(w.astype(np.int64))]
+
+
+def _butterfly_from_gathers(block0, block1, n, size, complex):
+    """Two-block Butterfly (decreasing stride first) from its factors given as gathers
+    (x -> x[f]): block0 with block sizes n, n/2, ..., 2 and block1 with 2, 4, ..., n."""
+    from .butterfly import Butterfly  # (butterfly.py does not import this module)
+    log_n = n.bit_length() - 1
+    planes = []
+    for factors, sizes in ((block0, range(log_n, 0, -1)), (block1, range(1, log_n + 1))):
+        planes.append(torch.stack([matrix_to_butterfly_factor(perm_vec_to_mat(f, left=True), log_k, pytorch_format=True)
+                                   for f, log_k in zip(factors, sizes)]))
+    dtype = torch.get_default_dtype()
+    if complex:
+        from .complex_utils import real_dtype_to_complex
+        dtype = real_dtype_to_complex[dtype]
+    twiddle = torch.stack(planes).unsqueeze(0).to(dtype)
+    b = Butterfly(n, n, bias=False, complex=complex, increasing_stride=False, init=twiddle, nblocks=2)
+    b.in_size = b.out_size = size
+    return b
+
+
+def _padded_permutation(v):
+    if isinstance(v, torch.Tensor):
+        v = v.detach().cpu().numpy()
+    v = np.asarray(v, dtype=np.int64)
+    size = v.size
+    if size < 2:
+        raise ValueError("the permutation must have at least 2 elements")
+    if not np.array_equal(np.sort(v), np.arange(size)):
+        raise ValueError("v is not a permutation")
+    n = 1 << int(size - 1).bit_length()
+    return np.concatenate((v, np.arange(size, n, dtype=np.int64))), size, n
+
+
+def _to_increasing_stride(b, size):
+    """The decreasing-stride Butterfly of br[v[br]] read with increasing stride and its pairs
+    in bit-reversed order is a Butterfly of v (torch_butterfly/permutation.py:322-330)."""
+    from .butterfly import Butterfly
+    n = b.twiddle.shape[3] * 2
+    pairs = bitreversal_permutation(n // 2, pytorch_format=True)
+    out = Butterfly(n, n, bias=False, complex=b.twiddle.is_complex(), increasing_stride=True,
+                    init=b.twiddle.detach()[:, :, :, pairs].clone(), nblocks=2)
+    out.in_size = out.out_size = size
+    return out
+
+
+def perm2butterfly_slow(v, complex=False, increasing_stride=False):
+    """``b(x) == x[..., v]`` as perm2butterfly, built the way the existence proof goes: the
+    level-by-level swaps of ``modular_balance`` are the first block, the factors of the
+    modular-balanced rest the second (reference: torch_butterfly/permutation.py:304-348)."""
+    full, size, n = _padded_permutation(v)
+    if increasing_stride:
+        br = bitreversal_permutation(n)
+        return _to_increasing_stride(perm2butterfly_slow(br[full[br]], complex, False), size)
+    # invert(full) = w[s_last[...[s_first]]] with s the swaps, so
+    # x[full] = x[s_first]...[s_last][invert(w)] and invert(w) = invert(f_2)[...[invert(f_n)]].
+    swaps, w = modular_balance(invert(full))
+    block1 = [invert(f) for f in reversed(_balanced_factor_vectors(w))]
+    return _butterfly_from_gathers(swaps, block1, n, size, complex)
+
+
+def swap_locations_to_twiddle_factor(n, swap_locations):
+    """(n/2, 2, 2) factor of straight switches, crossed at the given pair indices."""
+    twiddle = torch.eye(2).repeat(n // 2, 1, 1)
+    twiddle[torch.as_tensor(np.asarray(swap_locations, dtype=np.int64))] = torch.tensor([[0.0, 1.0], [1.0, 0.0]])
+    return twiddle
+
+
+def outer_twiddle_factors(v):
+    """One level of the permutation-to-butterfly recursion for a batch of permutations v
+    (batch, size), left-multiplication format: the switch factor applied first
+    (batch * size/2, 2, 2), the one applied last (same shape), and the 2 * batch permutations
+    of size/2 left between them (reference: torch_butterfly/permutation.py:358-392)."""
+    v = np.asarray(v)
+    batch, size = v.shape
+    if size < 2:
+        raise ValueError("size must be at least 2")
+    half = size // 2
+    first, rest = [], []
+    for row in v:
+        low, balanced = half_balance(invert(row), return_swap_locations=True)
+        first.append(swap_locations_to_twiddle_factor(size, low))
+        rest.append(invert(balanced))
+    rest = np.stack(rest)                                     # rest[b][c]: source of output c
+    crossed = rest[:, :half] >= half                          # output pair c takes its low element from the top half
+    rows, cols = np.nonzero(crossed)
+    last = swap_locations_to_twiddle_factor(batch * size, rows * half + cols)
+    lo, hi = rest[:, :half].copy(), rest[:, half:].copy()
+    lo[crossed], hi[crossed] = rest[:, half:][crossed], rest[:, :half][crossed]
+    inner = np.concatenate((lo, hi), axis=1) % half
+    inner = inner.reshape(batch * 2, half)
+    if not np.array_equal(np.sort(inner, axis=1), np.broadcast_to(np.arange(half), inner.shape)):
+        raise AssertionError("the inner vectors are not permutations")
+    return torch.cat(first), last, inner
 
 
 def _benes_switches(perm, log_n, increasing_stride):

@@ -380,3 +380,26 @@ def test_mult_factors(n, cplx):
             value = lo.factor_apply(lo.tied_expand(tied[None], log_stride, n), log_stride, value)
             assert rel_err(back(steps[i + 1]), value[:, 0]) < FW_TOL
         assert rel_err(back(steps[-1]), y_ref[:, 0]) < FW_TOL
+
+
+def test_learnable_permutation_on_the_device():
+    """The relaxed permutation product is plain tensor work: on the device it gives what it
+    gives on the host (which tests/test_host.py holds against dense matrices), gradients included."""
+    from butterfly_amd import legacy_permutation as lp
+    torch.manual_seed(11)
+    for n, share, inc, tail in [(64, False, False, ()), (256, True, True, (2,)), (1024, False, True, ())]:
+        say("learnable permutation", n, share, inc, tail)
+        host = lp.Permutation(n, share_logit=share, increasing_stride=inc).double()
+        onboard = lp.Permutation(n, share_logit=share, increasing_stride=inc).double().cuda()
+        with torch.no_grad():
+            onboard.logit.copy_(host.logit)
+        x = torch.randn(33, n, *tail, dtype=torch.float64)
+        g = torch.randn(33, n, *tail, dtype=torch.float64)
+        xh, xd = x.clone().requires_grad_(), x.cuda().requires_grad_()
+        yh, yd = host(xh), onboard(xd)
+        gh = torch.autograd.grad(yh, (xh, host.logit), g)
+        gd = torch.autograd.grad(yd, (xd, onboard.logit), g.cuda())
+        assert torch.allclose(yd.cpu(), yh, atol=1e-12)
+        for a, b in zip(gd, gh):
+            assert torch.allclose(a.cpu(), b, atol=1e-10)
+        assert onboard.argmax().cpu().tolist() == host.argmax().tolist()

@@ -265,7 +265,9 @@ def test_permutation_routing_and_helpers_on_the_host():
     assert np.array_equal(permutation.wavelet_permutation(2), [0, 1])
     m = permutation.perm_vec_to_mat(np.array([2, 0, 3, 1]))
     x = np.arange(4) * 10
-    assert np.array_equal(m @ x, x[[2, 0, 3, 1]])
+    assert np.array_equal(m, [[0, 1, 0, 0], [0, 0, 0, 1], [1, 0, 0, 0], [0, 0, 1, 0]])   # M[p[i], i] = 1
+    assert np.array_equal(x @ m, x[[2, 0, 3, 1]])
+    assert np.array_equal(permutation.perm_vec_to_mat(np.array([2, 0, 3, 1]), left=True) @ x, x[[2, 0, 3, 1]])
     assert np.array_equal(permutation.perm_mat_to_vec(m), [2, 0, 3, 1])
     assert np.array_equal(permutation.perm_mat_to_vec(permutation.perm_vec_to_mat([2, 0, 3, 1], left=True), left=True),
                           [2, 0, 3, 1])
@@ -447,3 +449,273 @@ def test_modules_run_on_host_tensors():
     assert torch.allclose(f(z), torch.fft.fft(z, norm="ortho"), atol=1e-5)
     dbl = butterfly_amd.Butterfly(16, 16, bias=False).double()
     assert dbl(torch.randn(2, 16, dtype=torch.float64)).dtype == torch.float64
+
+
+def _soft_factor_matrix(n, stride, p, q0, q1):
+    """Dense matrix of one relaxed permutation factor, entry by entry from its definition:
+    inside every group of 2 * stride elements, with weight p the even elements are dealt to the
+    first half and the odd ones to the second; then half a is reversed with weight q_a."""
+    deal = np.zeros((n, n))
+    flip = np.zeros((n, n))
+    q = (q0, q1)
+    for base in range(0, n, 2 * stride):
+        for a in range(2):
+            for j in range(stride):
+                row = base + a * stride + j
+                deal[row, row] += 1 - p
+                deal[row, base + 2 * j + a] += p
+                flip[row, row] += 1 - q[a]
+                flip[row, base + a * stride + stride - 1 - j] += q[a]
+    return flip @ deal
+
+
+@pytest.mark.parametrize("inc", [False, True])
+def test_legacy_learnable_permutation(inc):
+    """The relaxed permutation product against dense matrices built from the definition of a
+    factor (output, gradients of input and probabilities), its hard limits against known
+    permutations, and the module's bookkeeping (reference: butterfly/permutation.py,
+    butterfly/permutation_multiply.py:18-52)."""
+    from butterfly_amd import legacy_permutation as lp
+    rng = np.random.default_rng(77 + inc)
+    n, B = 32, 5
+    m = 5
+    prob = rng.uniform(0.05, 0.95, (m - 1, 3))
+    order = list(range(1, m)) if inc else list(range(1, m))[::-1]
+    dense = np.eye(n)
+    for k in order:
+        dense = _soft_factor_matrix(n, 1 << k, *prob[k - 1]) @ dense
+    x = rng.standard_normal((B, n))
+    g = rng.standard_normal((B, n))
+    pt = torch.tensor(prob, requires_grad=True)
+    xt = torch.tensor(x, requires_grad=True)
+    y = lp.permutation_mult(pt, xt, increasing_stride=inc)
+    assert np.allclose(y.detach().numpy(), x @ dense.T, atol=1e-12)
+    d_p, d_x = torch.autograd.grad(y, (pt, xt), torch.tensor(g))
+    assert np.allclose(d_x.numpy(), g @ dense, atol=1e-12)
+    eps = 1e-6
+    for k, c in [(0, 0), (1, 2), (m - 2, 1)]:
+        moved = prob.copy()
+        moved[k, c] += eps
+        dense2 = np.eye(n)
+        for kk in order:
+            dense2 = _soft_factor_matrix(n, 1 << kk, *moved[kk - 1]) @ dense2
+        fd = np.sum(g * (x @ (dense2 - dense).T)) / eps
+        assert abs(d_p[k, c].item() - fd) < 1e-4 * max(1.0, abs(fd))
+    # complex rows are pairs moved together; intermediates start at the input and end at the output
+    xc = torch.tensor(rng.standard_normal((B, n, 2)))
+    yc = lp.permutation_mult(pt.detach(), xc, increasing_stride=inc, return_intermediates=True)
+    assert yc.shape == (m, B, n, 2) and torch.equal(yc[0], xc)
+    for part in range(2):
+        assert np.allclose(yc[-1][..., part].numpy(), xc[..., part].numpy() @ dense.T, atol=1e-12)
+    # hard limits: dealing inside a group of 2^b elements reads position p from p with its low b bits
+    # rotated left by one; widest group first, the rotations compose to the bit reversal
+    hard = torch.zeros(m - 1, 3, dtype=torch.float64)
+    hard[:, 0] = 1
+    idx = torch.arange(n, dtype=torch.float64).unsqueeze(0)
+
+    def rotl(p, b):
+        low = p & ((1 << b) - 1)
+        return (p - low) | ((low << 1) & ((1 << b) - 1)) | (low >> (b - 1))
+    want = []
+    for p in range(n):
+        src = p
+        for b in (range(2, m + 1) if not inc else range(m, 1, -1)):   # last applied factor first
+            src = rotl(src, b)
+        want.append(src)
+    if not inc:
+        assert want == [int(format(i, f"0{m}b")[::-1], 2) for i in range(n)]
+    assert lp.permutation_mult(hard, idx, increasing_stride=inc).squeeze(0).long().tolist() == want
+    # one factor over the whole row: reverse the second half only
+    out = lp.permutation_mult_single(torch.tensor([0.0, 0.0, 1.0], dtype=torch.float64), idx).squeeze(0).long().tolist()
+    assert out == list(range(n // 2)) + list(range(n - 1, n // 2 - 1, -1))
+    # modules
+    torch.manual_seed(5)
+    for share in (False, True):
+        mod = lp.Permutation(n, share_logit=share, increasing_stride=inc)
+        assert tuple(mod.logit.shape) == ((3,) if share else (m - 1, 3))
+        with torch.no_grad():
+            mod.logit.copy_(torch.where(mod.logit > 0, 30.0, -30.0))   # saturated: a permutation up to 1e-12
+        p = mod.argmax()
+        assert sorted(p.tolist()) == list(range(n))
+        xr = torch.randn(B, n)
+        assert torch.allclose(mod(xr), lp.FixedPermutation(p)(xr), atol=1e-5)
+        assert torch.allclose(mod(xr), xr[:, p], atol=1e-5)
+    fac = lp.PermutationFactor(n)
+    with torch.no_grad():
+        fac.logit.copy_(torch.tensor([30.0, -30.0, 30.0]))
+    assert torch.allclose(fac(xr), xr[:, fac.argmax()], atol=1e-5)
+    assert fac.argmax().tolist() == list(range(0, n, 2)) + list(range(n - 1, 0, -2))
+    with pytest.raises(ValueError):
+        lp.Permutation(24)
+    with pytest.raises(ValueError):
+        lp.permutation_mult(torch.rand(5, 3), torch.randn(2, 32))
+
+
+def test_permutation_factorisation_following_the_existence_proof():
+    """half_balance / modular_balance / modular_balanced_to_butterfly_factor /
+    perm2butterfly_slow / outer_twiddle_factors: the properties the reference's own tests state
+    (tests/test_permutation.py:34-67), which define these functions up to the free choice inside
+    every loop of swaps."""
+    import butterfly_amd
+    from butterfly_amd import permutation as P
+    rng = np.random.default_rng(21)
+    for n in (2, 4, 16, 64, 256):
+        for _ in range(10):
+            v = rng.permutation(n)
+            perm, balanced = P.half_balance(v)
+            assert np.array_equal(balanced, v[perm]) and np.array_equal(perm[perm], np.arange(n))
+            assert np.all(np.abs(perm - np.arange(n)) % (n // 2) == 0)           # only i <-> i + n/2
+            for half in (balanced[:n // 2], balanced[n // 2:]):
+                assert np.array_equal(np.sort(half % (n // 2)), np.arange(n // 2))
+            low, balanced2 = P.half_balance(v, return_swap_locations=True)
+            assert np.array_equal(balanced2, balanced) and sorted(low) == list(np.flatnonzero(perm[:n // 2] != np.arange(n // 2)))
+            perms, w = P.modular_balance(v)
+            assert len(perms) == n.bit_length() - 1 and P.is_modular_balanced(w)
+            assert P.is_modular_balanced(P.perm_vec_to_mat(w))
+            v2 = v
+            for p in perms:
+                v2 = v2[p]
+            assert np.array_equal(v2, w)
+            back = w
+            for p in reversed(perms):
+                back = back[P.invert(p)]
+            assert np.array_equal(back, v)
+            mat = P.perm_vec_to_mat(v)
+            for p in perms:                                   # x M_v M_p = x[v][p]
+                mat = mat @ P.perm_vec_to_mat(p)
+            assert np.array_equal(mat, P.perm_vec_to_mat(w))
+            factors = P.modular_balanced_to_butterfly_factor(w)
+            prod = np.eye(n, dtype=np.int64)
+            for i, f in enumerate(factors):
+                assert P.is_butterfly_factor(f, n >> i)
+                prod = prod @ f
+            assert np.array_equal(prod, P.perm_vec_to_mat(w))
+            assert all(np.array_equal(a, b) for a, b in
+                       zip(factors, P.modular_balanced_to_butterfly_factor(P.perm_vec_to_mat(w))))
+    assert not P.is_modular_balanced(np.array([0, 2, 1, 3]))
+    assert P.is_modular_balanced(np.array([0, 1, 2, 3])) and P.is_modular_balanced(np.array([3, 0, 1, 2]))
+    with pytest.raises(ValueError):
+        P.modular_balanced_to_butterfly_factor(np.array([0, 2, 1, 3]))
+    for n in (2, 13, 38):
+        for inc in (False, True):
+            for cplx in (False, True):
+                for _ in range(5):
+                    v = torch.from_numpy(rng.permutation(n))
+                    b = P.perm2butterfly_slow(v, cplx, inc)
+                    assert (b.in_size, b.out_size, b.nblocks, b.increasing_stride) == (n, n, 2, inc)
+                    x = torch.arange(n, dtype=torch.float32).to(torch.complex64 if cplx else torch.float32)
+                    assert torch.equal(b(x), x[v])
+    # the level-by-level recursion: first switch column, last switch column, two half-size problems
+    for log_n in (1, 3, 6):
+        n = 1 << log_n
+        v = rng.permutation(n)
+        cur = v[None]
+        first, last = [], []
+        for level in range(log_n):
+            f, l, cur = P.outer_twiddle_factors(cur)
+            assert f.shape == l.shape == (n // 2, 2, 2) and cur.shape == (2 << level, n >> (level + 1))
+            first.append(f)
+            last.append(l)
+        twiddle = torch.stack([torch.stack(first), torch.stack(last).flip([0])]).unsqueeze(0)
+        b = butterfly_amd.Butterfly(n, n, bias=False, increasing_stride=False, init=twiddle, nblocks=2)
+        x = torch.arange(n, dtype=torch.float32)
+        assert torch.equal(b(x), x[torch.from_numpy(v)])
+    v = torch.from_numpy(rng.permutation(11))
+    x = torch.randn(3, 11)
+    assert torch.equal(P.FixedPermutation(v).to_butterfly(increasing_stride=True)(x), x[:, v])
+    t = P.swap_locations_to_twiddle_factor(8, [1, 3])
+    assert t.shape == (4, 2, 2) and torch.equal(t[0], torch.eye(2)) and torch.equal(t[1], torch.tensor([[0.0, 1.0], [1.0, 0.0]]))
+
+
+def test_complex_helpers():
+    """complex_matmul and index_last_dim as the reference's tests/test_complex_utils.py checks them
+    (against broadcast-multiply-and-sum, gradients included), the four-real-products form, and
+    ComplexLinear against the product written out."""
+    from butterfly_amd import complex_utils as cu
+    torch.manual_seed(3)
+    X = torch.randn(3, 5, 64, 16, dtype=torch.complex64, requires_grad=True)
+    Y = torch.randn(3, 5, 16, 32, dtype=torch.complex64, requires_grad=True)
+    want = (X.unsqueeze(-1) * Y.unsqueeze(-3)).sum(dim=-2)
+    g = torch.randn_like(want)
+    for product in (cu.complex_matmul, cu.complex_matmul_torch):
+        got = product(X, Y)
+        assert torch.allclose(got, want, 1e-3, 1e-5)
+        for a, b in zip(torch.autograd.grad(got, (X, Y), g), torch.autograd.grad(want, (X, Y), g, retain_graph=True)):
+            assert torch.allclose(a, b, 1e-3, 1e-4)
+    p = torch.randperm(17)
+    x = torch.randn(2, 3, 17, requires_grad=True)
+    out = cu.index_last_dim(x, p)
+    gg = torch.randn_like(out)
+    assert torch.equal(out, x[..., p])
+    assert torch.equal(torch.autograd.grad(out, x, gg)[0], torch.autograd.grad(x[..., p], x, gg)[0])
+    assert cu.IndexLastDim.apply(x, p).equal(out) and cu.Real2ComplexFn.apply(x).dtype == torch.complex64
+    lin = cu.ComplexLinear(12, 7)
+    assert lin.weight.shape == (7, 12) and lin.weight.dtype == torch.complex64 and lin.bias.shape == (7,)
+    assert lin.weight.abs().max() <= 1 / 12 ** 0.5 + 1e-6
+    z = torch.randn(4, 5, 12, dtype=torch.complex64)
+    assert torch.allclose(lin(z), (z.unsqueeze(-2) * lin.weight).sum(-1) + lin.bias, 1e-4, 1e-5)
+    assert cu.ComplexLinear(12, 7, bias=False).bias is None
+
+
+def test_legacy_plain_pytorch_twins_and_dyadic_multiply():
+    """The legacy package's `*_torch` names and `butterfly_mult_dyadic_torch` (factors with
+    arbitrary strides in the order given), on host tensors, against the numpy restatement's
+    single-factor step applied literally, intermediates included."""
+    from butterfly_amd import legacy
+    from oracle import legacy_oracle as lo
+    rng = np.random.default_rng(31)
+    n, m, S, B = 16, 4, 2, 5
+    for cplx in (False, True):
+        def to_t(a):
+            return torch.from_numpy(np.stack((a.real, a.imag), -1).astype(np.float32)) if cplx else torch.from_numpy(a.astype(np.float32))
+
+        def to_n(t):
+            a = t.detach().numpy().astype(np.float64)
+            return a[..., 0] + 1j * a[..., 1] if cplx else a
+
+        def rnd(shape):
+            a = rng.standard_normal(shape)
+            return a + 1j * rng.standard_normal(shape) if cplx else a
+        x = rnd((B, S, n))
+        strides = [2, 0, 3, 3, 1]
+        tw = rnd((S, len(strides), n // 2, 2, 2)) / np.sqrt(2)
+        steps = legacy.butterfly_mult_dyadic_torch(to_t(tw), to_t(x), strides, return_intermediates=True)
+        value = x
+        assert rel_err(to_n(steps[0]), value) < 1e-6
+        for i, ls in enumerate(strides):
+            value = lo.factor_apply(tw[:, i], ls, value)
+            assert rel_err(to_n(steps[i + 1]), value) < 1e-5
+        assert rel_err(to_n(legacy.butterfly_mult_dyadic_torch(to_t(tw), to_t(x), strides)), value) < 1e-5
+        for inc in (True, False):
+            untied = rnd((S, m, n // 2, 2, 2)) / np.sqrt(2)
+            y_ref = lo.butterfly_mult_untied(untied, x, inc)
+            assert rel_err(to_n(legacy.butterfly_mult_untied_torch(to_t(untied), to_t(x), inc)), y_ref) < 1e-5
+            trail = legacy.butterfly_mult_untied_torch(to_t(untied), to_t(x), inc, return_intermediates=True)
+            assert trail.shape[0] == m + 1 and rel_err(to_n(trail[-1]), y_ref) < 1e-5
+            value = x
+            for i, ls in enumerate(range(m) if inc else range(m - 1, -1, -1)):
+                value = lo.factor_apply(untied[:, ls], ls, value)
+                assert rel_err(to_n(trail[i + 1]), value) < 1e-5
+            tied = rnd((S, n - 1, 2, 2)) / np.sqrt(2)
+            y_ref = lo.butterfly_mult(tied, x, inc)
+            assert rel_err(to_n(legacy.butterfly_mult_torch(to_t(tied), to_t(x), inc)), y_ref) < 1e-5
+            assert rel_err(to_n(legacy.butterfly_mult_torch(to_t(tied), to_t(x), inc, True)[-1]), y_ref) < 1e-5
+    bbt = rng.standard_normal((S, 2 * m, n // 2, 2, 2)) / np.sqrt(2)
+    xr = rng.standard_normal((B, S, n))
+    got = legacy.bbt_mult_untied_torch(torch.from_numpy(bbt).float(), torch.from_numpy(xr).float())
+    assert rel_err(got.numpy().astype(np.float64), lo.bbt_mult_untied(bbt, xr)) < 1e-5
+    assert legacy.butterfly_ortho_mult_tied_torch is legacy.butterfly_ortho_mult_tied
+    with pytest.raises(ValueError):
+        legacy.butterfly_mult_dyadic_torch(torch.zeros(S, 2, n // 2, 2, 2), torch.zeros(B, S, n), [0, 1, 2])
+
+
+def test_legacy_pair_helpers():
+    from butterfly_amd import legacy
+    torch.manual_seed(2)
+    a, b = torch.randn(3, 4, 5, 2), torch.randn(3, 5, 6, 2)
+    ac, bc = torch.view_as_complex(a), torch.view_as_complex(b)
+    assert torch.allclose(torch.view_as_complex(legacy.complex_matmul(a, b)), ac @ bc, atol=1e-5)
+    assert torch.allclose(torch.view_as_complex(legacy.complex_mul(a[:, :, :1], a)), ac[:, :, :1] * ac, atol=1e-6)
+    assert torch.equal(legacy.conjugate(a), a * torch.tensor([1.0, -1.0]))
+    assert torch.equal(legacy.real_to_complex(a[..., 0])[..., 1], torch.zeros(3, 4, 5))
+    assert legacy.bitreversal_permutation(8).tolist() == [0, 4, 2, 6, 1, 5, 3, 7]
