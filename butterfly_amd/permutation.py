@@ -162,13 +162,16 @@ def perm_mat_to_vec(m, left=False):
 
 
 def is_2x2_block_diag(mat):
-    """True when mat is block diagonal with 2x2 blocks."""
+    """True when each of the four quadrants of the (even-sized, square) matrix is diagonal, i.e.
+    entry (i, j) vanishes unless i - j is a multiple of half the size: a 2 x 2 grid of diagonal
+    blocks, the shape of one butterfly factor over the whole matrix
+    (reference: torch_butterfly/permutation.py:121-130)."""
     mat = np.asarray(mat)
     n = mat.shape[0]
     if mat.shape != (n, n) or n % 2:
         return False
-    mask = np.kron(np.eye(n // 2, dtype=bool), np.ones((2, 2), dtype=bool))
-    return not np.any(mat[~mask])
+    i, j = np.indices((n, n))
+    return not np.any(mat[(i - j) % (n // 2) != 0])
 
 
 def is_butterfly_factor(mat, k):

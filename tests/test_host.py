@@ -271,7 +271,10 @@ def test_permutation_routing_and_helpers_on_the_host():
     assert np.array_equal(permutation.perm_mat_to_vec(m), [2, 0, 3, 1])
     assert np.array_equal(permutation.perm_mat_to_vec(permutation.perm_vec_to_mat([2, 0, 3, 1], left=True), left=True),
                           [2, 0, 3, 1])
-    assert permutation.is_2x2_block_diag(np.kron(np.eye(3), np.ones((2, 2))))
+    # four diagonal quadrants (one butterfly factor over the whole matrix), not 2 x 2 blocks on the diagonal
+    assert permutation.is_2x2_block_diag(np.kron(np.ones((2, 2)), np.diag([1.0, 2.0, 3.0])))
+    assert permutation.is_2x2_block_diag(np.ones((2, 2)))
+    assert not permutation.is_2x2_block_diag(np.kron(np.eye(3), np.ones((2, 2))))
     assert not permutation.is_2x2_block_diag(np.ones((4, 4)))
     with pytest.raises(ValueError):
         permutation.perm2butterfly(np.array([0, 0, 1]))
