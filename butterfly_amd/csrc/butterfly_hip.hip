@@ -1177,6 +1177,11 @@ BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false, b
     const size_t row_bytes = (size_t)n * e;
     const Schedule sc = make_schedule(p, base4);
     pl.nstages = sc.per * sc.nblocks;
+    if (p->batch == 0 || p->nstacks == 0) {
+        // no rows: nothing is launched but the zero fill of d_twiddle, no workspace, any row length
+        pl.fits = true;
+        return pl;
+    }
     if (fast4_ok(p, base4, true)) {
         pl.fits = true;
         pl.fast4 = true;
@@ -1328,6 +1333,10 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
     const Schedule sc = make_schedule(p, base4);
     const int64_t n = (int64_t)1 << p->log_n;
     const bool permuted = in_perm || out_index;
+    if (p->batch == 0 || p->nstacks == 0) {
+        // no rows: d_input is empty and every d_twiddle entry is an empty sum, whatever the row length
+        return launch_reduce(p, sc, 0, sc.per * sc.nblocks, 0, nullptr, 4 * n, d_tw2, d_tw4, stream);
+    }
     const BwPlan pl = plan_bw(p, base4, saved != nullptr, permuted);
     if (!pl.fits)
         return fail(BF_ERR_UNSUPPORTED, "n = %lld does not fit in LDS for the backward pass", (long long)n);

@@ -468,6 +468,69 @@ def test_operators_match_oracle_and_autograd():
         assert rel_err(y2.cpu().numpy(), oracle.butterfly_fw(tv_np, x, True)) < FW_TOL
 
 
+@pytest.mark.parametrize("L,nb", [(3, 1), (10, 2), (12, 2), (14, 1)])
+def test_empty_batch(L, nb):
+    """No rows at all: outputs and input gradients are empty tensors of the right shape, every
+    d_twiddle (and d_bias) entry is an empty sum, i.e. exactly zero -- for every kernel family the
+    size would otherwise pick, float and complex64, base 2, base 4, with bias and column tables."""
+    import butterfly_amd  # noqa: F401
+    ops = torch.ops.torch_butterfly
+    n = 1 << L
+    S, O = 2, n - 3
+    for tdt in (torch.float32, torch.complex64):
+        say("empty batch", L, nb, tdt)
+        # scratch the allocator's blocks so that an output nobody writes does not read as zero
+        junk = torch.full((S * nb * L * n * 8,), 7.0, device="cuda")
+        del junk
+        tw = torch.randn(S, nb, L, n // 2, 2, 2, dtype=tdt, device="cuda", requires_grad=True)
+        x = torch.empty(0, S, n, dtype=tdt, device="cuda", requires_grad=True)
+        g = torch.empty(0, S, O, dtype=tdt, device="cuda")
+        y = ops.butterfly_multiply_fw(tw, x, True, O)
+        assert y.shape == (0, S, O)
+        dtw, dx = ops.butterfly_multiply_bw(tw, x, torch.empty(0, S, n, dtype=tdt, device="cuda"), True)
+        assert dx.shape == (0, S, n) and dtw.shape == tw.shape and not dtw.any()
+        y = ops.butterfly_multiply(tw, x, False, O)
+        dtw, dx = torch.autograd.grad(y, (tw, x), g)
+        assert y.shape == (0, S, O) and dx.shape == (0, S, n) and not dtw.any()
+        bias = torch.randn(S, O, dtype=tdt, device="cuda", requires_grad=True)
+        table = torch.randperm(n, device="cuda").int()
+        y = ops.butterfly_multiply_perm(tw, x, table, None, bias, True, O)
+        dtw, dx, db = torch.autograd.grad(y, (tw, x, bias), g)
+        assert y.shape == (0, S, O) and dx.shape == (0, S, n) and not dtw.any() and not db.any()
+        if L <= 12:
+            tw4 = torch.randn(S, nb, L // 2, n // 4, 4, 4, dtype=tdt, device="cuda", requires_grad=True)
+            tw2 = torch.randn(S, nb, L % 2, n // 2, 2, 2, dtype=tdt, device="cuda", requires_grad=True)
+            y = ops.butterfly_multiply_base4(tw4, tw2, x, True, O)
+            d4, d2, dx = torch.autograd.grad(y, (tw4, tw2, x), g, allow_unused=True)
+            assert y.shape == (0, S, O) and dx.shape == (0, S, n) and not d4.any()
+            assert d2 is None or not d2.any()
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("L,nb", [(3, 1), (10, 2), (12, 2)])
+def test_empty_rows(L, nb):
+    """Rows of no input columns (everything is padding: the output is the bias or zero, d_input is
+    empty, d_twiddle zero) and of no output columns (empty output; a zero gradient flows back)."""
+    import butterfly_amd  # noqa: F401
+    ops = torch.ops.torch_butterfly
+    n = 1 << L
+    B, S = 37, 2
+    for tdt in (torch.float32, torch.complex64):
+        say("empty rows", L, nb, tdt)
+        tw = torch.randn(S, nb, L, n // 2, 2, 2, dtype=tdt, device="cuda", requires_grad=True)
+        x0 = torch.empty(B, S, 0, dtype=tdt, device="cuda", requires_grad=True)
+        g = torch.randn(B, S, n, dtype=tdt, device="cuda")
+        y = ops.butterfly_multiply(tw, x0, True, None)
+        dtw, dx = torch.autograd.grad(y, (tw, x0), g)
+        assert y.shape == (B, S, n) and not y.any() and dx.shape == (B, S, 0) and not dtw.any()
+        x = torch.randn(B, S, n, dtype=tdt, device="cuda", requires_grad=True)
+        y = ops.butterfly_multiply(tw, x, False, 0)
+        assert y.shape == (B, S, 0)
+        dtw, dx = torch.autograd.grad(y, (tw, x), torch.empty(B, S, 0, dtype=tdt, device="cuda"))
+        assert dx.shape == (B, S, n) and not dx.any() and not dtw.any()
+    torch.cuda.synchronize()
+
+
 def test_operator_errors():
     import butterfly_amd  # noqa: F401
     ops = torch.ops.torch_butterfly
