@@ -49,7 +49,7 @@ def scale_twiddle(twiddle, increasing_stride, in_scale=None, out_scale=None):
         return torch.ops.torch_butterfly.butterfly_scale_twiddle(twiddle, cast(in_scale), cast(out_scale),
                                                                  increasing_stride)
     stacks, nblocks, log_n, half = twiddle.shape[:4]
-    n = 2 * half
+    n = 1 << log_n
 
     def pairs(vec, rows, stride):
         # (rows, n) entries by element -> (rows, n/2, 2) by pair index and position in the pair
@@ -202,14 +202,14 @@ class Butterfly(nn.Module):
         else:
             inc = self.increasing_stride
         if in_perm is not None or out_index is not None:
-            cols = output_size if output_size is not None else twiddle.shape[3] * 2
+            cols = output_size if output_size is not None else 1 << twiddle.shape[2]
             bias = None if self.bias is None else self.bias_rows(cols, subtwiddle)
             x = butterfly_multiply_perm(twiddle, x, in_perm, out_index, bias, inc, output_size)
         elif self.bias is None:
             x = butterfly_multiply(twiddle, x, inc, output_size)
         else:
             # the kernel that writes the output adds the bias, laid out as (stacks, columns)
-            cols = output_size if output_size is not None else twiddle.shape[3] * 2
+            cols = output_size if output_size is not None else 1 << twiddle.shape[2]
             x = butterfly_multiply_bias(twiddle, x, self.bias_rows(cols, subtwiddle), inc, output_size)
         return self.post_process(input, x, out_size=x.size(-1) if subtwiddle else None, add_bias=False)
 

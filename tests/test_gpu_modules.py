@@ -232,3 +232,69 @@ def test_butterfly_bmm_equals_loop_over_layers():
                         ht, hb = torch.autograd.grad(layer(x[:, i]), (layer.twiddle, layer.bias), g[:, i])
                         assert close(gtw[i * bmm.nstacks:(i + 1) * bmm.nstacks], ht, atol=1e-4)
                         assert close(gb[i], hb, atol=1e-4)
+
+
+@pytest.mark.parametrize("chunk", range(3))
+def test_random_layer_configurations_match_the_host_path(chunk):
+    """Seeded random layers (sizes that need padding, trimming and several stacks, real and
+    complex, 1-3 blocks, both stride orders, bias or none; Butterfly, ButterflyBase4, ButterflyBmm,
+    ButterflyUnitary) with random forward flags: output and every gradient on the device against
+    the same layer on host tensors, whose multiply is the operators' host loop (bit-exact with the
+    reference's CPU path).  The device takes the fused routes (bias added by the kernel, d_bias
+    summed by the backward kernel), the host the composed ones."""
+    import copy
+    import butterfly_amd as bfa
+    rng = np.random.default_rng(4400 + chunk)
+    torch.manual_seed(4400 + chunk)
+    for i in range(25):
+        kind = str(rng.choice(["butterfly", "butterfly", "base4", "bmm", "unitary"]))
+        in_size = int(rng.choice([1, 2, 3, 7, 16, 33, 100, 512, 1000, 1500]))
+        out_size = int(rng.choice([1, 5, 16, 40, 130, 700, 2100]))
+        cplx = bool(rng.random() < 0.4) or kind == "unitary"
+        inc = bool(rng.random() < 0.5)
+        nblocks = int(rng.choice([1, 2, 3]))
+        bias = bool(rng.random() < 0.6)
+        lead = [(4,), (3, 5), (2, 1, 3)][int(rng.integers(0, 3))]
+        flags = {}
+        if kind in ("butterfly", "unitary") and rng.random() < 0.4:
+            flags = {"conjugate": bool(rng.random() < 0.5)}
+            if in_size == out_size or rng.random() < 0.3:
+                flags["transpose"] = True
+        say(f"layer case {chunk}.{i}:", kind, in_size, out_size, cplx, inc, nblocks, bias, lead, flags)
+        if kind == "butterfly":
+            init = str(rng.choice(["randn", "ortho"]))
+            host = bfa.Butterfly(in_size, out_size, bias, cplx, inc, init, nblocks)
+        elif kind == "base4":
+            host = bfa.ButterflyBase4(in_size, out_size, bias, cplx, inc, "randn", nblocks)
+        elif kind == "bmm":
+            host = bfa.ButterflyBmm(in_size, out_size, 3, bias, cplx, inc, nblocks=nblocks)
+            lead = lead + (3,)
+        else:
+            host = bfa.ButterflyUnitary(in_size, out_size, bias, inc, nblocks)
+        dev_layer = copy.deepcopy(host).cuda()
+        dtype = torch.complex64 if cplx else torch.float32
+        width = in_size
+        if flags.get("transpose"):
+            # the transposed layer maps the n-padded output side back: feed what its matrix accepts
+            width = min(out_size, host.n) if host.nstacks == 1 else None
+        if width is None:
+            continue
+        x = torch.randn(*lead, width, dtype=dtype)
+        xh, xd = x.clone().requires_grad_(), x.cuda().requires_grad_()
+        yh, yd = host(xh, **flags), dev_layer(xd, **flags)
+        assert yd.shape == yh.shape
+        g = torch.randn_like(yh)
+        wrt_h = (xh,) + tuple(host.parameters())
+        wrt_d = (xd,) + tuple(dev_layer.parameters())
+        gh = torch.autograd.grad(yh, wrt_h, g, allow_unused=True)
+        gd = torch.autograd.grad(yd, wrt_d, g.cuda(), allow_unused=True)
+        scale = max(1.0, yh.abs().max().item())
+        assert (yd.cpu() - yh).abs().max().item() <= 1e-4 * scale
+        for a, b in zip(gd, gh):
+            # (an empty parameter -- the twiddle of a layer of size 1, the 4x4 factors of a layer of
+            # size 2 -- may come back as an empty gradient on one side and as None on the other)
+            assert (a is None or a.numel() == 0) == (b is None or b.numel() == 0)
+            if a is not None and b is not None:
+                assert a.shape == b.shape
+                if b.numel():
+                    assert (a.cpu() - b).abs().max().item() <= 2e-4 * max(1.0, b.abs().max().item())

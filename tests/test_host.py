@@ -722,3 +722,19 @@ def test_legacy_pair_helpers():
     assert torch.equal(legacy.conjugate(a), a * torch.tensor([1.0, -1.0]))
     assert torch.equal(legacy.real_to_complex(a[..., 0])[..., 1], torch.zeros(3, 4, 5))
     assert legacy.bitreversal_permutation(8).tolist() == [0, 4, 2, 6, 1, 5, 3, 7]
+
+
+def test_layers_of_size_one():
+    """in_size = 1 is n = 1, log n = 0: no factors at all, every stack copies its input and adds
+    its bias.  (The bias used to be laid out over 2 * (n / 2) = 0 columns there.)"""
+    import butterfly_amd
+    torch.manual_seed(0)
+    x = torch.randn(4, 1)
+    b = butterfly_amd.Butterfly(1, 5, bias=True)
+    assert b.twiddle.numel() == 0 and b.nstacks == 5
+    assert torch.allclose(b(x), x.expand(4, 5) + b.bias)
+    bmm = butterfly_amd.ButterflyBmm(1, 5, 3, bias=True, nblocks=2)
+    xs = torch.randn(4, 3, 1)
+    assert torch.allclose(bmm(xs), xs.expand(4, 3, 5) + bmm.bias)
+    g = torch.autograd.grad(bmm(xs).sum(), bmm.bias)[0]
+    assert torch.equal(g, torch.full_like(g, 4.0))
