@@ -4,6 +4,7 @@ eager calls give for the operands then in place (bit for bit: the kernels' summa
 not depend on how they are launched)."""
 import sys
 
+import numpy as np
 import pytest
 import torch
 
@@ -81,3 +82,32 @@ def test_forward_only_and_argument_checks():
         step(x, x)
     with pytest.raises(ValueError, match="device tensor"):
         butterfly_amd.GraphedStep(layer, x.cpu())
+
+
+def test_random_zoo_layers_replay_bit_identically():
+    """Forty seeded random layers (every `special` constructor, the legacy layer, KOP2d; the
+    generator of test_gpu_zoo_random.py) recorded as one graph each: three replays with fresh
+    inputs and output gradients, each bit-identical to the eager forward + autograd backward."""
+    import butterfly_amd as bfa
+    from test_gpu_zoo_random import draw_layer
+    for seed in range(8100, 8140):
+        rng = np.random.default_rng(seed)
+        torch.manual_seed(seed)
+        kind, layer, x = draw_layer(rng)
+        print("graphed zoo case", seed, kind, tuple(x.shape), flush=True)
+        layer, x = layer.cuda(), x.cuda()
+        params = [p for p in layer.parameters() if p.requires_grad]
+        with torch.no_grad():
+            g = torch.randn_like(layer(x))
+        step = bfa.GraphedStep(layer, x, g, params)
+        for _ in range(3):
+            x2, g2 = torch.randn_like(x), torch.randn_like(g)
+            y, grads = step(x2, g2)
+            y, grads = y.clone(), [t.clone() for t in grads]
+            torch.cuda.synchronize()
+            xe = x2.clone().requires_grad_()
+            ye = layer(xe)
+            want = torch.autograd.grad(ye, [xe] + params, g2)
+            assert torch.equal(y, ye.detach())
+            for a, b in zip(grads, want):
+                assert torch.equal(a, b)

@@ -71,11 +71,12 @@ def draw_layer(rng):
         m = special.wavelet_haar(p2, with_perm=f()); x = torch.randn(5, p2)
     elif kind == "legacy":
         param = str(rng.choice(["regular", "regular", "ortho", "odo", "obdobt", "ds", "logit", "ortho2"]))
-        cplx = f() and param == "regular"
         nblocks = int(rng.choice([0, 1, 2])) if param in ("regular", "ortho", "odo", "obdobt") else 0
         if param in ("odo", "obdobt"):
             nblocks = max(nblocks, 1)
-        tied = f() and nblocks == 0          # B B^T blocks exist for untied weights only
+        # B B^T blocks exist for untied real weights only
+        tied = f() and nblocks == 0
+        cplx = f() and param == "regular" and nblocks == 0
         in_size, out_size = int(rng.choice([4, 7, 16, 100, 512])), int(rng.choice([3, 16, 40, 700]))
         m = legacy.Butterfly(in_size, out_size, bias=f(), complex=cplx, tied_weight=tied, increasing_stride=f(),
                              ortho_init=f(), param=param, nblocks=nblocks, expansion=int(rng.choice([1, 1, 2])),
