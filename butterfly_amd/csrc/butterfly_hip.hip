@@ -12,6 +12,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <utility>
 
 #include "common.hpp"
 #include "generic.hpp"
@@ -119,28 +120,35 @@ View dense_view(int64_t nstacks, int64_t n)
     return v;
 }
 
-// ---- one-time kernel attributes ---------------------------------------------------------
+// ---- kernel attributes, once per device ---------------------------------------------------
+//
+// The LDS fallback kernels ask for more dynamic LDS than the default limit; that permission is a
+// property of the function on one device, so it is set the first time a call runs on a device.
 
-std::once_flag g_attr_once;
-hipError_t g_attr_status = hipSuccess;
-
-void set_attributes()
-{
-    auto set = [](const void *fn, size_t bytes) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-        if (e != hipSuccess && g_attr_status == hipSuccess) g_attr_status = e;
-    };
-    set(reinterpret_cast<const void *>(&generic_fw_kernel<float>), kGenericFwLds);
-    set(reinterpret_cast<const void *>(&generic_fw_kernel<float2>), kGenericFwLds);
-    set(reinterpret_cast<const void *>(&generic_bw_kernel<float>), kGenericBwLds);
-    set(reinterpret_cast<const void *>(&generic_bw_kernel<float2>), kGenericBwLds);
-}
+constexpr int kMaxDevices = 64;
+std::mutex g_device_mutex;
+bool g_attr_done[kMaxDevices];
 
 int ensure_attributes()
 {
-    std::call_once(g_attr_once, set_attributes);
-    if (g_attr_status != hipSuccess)
-        return fail(BF_ERR_HIP, "hipFuncSetAttribute failed: %s", hipGetErrorString(g_attr_status));
+    int device = -1;
+    BF_HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices)
+        return fail(BF_ERR_UNSUPPORTED, "device ordinal %d is outside the %d the library keeps state for", device,
+                    kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_device_mutex);
+    if (g_attr_done[device]) return BF_OK;
+    const std::pair<const void *, size_t> wanted[] = {
+        {reinterpret_cast<const void *>(&generic_fw_kernel<float>), kGenericFwLds},
+        {reinterpret_cast<const void *>(&generic_fw_kernel<float2>), kGenericFwLds},
+        {reinterpret_cast<const void *>(&generic_bw_kernel<float>), kGenericBwLds},
+        {reinterpret_cast<const void *>(&generic_bw_kernel<float2>), kGenericBwLds},
+    };
+    for (const auto &w : wanted) {
+        const hipError_t e = hipFuncSetAttribute(w.first, hipFuncAttributeMaxDynamicSharedMemorySize, (int)w.second);
+        if (e != hipSuccess) return fail(BF_ERR_HIP, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+    }
+    g_attr_done[device] = true;
     return BF_OK;
 }
 
@@ -148,8 +156,6 @@ int ensure_attributes()
 // kernels (one workgroup per compute unit), the partial areas and the measured crossovers are
 // sized from it.  Host-only queries on a machine without a device plan for an MI355X (256).
 constexpr int kDefaultNumCU = 256;
-constexpr int kMaxDevices = 64;
-std::mutex g_device_mutex;
 int g_num_cu[kMaxDevices];
 
 int num_cu()
