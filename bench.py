@@ -27,6 +27,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+VALU_PEAK_TFLOPS = 157.3   # MI355X fp32 vector / matrix peak
 HBM_PEAK_GBS = 8000.0
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_all_configs.md")
 KERNEL_SOURCES = os.path.join(ROOT, "butterfly_amd", "csrc")
@@ -142,6 +143,16 @@ def algorithmic_bytes(c):
     fw = 2 * row * c["batch"] + twiddle            # read input, write output, read twiddle
     bw = 3 * row * c["batch"] + 2 * twiddle        # read input + grad, write d_input; twiddle in, d_twiddle out
     return fw, (bw if c["bw"] else 0)
+
+
+def algorithmic_flops(c):
+    """Floating-point operations of one step, counted as the algorithm's multiply-adds (2 flops
+    each): 2 per element and 2x2 stage in each sweep (4 per 4x4 stage, which stands for two),
+    4 times that for complex64; sweeps = forward, and for the backward call the replay, the
+    input gradient and the factor gradient."""
+    n = 1 << c["log_n"]
+    per_sweep = c["nstacks"] * n * c["nblocks"] * c["log_n"] * 2 * (4 if c["cplx"] else 1)
+    return 2.0 * per_sweep * c["batch"] * (4 if c["bw"] else 1)
 
 
 def cpu_baseline(name, c):
@@ -415,6 +426,12 @@ def main():
                      "traffic": None if args.graph else measured_traffic(args.config)},
         "graphed": bool(args.graph),
     }
+    # second roofline of the path: the same step against the fp32 vector rate (no MFMA: the
+    # factors are 2x2 / 4x4 blocks, not a dense contraction)
+    flops = algorithmic_flops(dict(c, bw=c["bw"] or c.get("graphed_bw", False)))
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    line["valu"] = {"achieved": tflops, "peak": VALU_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / VALU_PEAK_TFLOPS,
+                    "flops_per_step": flops}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.config, c)
     print(json.dumps(line), flush=True)
