@@ -1,0 +1,25 @@
+"""The C ABI without PyTorch: tests/c_abi/abi_check.cpp is a plain C++ program (hipMalloc, the
+null stream, the library's workspace queries) that links libbutterfly_hip.so and checks float,
+complex64 and base-4 calls against the CPU restatement.  It is built with the other native code
+(`__graft_entry__.build()` / `python tests/c_abi/build.py`) and run here as a child process."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+BINARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_abi", "abi_check.out")
+
+
+def test_c_abi_from_plain_cxx():
+    if not os.path.isfile(BINARY):
+        pytest.fail("tests/c_abi/abi_check.out is not built: run python tests/c_abi/build.py")
+    run = subprocess.run([BINARY], capture_output=True, text=True, timeout=300)
+    print(run.stdout, run.stderr, flush=True)
+    assert run.returncode == 0, run.stdout[-2000:]
+    lines = run.stdout.splitlines()
+    cases = [line for line in lines if line.startswith("base-")]
+    assert len(cases) == 8 and all(line.endswith(" ok") for line in cases)
+    assert lines[-1] == "all cases ok"
+    assert any(line.startswith("output_size > n: rc -1") for line in lines)
