@@ -507,7 +507,9 @@ int launch_span(bool cplx, const Pass &q, bool backward, bool two_rows, const Fa
     case HH * 3 + 2: ok = launch_span_t<HH, 2>(cplx, backward, two_rows, fw, bw, grid, stream); break;
     bool ok = false;
     switch (q.H * 3 + q.mode) {
+#ifndef BF_DEV_SUBSET
         BF_SPAN_CASES(1) BF_SPAN_CASES(2) BF_SPAN_CASES(3) BF_SPAN_CASES(4) BF_SPAN_CASES(5) BF_SPAN_CASES(6)
+#endif
         default: break;
     }
 #undef BF_SPAN_CASES
@@ -519,14 +521,23 @@ int launch_span(bool cplx, const Pass &q, bool backward, bool two_rows, const Fa
     do {                                                                                 \
         const int key_ = (Q).L * 4 + ((Q).NB - 1) * 2 + ((Q).inc ? 1 : 0);               \
         switch (key_) {                                                                  \
-            BF_FAST_CASES(FN, 1, __VA_ARGS__) BF_FAST_CASES(FN, 2, __VA_ARGS__)          \
-            BF_FAST_CASES(FN, 3, __VA_ARGS__) BF_FAST_CASES(FN, 4, __VA_ARGS__)          \
-            BF_FAST_CASES(FN, 5, __VA_ARGS__) BF_FAST_CASES(FN, 6, __VA_ARGS__)          \
-            BF_FAST_CASES(FN, 7, __VA_ARGS__) BF_FAST_CASES(FN, 8, __VA_ARGS__)          \
-            BF_FAST_CASES(FN, 9, __VA_ARGS__) BF_FAST_CASES(FN, 10, __VA_ARGS__)         \
+            BF_FAST_SHORT_CASES(FN, __VA_ARGS__) BF_FAST_CASES(FN, 10, __VA_ARGS__)      \
             default: return fail(BF_ERR_UNSUPPORTED, "no fast kernel for this shape");   \
         }                                                                                \
     } while (0)
+// BF_DEV_SUBSET (development builds only): instantiate nothing but the kernels of 1024-element
+// float / complex64 rows, so that a variant of those compiles in a fraction of the time; every
+// other shape answers BF_ERR_UNSUPPORTED.  The shipped library is built without it.
+#ifdef BF_DEV_SUBSET
+#define BF_FAST_SHORT_CASES(FN, ...)
+#else
+#define BF_FAST_SHORT_CASES(FN, ...)                                                     \
+    BF_FAST_CASES(FN, 1, __VA_ARGS__) BF_FAST_CASES(FN, 2, __VA_ARGS__)                  \
+    BF_FAST_CASES(FN, 3, __VA_ARGS__) BF_FAST_CASES(FN, 4, __VA_ARGS__)                  \
+    BF_FAST_CASES(FN, 5, __VA_ARGS__) BF_FAST_CASES(FN, 6, __VA_ARGS__)                  \
+    BF_FAST_CASES(FN, 7, __VA_ARGS__) BF_FAST_CASES(FN, 8, __VA_ARGS__)                  \
+    BF_FAST_CASES(FN, 9, __VA_ARGS__)
+#endif
 #define BF_FAST_CASES(FN, LL, ...)                              \
     case LL * 4 + 0: FN<LL, 1, false>(__VA_ARGS__); break;      \
     case LL * 4 + 1: FN<LL, 1, true>(__VA_ARGS__); break;       \
@@ -576,12 +587,17 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
             const dim3 grid((unsigned)g.nwg, (unsigned)p->nstacks, 1);
             const dim3 block(kFastThreads);
             const bool cplx = p->dtype == BF_C64;
+#ifdef BF_DEV_SUBSET
+            (void)cplx; (void)grid; (void)block; (void)a;
+            return fail(BF_ERR_UNSUPPORTED, "development subset: no whole-block forward kernels");
+#else
             if (q.L == 12 && q.inc) hipLaunchKernelGGL((wide_fw_kernel<float, 12, true>), grid, block, 0, stream, a);
             else if (q.L == 12) hipLaunchKernelGGL((wide_fw_kernel<float, 12, false>), grid, block, 0, stream, a);
             else if (cplx && q.inc) hipLaunchKernelGGL((wide_fw_kernel<float2, 11, true>), grid, block, 0, stream, a);
             else if (cplx) hipLaunchKernelGGL((wide_fw_kernel<float2, 11, false>), grid, block, 0, stream, a);
             else if (q.inc) hipLaunchKernelGGL((wide_fw_kernel<float, 11, true>), grid, block, 0, stream, a);
             else hipLaunchKernelGGL((wide_fw_kernel<float, 11, false>), grid, block, 0, stream, a);
+#endif
             BF_HIP_CHECK(hipGetLastError());
         } else {
             const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), fw_rows(p), kFastFwWgPerCu,
@@ -661,6 +677,7 @@ void launch_fast4_t(bool backward, const Fast4Args &a, dim3 grid, hipStream_t st
 int launch_fast4(int L, bool inc, bool backward, const Fast4Args &a, dim3 grid, hipStream_t stream)
 {
     switch (L * 2 + (inc ? 1 : 0)) {
+#ifndef BF_DEV_SUBSET
         case 2 * 2 + 0: launch_fast4_t<2, false>(backward, a, grid, stream); break;
         case 2 * 2 + 1: launch_fast4_t<2, true>(backward, a, grid, stream); break;
         case 4 * 2 + 0: launch_fast4_t<4, false>(backward, a, grid, stream); break;
@@ -671,6 +688,7 @@ int launch_fast4(int L, bool inc, bool backward, const Fast4Args &a, dim3 grid, 
         case 8 * 2 + 1: launch_fast4_t<8, true>(backward, a, grid, stream); break;
         case 10 * 2 + 0: launch_fast4_t<10, false>(backward, a, grid, stream); break;
         case 10 * 2 + 1: launch_fast4_t<10, true>(backward, a, grid, stream); break;
+#endif
         default: return fail(BF_ERR_UNSUPPORTED, "no base-4 kernel for this shape");
     }
     BF_HIP_CHECK(hipGetLastError());
@@ -698,12 +716,16 @@ int launch_fast4g(bool cplx, int L, bool inc, bool backward, const Fast4GArgs &a
     case LL * 2 + 1: launch_fast4g_t<float2, LL, true>(backward, a, grid, stream); break;
     if (cplx) {
         switch (L * 2 + (inc ? 1 : 0)) {
+#ifndef BF_DEV_SUBSET
             BF_C4G(2) BF_C4G(3) BF_C4G(4) BF_C4G(5) BF_C4G(6) BF_C4G(7) BF_C4G(8)
+#endif
             default: return fail(BF_ERR_UNSUPPORTED, "no base-4 kernel for this shape");
         }
     } else {
         switch (L * 2 + (inc ? 1 : 0)) {
+#ifndef BF_DEV_SUBSET
             BF_F4G(3) BF_F4G(5) BF_F4G(7) BF_F4G(9) BF_F4G(10)
+#endif
             default: return fail(BF_ERR_UNSUPPORTED, "no base-4 kernel for this shape");
         }
     }

@@ -1005,6 +1005,19 @@ __device__ __forceinline__ void store_pair(float2 *p, float2 a, float2 b)
     *reinterpret_cast<float4 *>(p) = make_float4(a.x, a.y, b.x, b.y);
 }
 
+__device__ __forceinline__ void load_pair(const float *p, float &a, float &b)
+{
+    const float2 v = *reinterpret_cast<const float2 *>(p);
+    a = v.x;
+    b = v.y;
+}
+__device__ __forceinline__ void load_pair(const float2 *p, float2 &a, float2 &b)
+{
+    const float4 v = *reinterpret_cast<const float4 *>(p);
+    a = make_float2(v.x, v.y);
+    b = make_float2(v.z, v.w);
+}
+
 // The R values a thread holds for one walk (one per row group in flight) as one LDS access.
 template <typename T, int R>
 __device__ __forceinline__ void put_rows(T *base, int idx, const T (&v)[R])
@@ -1403,8 +1416,10 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
 #pragma unroll
     for (int r = 0; r < R; ++r) carry[r] = vF[r] = gv[r] = zero_of(T());
     const int nit = (ng + R - 1) / R;
-    // with a deferred closing transpose one more (empty) iteration flushes the last groups
+    // (rows in registers: with a deferred closing transpose one more, empty, iteration flushes the
+    // last groups; the LDS flavour flushes them on its own behind the loop)
     const int it_end = Q::DEFER ? nit + 1 : nit;
+    int flush_it = 0;
     if constexpr (DIRECT) {
         wait_rows_in_lds<0>();
         __syncthreads();
@@ -1415,15 +1430,16 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         iteration(std::integral_constant<int, 0>{}, masked, it, vF, gv, carry, actP, actQ);
         iteration(std::integral_constant<int, 1>{}, masked, it + 1, vF, gv, carry, actQ, actP);
         // iterations it, it + 1 are FULL when the furthest group they request exists in every slot
-        for (it = 1; it < it_end && (R * (it + 2 + AHEAD) + R) * SLOTS <= rows_valid; it += 2) {
+        for (it = 1; it < nit && (R * (it + 2 + AHEAD) + R) * SLOTS <= rows_valid; it += 2) {
             iteration(std::integral_constant<int, 0>{}, unmasked, it, vF, gv, carry, actP, actQ);
             iteration(std::integral_constant<int, 1>{}, unmasked, it + 1, vF, gv, carry, actQ, actP);
         }
-        for (; it < it_end; it += 2) {
+        for (; it < nit; it += 2) {
             iteration(std::integral_constant<int, 0>{}, masked, it, vF, gv, carry, actP, actQ);
             iteration(std::integral_constant<int, 1>{}, masked, it + 1, vF, gv, carry, actQ, actP);
         }
         wait_rows_in_lds<0>();  // requests past the last group (they fetch nothing)
+        flush_it = it - 1;   // the last iteration that ran (it may lie past the last group)
     } else {
         // complex64: an iteration is long enough to cover the fetch, and four more registers
         // held across a whole iteration would not fit
@@ -1468,6 +1484,18 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     int t2 = t;
     asm volatile("" : "+v"(t2));
     const FastCoords c2 = fast_coords<L>(t2);
+    if constexpr (DIRECT && Q::DEFER) {
+        // The input gradient of the last iteration is still in layout B in `carry`: the closing
+        // transposition on its own, through the half of the carry buffer that the next iteration
+        // would have used (last touched two barriers ago).
+        T *carry_buf = lds_carry + (flush_it & 1) * R * kFastRowWords;
+        put_rows<T, R>(carry_buf, c2.fB, carry);
+        __syncthreads();
+        T done[R];
+        get_rows<T, R>(carry_buf, c2.fA, done);
+#pragma unroll
+        for (int r = 0; r < R; ++r) store_grad(R * flush_it + r, done[r]);
+    }
     if constexpr (BIAS_SUM) {
         if (bias_on) {
             const int64_t bcol = P::column(chunk, Q::SB ? c2.eB : c2.eA, a.low_bits);
@@ -1481,21 +1509,52 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
     T *part = reinterpret_cast<T *>(a.partial) + ((int64_t)blockIdx.x * gridDim.y + stack) * NS * a.partial_slot +
               P::pair_base(chunk) * 4;
     if constexpr (SLOTS == 1) {
+        // Per stage the thread ends up with row r of its pair's 2x2 block: dT[r][r] is its own sum,
+        // dT[r][1 - r] its own cross sum (row form) or the cross sum of the pair's other thread,
+        // which holds dT[1 - (1 - r)][1 - r] (column form: one more exchange).
+        static_for<0, NS>([&](auto S) {
+            constexpr int s = S;
+            if constexpr (COL) acc_cross[s] = partner<P::kind(s)>(acc_cross[s], c2.bperm_addr);
+        });
+        // The sums of a stage that ran in layout B belong to elements 16 apart within a wavefront,
+        // i.e. to 16-byte pieces 256 bytes apart in the slice.  They first travel through LDS (the
+        // factor slots or transposition buffers, dead by now) to the thread that holds the element
+        // in layout A, so that every wavefront stores 512 consecutive bytes per stage.
+        struct Late { int n; int s[NS]; };
+        constexpr Late late = [] {
+            Late l{};
+            for (int s = 0; s < NS; ++s)
+                if (P::layout(s) != 0) l.s[l.n++] = s;
+            return l;
+        }();
+        if constexpr (late.n > 0) {
+            T *stage = TB_LDS ? lds_tb : lds;
+            constexpr int room = (TB_LDS ? NS * kFastThreads : 4 * R * kFastRowWords) / (2 * kFastRowWords);
+            static_assert(room >= 1, "staging area for the partial sums");
+            constexpr int nbatch = (late.n + room - 1) / room;
+            static_for<0, nbatch>([&](auto BB) {
+                constexpr int j0 = BB * room;
+                constexpr int j1 = j0 + room < late.n ? j0 + room : late.n;
+                __syncthreads();   // the area is free: row loop or previous batch done
+                static_for<j0, j1>([&](auto J) {
+                    constexpr int s = late.s[J];
+                    store_pair(stage + ((J - j0) * kFastRowWords + c2.fB) * 2, acc_self[s], acc_cross[s]);
+                });
+                __syncthreads();
+                static_for<j0, j1>([&](auto J) {
+                    constexpr int s = late.s[J];
+                    load_pair(stage + ((J - j0) * kFastRowWords + c2.fA) * 2, acc_self[s], acc_cross[s]);
+                });
+            });
+        }
         static_for<0, NS>([&](auto S) {
             constexpr int s = S;
             constexpr int bit = P::bit(s);
-            constexpr int lay = P::layout(s);
-            const int e = lay ? c2.eB : c2.eA;
+            const int e = c2.eA;
             const int r = (e >> bit) & 1;
             const int i = P::pair_index(chunk, e, bit, a.low_bits);
             T *d = part + (int64_t)s * a.partial_slot + i * 4;
-            // The thread writes row r of the 2x2 block as one access: dT[r][r] is its own sum,
-            // dT[r][1 - r] its own cross sum (row form) or the cross sum of the pair's other
-            // thread, which holds dT[1 - (1 - r)][1 - r] (column form: one more exchange).
-            T other;
-            if constexpr (COL) other = partner<P::kind(s)>(acc_cross[s], c2.bperm_addr);
-            else other = acc_cross[s];
-            store_pair(d + 2 * r, r ? other : acc_self[s], r ? acc_self[s] : other);
+            store_pair(d + 2 * r, r ? acc_cross[s] : acc_self[s], r ? acc_self[s] : acc_cross[s]);
         });
     } else {
         // (the factor slots in LDS are dead by now and serve as the staging area)

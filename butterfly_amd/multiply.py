@@ -55,7 +55,7 @@ def butterfly_multiply_perm(twiddle: torch.Tensor, input: torch.Tensor, in_perm:
     twiddle, input and bias.  The reference runs each permutation as a separate gather
     (torch_butterfly/permutation.py:55-78)."""
     if not input.is_cuda:
-        n = 2 * twiddle.shape[3]
+        n = 1 << twiddle.shape[2]   # (not 2 * pairs: a layer of size 1 has no pairs)
         cols = n if output_size is None else output_size
         x = input
         if in_perm is not None:

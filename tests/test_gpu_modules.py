@@ -70,6 +70,34 @@ def test_module_bias_matches_separate_addition():
             assert close(a, r, rtol=1e-3, atol=1e-4 * max(1.0, r.abs().max().item()))
 
 
+def test_linear_dropin_of_4096_against_the_oracle():
+    """Butterfly(4096, 4096, bias=True, init='ortho', nblocks=2), the nn.Linear drop-in of the
+    quoted configurations, at a batch where its backward passes keep two row groups in flight:
+    output, d_input, d_twiddle against the CPU oracle, d_bias against numpy's column sum."""
+    import butterfly_amd as bfa
+    from conftest import rel_err
+    from oracle import oracle
+    torch.manual_seed(11)
+    B, n = 4200, 4096
+    layer = bfa.Butterfly(n, n, bias=True, init="ortho", nblocks=2).cuda()
+    say("linear drop-in", B, n, "increasing_stride", layer.increasing_stride)
+    x = torch.randn(B, n, device="cuda", requires_grad=True)
+    g = torch.randn(B, n, device="cuda")
+    y = layer(x)
+    dx, dtw, db = torch.autograd.grad(y, (x, layer.twiddle, layer.bias), g)
+    torch.cuda.synchronize()
+    tw = layer.twiddle.detach().cpu().numpy()
+    bias = layer.bias.detach().cpu().numpy()
+    xh, gh = x.detach().cpu().numpy().reshape(B, 1, n), g.cpu().numpy().reshape(B, 1, n)
+    inc = bool(layer.increasing_stride)
+    y_ref = oracle.butterfly_fw(tw, xh, inc, None).reshape(B, n) + bias
+    assert rel_err(y.detach().cpu().numpy(), y_ref) < 1e-5
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, xh, gh, inc)
+    assert rel_err(dx.cpu().numpy(), dx_ref.reshape(B, n)) < 1e-4
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < 1e-4
+    assert rel_err(db.cpu().numpy(), gh.reshape(B, n).sum(0, dtype=np.float64).astype(np.float32)) < 1e-4
+
+
 def test_autograd_through_module_reduces_loss():
     import butterfly_amd as bfa
     torch.manual_seed(0)

@@ -941,6 +941,12 @@ SAVING_CASES = [
     (np.complex64, 40, 1, 9, 2, None, None, False),
     (np.complex64, 10, 2, 12, 3, None, None, True),
     (np.complex64, 600, 1, 12, 1, 4000, None, True),
+    # the kernels the quoted 4096-wide configurations are timed through: two row groups in flight
+    # (16 or more row groups per workgroup) on two blocks of 4096, both stride orders, and the
+    # complex64 one-block plan at a batch that fills every workgroup
+    (np.float32, 4200, 1, 12, 2, None, None, True),
+    (np.float32, 4200, 1, 12, 2, None, None, False),
+    (np.complex64, 2048, 1, 12, 1, None, None, True),
 ]
 
 
@@ -1142,3 +1148,36 @@ def test_base4_single_pass_saves_nothing():
     t2 = torch.zeros(1, 1, 0, 128, 2, 2).cuda()
     x = torch.randn(10, 1, 256).cuda()
     assert _capi.multiply_base4_fw_bw_saving(t4, t2, x, torch.randn_like(x), True) is None
+
+
+def test_two_streams_with_their_own_workspaces():
+    """Two problems enqueued alternately on two streams (default priority), each call with a
+    workspace of its own: the library keeps no state between calls, so both streams' results must
+    equal the oracle's whatever the interleaving on the device."""
+    from butterfly_amd import _capi
+    rng = np.random.default_rng(7300)
+    cases = [make_case(rng, np.float32, 3000, 1, 10, 2), make_case(rng, np.complex64, 300, 1, 12, 1)]
+    incs = [False, True]
+    refs = [(oracle.butterfly_fw(tw, x, inc), *oracle.butterfly_bw(tw, x, g, inc)) for (tw, x, g), inc in zip(cases, incs)]
+    ops = [tuple(dev(a) for a in c) for c in cases]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    results = [[], []]
+    say("two streams: enqueue")
+    for rep in range(4):
+        for k in (0, 1):
+            with torch.cuda.stream(streams[k]):
+                tw, x, g = ops[k]
+                y = _capi.multiply_fw(tw, x, incs[k])
+                dtw, dx = _capi.multiply_bw(tw, x, g, incs[k])
+                results[k].append((y, dtw, dx))
+    for s in streams:
+        s.synchronize()
+    torch.cuda.synchronize()
+    say("two streams: check")
+    for k in (0, 1):
+        y_ref, dtw_ref, dx_ref = refs[k]
+        for y, dtw, dx in results[k]:
+            assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+            assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+            assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL

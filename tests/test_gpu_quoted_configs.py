@@ -92,6 +92,65 @@ def test_dft_factors_at_4096_all_gradients():
     assert rel_err(y, ref.astype(np.complex64)) < FW_TOL
 
 
+def check_saving_pair(tw, x, g, inc, what=""):
+    """The activation-keeping forward / backward pair (what the operator runs under autograd)
+    against the oracle."""
+    from butterfly_amd import _capi
+    say("saving pair", what, tw.dtype, x.shape, tw.shape[1], inc)
+    r = _capi.multiply_fw_bw_saving(dev(tw), dev(x), dev(g), inc, None)
+    assert r is not None, "this problem keeps activations between its backward passes"
+    y, dtw, dx, _ = r
+    torch.cuda.synchronize()
+    y, dtw, dx = y.cpu().numpy(), dtw.cpu().numpy(), dx.cpu().numpy()
+    y_ref = oracle.butterfly_fw(tw, x, inc, None)
+    assert rel_err(y, y_ref) < FW_TOL, what
+    del y_ref
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+    assert rel_err(dx, dx_ref) < BW_TOL, what
+    assert rel_err(dtw, dtw_ref) < BW_TOL, what
+
+
+def test_dft_factors_at_4096_through_the_activation_keeping_pair():
+    """The complex64 FFT configuration the way its benchmark line is timed: forward that keeps the
+    activation between the two backward passes, backward that starts from it; DFT factors, 2048
+    rows (every workgroup of both passes walks several row groups)."""
+    from butterfly_amd import special
+    L, B = 12, 2048
+    n = 1 << L
+    rng = np.random.default_rng(4106)
+    tw = special.fft(n, normalized=True, with_br_perm=False).twiddle.detach().cpu().numpy()
+    x, g = randn(rng, (B, 1, n), np.complex64), randn(rng, (B, 1, n), np.complex64)
+    check_saving_pair(tw, x, g, True, what="DFT factors, kept activations")
+
+
+def test_fft_configuration_at_full_size():
+    """(8192, 1, 4096) complex64 with the DFT factors, all 8192 rows: plain calls and the
+    activation-keeping pair, output / d_input / d_twiddle against the oracle (whose backward
+    scratch is 3 GiB here)."""
+    from butterfly_amd import special
+    L, B = 12, 8192
+    n = 1 << L
+    rng = np.random.default_rng(4107)
+    tw = special.fft(n, normalized=True, with_br_perm=False).twiddle.detach().cpu().numpy()
+    x, g = randn(rng, (B, 1, n), np.complex64), randn(rng, (B, 1, n), np.complex64)
+    from butterfly_amd import _capi
+    say("FFT configuration at full size")
+    twd, xd, gd = dev(tw), dev(x), dev(g)
+    y = _capi.multiply_fw(twd, xd, True, None).cpu().numpy()
+    dtw, dx = (t.cpu().numpy() for t in _capi.multiply_bw(twd, xd, gd, True))
+    ys, dtws, dxs, _ = _capi.multiply_fw_bw_saving(twd, xd, gd, True, None)
+    torch.cuda.synchronize()
+    ys, dtws, dxs = ys.cpu().numpy(), dtws.cpu().numpy(), dxs.cpu().numpy()
+    del twd, xd, gd
+    torch.cuda.empty_cache()
+    y_ref = oracle.butterfly_fw(tw, x, True, None)
+    assert rel_err(y, y_ref) < FW_TOL and rel_err(ys, y_ref) < FW_TOL
+    del y_ref, y, ys
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, True)
+    assert rel_err(dx, dx_ref) < BW_TOL and rel_err(dxs, dx_ref) < BW_TOL
+    assert rel_err(dtw, dtw_ref) < BW_TOL and rel_err(dtws, dtw_ref) < BW_TOL
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.complex64], ids=["f32", "c64"])
 @pytest.mark.parametrize("inc", [True, False], ids=["inc", "dec"])
 def test_reference_race_condition_shape(dtype, inc):

@@ -738,3 +738,16 @@ def test_layers_of_size_one():
     assert torch.allclose(bmm(xs), xs.expand(4, 3, 5) + bmm.bias)
     g = torch.autograd.grad(bmm(xs).sum(), bmm.bias)[0]
     assert torch.equal(g, torch.full_like(g, 4.0))
+
+
+def test_permuted_multiply_of_size_one_on_the_host():
+    """The host form of butterfly_multiply_perm at n = 1 (log n = 0, no pairs) with a column
+    table: one column in, one column out, the bias added."""
+    from butterfly_amd.multiply import butterfly_multiply_perm
+    tw = torch.zeros(3, 2, 0, 0, 2, 2)
+    x = torch.randn(4, 3, 1)
+    table = torch.zeros(1, dtype=torch.int32)
+    bias = torch.randn(3, 1)
+    y = butterfly_multiply_perm(tw, x, table, table, bias, True, None)
+    assert y.shape == (4, 3, 1) and torch.allclose(y, x + bias)
+    assert torch.allclose(butterfly_multiply_perm(tw, x, None, None, None, False, 1), x)
