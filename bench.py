@@ -10,9 +10,12 @@ fp32, nblocks = 2, decreasing stride first.  The other configurations of the bas
 second over the K timed steps, operands resident in HBM.  Before the W warmup steps the same
 step runs untimed for T milliseconds (default 250): the GPU needs a few tens of milliseconds
 of sustained load to reach its steady clocks, and K steps of a 0.2 ms workload would
-otherwise be timed entirely inside that ramp.  ``roofline`` describes the
-dominant call (the backward pass where there is one), timed with device events on the launch
-stream.  ``cpu_baseline`` is the single-threaded reference C++ (or, for base-4 and where the
+otherwise be timed entirely inside that ramp.  The K steps are then timed twice: once with
+nothing between them (host clock around two device synchronisations: ``value``, ``ms_per_step``)
+and once with a device event between consecutive calls on the launch stream (``fw_ms``,
+``bw_ms``).  ``roofline`` describes the dominant call (the backward pass where there is one)
+from those events, and the dominant kernel by itself (``kernel_name``, ``kernel_us``) from the
+committed rocprofv3 kernel-trace summary of the same command.  ``cpu_baseline`` is the single-threaded reference C++ (or, for base-4 and where the
 reference build is absent, the repo's CPU restatement) timed on this host on a bounded sample.
 """
 import argparse
@@ -62,6 +65,30 @@ def measured_traffic(config):
             except ValueError:
                 return None
     return None
+
+KERNEL_TABLE = os.path.join(ROOT, "profiles", "kernel_trace_all_configs.md")
+
+
+def measured_kernel(config):
+    """(rocprof kernel name, average microseconds per launch, algorithmic bytes per launch) of the
+    dominant kernel of `config`, from the `rocprofv3 --kernel-trace --stats` table under profiles/
+    (a line `| config | digest | kernel | us | bytes |`), or None when there is no reading for this
+    configuration or the sources have changed since it was taken."""
+    try:
+        with open(KERNEL_TABLE) as f:
+            lines = f.read().splitlines()
+    except OSError:
+        return None
+    digest = kernel_source_digest()
+    for line in lines:
+        cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 5 and cells[0] == config and cells[1] == digest:
+            try:
+                return cells[2], float(cells[3]), float(cells[4])
+            except ValueError:
+                return None
+    return None
+
 
 CONFIGS = {
     # name: batch, nstacks, log_n, nblocks, increasing_stride, complex, base4, backward, cpu sample batch
@@ -387,11 +414,23 @@ def main():
         for _ in range(5):
             dst.copy_(x)
         torch.cuda.synchronize()
-    # One event between consecutive calls: the end of a call is the start of the next one.
+    # Two timed regions of K steps each.  The first has nothing in it but the steps, bracketed by
+    # device synchronisation and the host clock: `value` and `ms_per_step` come from it (an event
+    # record costs the host several microseconds and the device a signal packet between two
+    # kernels, which is a third of a step at the small configurations).  The second repeats the K
+    # steps with one device event between consecutive calls (the end of a call is the start of the
+    # next one) and gives the split into forward and backward call that `roofline` is priced on.
     per_step = 2 if c["bw"] else 1
-    marks = [torch.cuda.Event(enable_timing=True) for _ in range(per_step * args.steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    for i in range(args.steps):
+        fw_call()
+        if c["bw"]:
+            bw_call()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(per_step * args.steps + 1)]
+    torch.cuda.synchronize()
     marks[0].record()
     for i in range(args.steps):
         fw_call()
@@ -400,7 +439,6 @@ def main():
             bw_call()
             marks[per_step * i + 2].record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     span = lambda j: marks[j].elapsed_time(marks[j + 1])
     fw_ms = sum(span(per_step * i) for i in range(args.steps)) / args.steps
     bw_ms = sum(span(per_step * i + 1) for i in range(args.steps)) / args.steps if c["bw"] else 0.0
@@ -426,6 +464,12 @@ def main():
                      "traffic": None if args.graph else measured_traffic(args.config)},
         "graphed": bool(args.graph),
     }
+    # the dominant kernel by itself, from the committed kernel-trace summary of this same command
+    # (its average launch duration and the algorithmic bytes of one launch)
+    kern = None if args.graph else measured_kernel(args.config)
+    if kern:
+        line["roofline"].update({"kernel_name": kern[0], "kernel_us": kern[1], "kernel_bytes": kern[2],
+                                 "frac_kernel": kern[2] / (kern[1] * 1e-6) / 1e9 / HBM_PEAK_GBS})
     # second roofline of the path: the same step against the fp32 vector rate (no MFMA: the
     # factors are 2x2 / 4x4 blocks, not a dense contraction)
     flops = algorithmic_flops(dict(c, bw=c["bw"] or c.get("graphed_bw", False)))

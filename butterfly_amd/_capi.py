@@ -12,6 +12,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libbutterfly_hip.so")
 
 BF_F32, BF_C64 = 0, 1
+BF_ERR_INVALID, BF_ERR_UNSUPPORTED, BF_ERR_HIP, BF_ERR_WORKSPACE = -1, -2, -3, -4
 
 SYMBOLS = [
     "bf_version", "bf_hip_version", "bf_last_error",
@@ -95,13 +96,13 @@ def lib():
         L.bf_butterfly_multiply_fw_saving.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_bw_saved_workspace_bytes.argtypes = [pp, ctypes.c_int]
         L.bf_butterfly_multiply_bw_saved_workspace_bytes.restype = sz
-        L.bf_butterfly_multiply_bw_saved.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_bw_saved.argtypes = [pp, vp, vp, vp, vp, sz, vp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_base4_saved_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_base4_saved_bytes.restype = sz
         L.bf_butterfly_multiply_base4_fw_saving.argtypes = [pp, vp, vp, vp, vp, vp, sz, vp]
         L.bf_butterfly_multiply_base4_bw_saved_workspace_bytes.argtypes = [pp]
         L.bf_butterfly_multiply_base4_bw_saved_workspace_bytes.restype = sz
-        L.bf_butterfly_multiply_base4_bw_saved.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.bf_butterfly_multiply_base4_bw_saved.argtypes = [pp, vp, vp, vp, vp, vp, sz, vp, vp, vp, vp, sz, vp]
         _lib = L
     return _lib
 
@@ -115,6 +116,15 @@ class ButterflyError(RuntimeError):
 def _check(rc):
     if rc != 0:
         raise ButterflyError(rc)
+
+
+SIZE_INVALID = ctypes.c_size_t(-1).value   # BF_SIZE_INVALID: the size queries' answer for a refused problem
+
+
+def _size(nbytes):
+    if nbytes == SIZE_INVALID:
+        raise ButterflyError(BF_ERR_INVALID)
+    return nbytes
 
 
 def _dtype_code(t):
@@ -157,7 +167,7 @@ def multiply_fw(twiddle, input, increasing_stride, output_size=None):
     p = make_problem(input, log_n, nb, increasing_stride, O)
     out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
     p.output_stride = _strides(out)
-    nbytes = lib().bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p))
+    nbytes = _size(lib().bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_fw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(out), _ptr(ws), nbytes,
                                           _stream()))
@@ -174,7 +184,7 @@ def multiply_bias_fw(twiddle, input, bias, increasing_stride, output_size=None):
     p = make_problem(input, log_n, nb, increasing_stride, O)
     out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
     p.output_stride = _strides(out)
-    nbytes = lib().bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p))
+    nbytes = _size(lib().bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_bias_fw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(bias), _ptr(out),
                                                _ptr(ws), nbytes, _stream()))
@@ -192,7 +202,7 @@ def bias_grad(grad):
     p.nblocks = 1
     p.output_stride = _strides(grad)
     d_bias = torch.empty(grad.shape[1], grad.shape[2], dtype=grad.dtype, device=grad.device)
-    nbytes = lib().bf_butterfly_bias_grad_workspace_bytes(ctypes.byref(p))
+    nbytes = _size(lib().bf_butterfly_bias_grad_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=grad.device)
     _check(lib().bf_butterfly_bias_grad(ctypes.byref(p), _ptr(grad), _ptr(d_bias), _ptr(ws), nbytes, _stream()))
     return d_bias
@@ -208,7 +218,7 @@ def multiply_bias_bw(twiddle, input, grad, increasing_stride):
     d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
     d_bias = torch.empty(grad.shape[1], grad.shape[2], dtype=grad.dtype, device=grad.device)
     p.d_input_stride = _strides(d_input)
-    nbytes = lib().bf_butterfly_multiply_bias_bw_workspace_bytes(ctypes.byref(p))
+    nbytes = _size(lib().bf_butterfly_multiply_bias_bw_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_bias_bw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
                                                _ptr(d_twiddle), _ptr(d_input), _ptr(d_bias), _ptr(ws), nbytes,
@@ -282,7 +292,7 @@ def multiply_perm_fw(twiddle, input, in_perm, out_index, bias, increasing_stride
     p = make_problem(input, log_n, nb, increasing_stride, O)
     out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
     p.output_stride = _strides(out)
-    nbytes = lib().bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p))
+    nbytes = _size(lib().bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_perm_fw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _table(in_perm, n),
                                                _table(out_index, n), None if bias is None else _ptr(bias),
@@ -303,7 +313,7 @@ def multiply_perm_bw(twiddle, input, grad, in_perm, out_index, increasing_stride
     p.d_input_stride = _strides(d_input)
     size_fn = lib().bf_butterfly_multiply_bias_bw_workspace_bytes if with_bias \
         else lib().bf_butterfly_multiply_bw_workspace_bytes
-    nbytes = size_fn(ctypes.byref(p))
+    nbytes = _size(size_fn(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_perm_bw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
                                                _table(in_perm, n), _table(out_index, n), _ptr(d_twiddle),
@@ -320,7 +330,7 @@ def multiply_bw(twiddle, input, grad, increasing_stride):
     d_twiddle = torch.empty_like(twiddle)
     d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
     p.d_input_stride = _strides(d_input)
-    nbytes = lib().bf_butterfly_multiply_bw_workspace_bytes(ctypes.byref(p))
+    nbytes = _size(lib().bf_butterfly_multiply_bw_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_bw(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad),
                                           _ptr(d_twiddle), _ptr(d_input), _ptr(ws), nbytes, _stream()))
@@ -345,10 +355,11 @@ def multiply_bw_noalloc(twiddle, input, grad, increasing_stride, d_twiddle=None,
 
 
 def multiply_fw_bw_saving(twiddle, input, grad, increasing_stride, output_size=None, bias=None, in_perm=None,
-                          out_index=None):
+                          out_index=None, saved_given=None):
     """Forward that leaves the backward's intermediate activations behind, then the backward that
     reads them.  Returns (output, d_twiddle, d_input, d_bias or None), or None when the problem
-    saves nothing."""
+    saves nothing.  saved_given: size to declare for the saved area to the backward (tests of the
+    size check; default: its real size)."""
     assert twiddle.is_contiguous() and twiddle.is_cuda and input.is_cuda and grad.is_cuda
     nb, log_n = twiddle.shape[1], twiddle.shape[2]
     n = 1 << log_n
@@ -358,7 +369,7 @@ def multiply_fw_bw_saving(twiddle, input, grad, increasing_stride, output_size=N
     p.output_stride = _strides(out)
     d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
     p.d_input_stride = _strides(d_input)
-    nsaved = lib().bf_butterfly_multiply_saved_bytes(ctypes.byref(p))
+    nsaved = _size(lib().bf_butterfly_multiply_saved_bytes(ctypes.byref(p)))
     if nsaved == 0:
         return None
     saved = torch.empty(nsaved, dtype=torch.uint8, device=input.device)
@@ -369,9 +380,10 @@ def multiply_fw_bw_saving(twiddle, input, grad, increasing_stride, output_size=N
     p.output_stride = _strides(grad)
     d_twiddle = torch.empty_like(twiddle)
     d_bias = None if bias is None else torch.empty_like(bias)
-    nbytes = lib().bf_butterfly_multiply_bw_saved_workspace_bytes(ctypes.byref(p), int(bias is not None))
+    nbytes = _size(lib().bf_butterfly_multiply_bw_saved_workspace_bytes(ctypes.byref(p), int(bias is not None)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_bw_saved(ctypes.byref(p), _ptr(twiddle), _ptr(input), _ptr(grad), _ptr(saved),
+                                                saved.numel() if saved_given is None else saved_given,
                                                 _table(in_perm, n), _table(out_index, n), _ptr(d_twiddle), _ptr(d_input),
                                                 None if d_bias is None else _ptr(d_bias), _ptr(ws), nbytes, _stream()))
     return out, d_twiddle, d_input, d_bias
@@ -386,7 +398,7 @@ def multiply_base4_fw(twiddle4, twiddle2, input, increasing_stride, output_size=
     p = make_problem(input, log_n, nb, increasing_stride, O)
     out = torch.empty(input.shape[0], input.shape[1], O, dtype=input.dtype, device=input.device)
     p.output_stride = _strides(out)
-    nbytes = lib().bf_butterfly_multiply_base4_fw_workspace_bytes(ctypes.byref(p))
+    nbytes = _size(lib().bf_butterfly_multiply_base4_fw_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_base4_fw(ctypes.byref(p), _ptr(twiddle4), _ptr(twiddle2),
                                                 _ptr(input), _ptr(out), _ptr(ws), nbytes, _stream()))
@@ -402,7 +414,7 @@ def multiply_base4_bw(twiddle4, twiddle2, input, grad, increasing_stride):
     d4, d2 = torch.empty_like(twiddle4), torch.empty_like(twiddle2)
     d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
     p.d_input_stride = _strides(d_input)
-    nbytes = lib().bf_butterfly_multiply_base4_bw_workspace_bytes(ctypes.byref(p))
+    nbytes = _size(lib().bf_butterfly_multiply_base4_bw_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_base4_bw(ctypes.byref(p), _ptr(twiddle4), _ptr(twiddle2), _ptr(input),
                                                 _ptr(grad), _ptr(d4), _ptr(d2), _ptr(d_input), _ptr(ws),
@@ -424,7 +436,7 @@ def multiply_base4_fw_bw_saving(twiddle4, twiddle2, input, grad, increasing_stri
     p.output_stride = _strides(out)
     d_input = torch.empty(input.shape, dtype=input.dtype, device=input.device)
     p.d_input_stride = _strides(d_input)
-    nsaved = lib().bf_butterfly_multiply_base4_saved_bytes(ctypes.byref(p))
+    nsaved = _size(lib().bf_butterfly_multiply_base4_saved_bytes(ctypes.byref(p)))
     if nsaved == 0:
         return None
     saved = torch.empty(nsaved, dtype=torch.uint8, device=input.device)
@@ -433,9 +445,10 @@ def multiply_base4_fw_bw_saving(twiddle4, twiddle2, input, grad, increasing_stri
     assert tuple(grad.shape) == tuple(out.shape)
     p.output_stride = _strides(grad)
     d4, d2 = torch.empty_like(twiddle4), torch.empty_like(twiddle2)
-    nbytes = lib().bf_butterfly_multiply_base4_bw_saved_workspace_bytes(ctypes.byref(p))
+    nbytes = _size(lib().bf_butterfly_multiply_base4_bw_saved_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=input.device)
     _check(lib().bf_butterfly_multiply_base4_bw_saved(ctypes.byref(p), _ptr(twiddle4), _ptr(twiddle2), _ptr(input),
-                                                      _ptr(grad), _ptr(saved), _ptr(d4), _ptr(d2), _ptr(d_input),
+                                                      _ptr(grad), _ptr(saved), saved.numel(), _ptr(d4), _ptr(d2),
+                                                      _ptr(d_input),
                                                       _ptr(ws), nbytes, _stream()))
     return out, d4, d2, d_input

@@ -389,14 +389,29 @@ int64_t row_cap(const bf_problem *p, bool backward)
 
 // Row-group partition of a LOW pass: `lanes` independent (stack, chunk) columns share the CUs;
 // a workgroup walks at most max_rows rows (more workgroups than compute units if need be).
+// `slices`: the pass is a base-2 backward pass, whose workgroups each end with a partial slice of
+// the d_twiddle sums (written once, read once by the reduce) whatever the number of rows they
+// walked.  With few rows that traffic outweighs the row loop: walking one more row group costs a
+// workgroup about as much as 27 * 1024 / n of its slices cost the device (measured on the
+// two-block 1024-element kernels at 256 ... 4096 rows: 1.1 us per row against 0.04 us per 160 KiB
+// slice written and re-read), so the host picks the number of row groups per workgroup that makes
+// groups * row + workgroups * slice least.
 FastGrid fast_grid(int64_t batch, int Lk, int64_t lanes, int rows_in_flight, int wg_per_cu,
-                   int64_t max_rows = kNoRowCap)
+                   int64_t max_rows = kNoRowCap, bool slices = false)
 {
     FastGrid g;
     g.slots = 1024 >> Lk;
     g.ngroups = (batch + g.slots - 1) / g.slots;
-    const int64_t want = std::max<int64_t>(1, (int64_t)num_cu() * wg_per_cu / lanes);
+    int64_t want = std::max<int64_t>(1, (int64_t)num_cu() * wg_per_cu / lanes);
     const int64_t iters = (g.ngroups + rows_in_flight - 1) / rows_in_flight;
+    if (slices && iters > 0) {
+        const double slice = 1.0 / (27.0 * (double)g.slots);   // in units of one row group's time
+        auto cost = [&](int64_t groups) { return (double)groups + (double)((iters + groups - 1) / groups) * slice; };
+        int64_t best = (iters + want - 1) / want;
+        for (int64_t groups = best + 1; groups <= iters && (double)groups < cost(best); ++groups)
+            if (cost(groups) < cost(best)) best = groups;
+        want = (iters + best - 1) / best;
+    }
     g.nwg = std::min(want, iters);
     g.groups_per_wg = ((iters + g.nwg - 1) / g.nwg) * rows_in_flight;
     const int64_t max_groups = ((max_rows / g.slots - kRowMargin) / rows_in_flight) * rows_in_flight;
@@ -428,7 +443,7 @@ bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
         const Pass &q = pl.pass[k];
         const FastGrid g = q.wide ? wide_grid(p->batch, p->nstacks)
                                   : fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), backward ? 1 : fw_rows(p),
-                                              backward ? 1 : kFastFwWgPerCu, cap);
+                                              backward ? 1 : kFastFwWgPerCu, cap, backward);
         rows = std::max(rows, (g.groups_per_wg + kFastFwRows + 2) * g.slots);
     }
     const int64_t dense[3] = {p->nstacks * n, n, 1};
@@ -1258,7 +1273,7 @@ BwPlan plan_bw(const bf_problem *p, bool base4, bool saved_boundaries = false, b
         int64_t nparts = 1, slices = 1;  // slices: partial (stage, 2n) slices of the pass that needs most
         for (int k = 0; k < mp.npass; ++k) {
             const Pass &q = mp.pass[k];
-            const int64_t np = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), 1, 1, row_cap(p, true)).nwg;
+            const int64_t np = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), 1, 1, row_cap(p, true), true).nwg;
             nparts = std::max(nparts, np);
             slices = std::max(slices, np * (q.t1 - q.t0));
         }
@@ -1515,7 +1530,7 @@ int backward(const bf_problem *p, bool base4, const void *tw2, const void *tw4, 
             const View giv = k == 0 ? dn_view : dense;
             int64_t nparts = 0;
             {
-                const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), 1, 1, row_cap(p, true));
+                const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), 1, 1, row_cap(p, true), true);
                 FastBwArgs a = {};
                 a.tw = tw2;
                 a.tw_stack_stride = sc.tw2_stack_stride;
@@ -1678,7 +1693,7 @@ const char *bf_last_error(void) { return g_last_error.c_str(); }
 
 size_t bf_butterfly_multiply_fw_workspace_bytes(const bf_problem *p)
 {
-    if (check_problem(p, false)) return 0;
+    if (check_problem(p, false)) return BF_SIZE_INVALID;
     return forward_workspace(p, false);
 }
 
@@ -1690,7 +1705,7 @@ int bf_butterfly_multiply_fw(const bf_problem *p, const void *twiddle, const voi
 
 size_t bf_butterfly_multiply_bw_workspace_bytes(const bf_problem *p)
 {
-    if (check_problem(p, true)) return 0;
+    if (check_problem(p, true)) return BF_SIZE_INVALID;
     return bw_workspace_total(p, false);
 }
 
@@ -1704,7 +1719,7 @@ int bf_butterfly_multiply_bw(const bf_problem *p, const void *twiddle, const voi
 
 size_t bf_butterfly_multiply_base4_fw_workspace_bytes(const bf_problem *p)
 {
-    if (check_problem(p, false)) return 0;
+    if (check_problem(p, false)) return BF_SIZE_INVALID;
     return forward_workspace(p, true);
 }
 
@@ -1716,7 +1731,7 @@ int bf_butterfly_multiply_bias_fw(const bf_problem *p, const void *twiddle, cons
 
 size_t bf_butterfly_bias_grad_workspace_bytes(const bf_problem *p)
 {
-    if (check_problem(p, false)) return 0;
+    if (check_problem(p, false)) return BF_SIZE_INVALID;
     return plan_bias_grad(p).bytes;
 }
 
@@ -1766,7 +1781,7 @@ static size_t bias_area_bytes(const bf_problem *p)
 
 size_t bf_butterfly_multiply_bias_bw_workspace_bytes(const bf_problem *p)
 {
-    if (check_problem(p, true)) return 0;
+    if (check_problem(p, true)) return BF_SIZE_INVALID;
     return align256(bw_workspace_total(p, false)) + bias_area_bytes(p);
 }
 
@@ -1848,7 +1863,7 @@ static size_t saved_bytes(const bf_problem *p)
 
 size_t bf_butterfly_multiply_saved_bytes(const bf_problem *p)
 {
-    if (check_problem(p, true)) return 0;
+    if (check_problem(p, true)) return BF_SIZE_INVALID;
     return saved_bytes(p);
 }
 
@@ -1895,20 +1910,28 @@ int bf_butterfly_multiply_fw_saving(const bf_problem *p, const void *twiddle, co
 
 size_t bf_butterfly_multiply_bw_saved_workspace_bytes(const bf_problem *p, int with_bias)
 {
-    if (check_problem(p, true)) return 0;
+    if (check_problem(p, true)) return BF_SIZE_INVALID;
     const size_t main_bytes = bw_workspace_total(p, true);
     return with_bias ? align256(main_bytes) + bias_area_bytes(p) : main_bytes;
 }
 
 int bf_butterfly_multiply_bw_saved(const bf_problem *p, const void *twiddle, const void *input, const void *grad,
-                                   const void *saved, const int32_t *in_perm, const int32_t *out_index,
-                                   void *d_twiddle, void *d_input, void *d_bias, void *workspace,
-                                   size_t workspace_bytes, void *stream)
+                                   const void *saved, size_t saved_bytes_given, const int32_t *in_perm,
+                                   const int32_t *out_index, void *d_twiddle, void *d_input, void *d_bias,
+                                   void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = check_problem(p, true);
     if (rc) return rc;
     if (!saved || saved_bytes(p) == 0)
         return fail(BF_ERR_INVALID, "this problem has no saved activations: use bf_butterfly_multiply_bw");
+    // The planes this call reads follow from its own plan (strides of grad and d_input, column
+    // tables): the caller's area must hold them.  A plan of a single pass reads none and runs as
+    // the plain call does (its workspace is the same either way).
+    const size_t planes = saved_bytes_of_plan(p, in_perm || out_index);
+    if (planes == 0) saved = nullptr;
+    else if (saved_bytes_given < planes)
+        return fail(BF_ERR_WORKSPACE, "the backward reads %zu bytes of saved activations, %zu given", planes,
+                    saved_bytes_given);
     if (d_bias)
         return bias_backward(p, twiddle, input, grad, d_twiddle, d_input, d_bias, workspace, workspace_bytes, stream,
                              in_perm, out_index, saved);
@@ -1955,7 +1978,7 @@ int bf_butterfly_multiply_base4_fw(const bf_problem *p, const void *twiddle4, co
 
 size_t bf_butterfly_multiply_base4_bw_workspace_bytes(const bf_problem *p)
 {
-    if (check_problem(p, true)) return 0;
+    if (check_problem(p, true)) return BF_SIZE_INVALID;
     return plan_bw(p, true).total;
 }
 
@@ -1981,7 +2004,7 @@ static size_t saved4_bytes(const bf_problem *p)
 
 size_t bf_butterfly_multiply_base4_saved_bytes(const bf_problem *p)
 {
-    if (check_problem(p, true)) return 0;
+    if (check_problem(p, true)) return BF_SIZE_INVALID;
     return saved4_bytes(p);
 }
 
@@ -2023,19 +2046,23 @@ int bf_butterfly_multiply_base4_fw_saving(const bf_problem *p, const void *twidd
 
 size_t bf_butterfly_multiply_base4_bw_saved_workspace_bytes(const bf_problem *p)
 {
-    if (check_problem(p, true)) return 0;
+    if (check_problem(p, true)) return BF_SIZE_INVALID;
     return plan_bw(p, true, true).total;
 }
 
 int bf_butterfly_multiply_base4_bw_saved(const bf_problem *p, const void *twiddle4, const void *twiddle2,
-                                         const void *input, const void *grad, const void *saved, void *d_twiddle4,
-                                         void *d_twiddle2, void *d_input, void *workspace, size_t workspace_bytes,
-                                         void *stream)
+                                         const void *input, const void *grad, const void *saved,
+                                         size_t saved_bytes_given, void *d_twiddle4, void *d_twiddle2, void *d_input,
+                                         void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = check_problem(p, true);
     if (rc) return rc;
-    if (!saved || saved4_bytes(p) == 0)
+    const size_t planes = saved4_bytes(p);
+    if (!saved || planes == 0)
         return fail(BF_ERR_INVALID, "this problem has no saved activations: use bf_butterfly_multiply_base4_bw");
+    if (saved_bytes_given < planes)
+        return fail(BF_ERR_WORKSPACE, "the backward reads %zu bytes of saved activations, %zu given", planes,
+                    saved_bytes_given);
     return backward(p, true, twiddle2, twiddle4, input, grad, d_twiddle2, d_twiddle4, d_input, workspace,
                     workspace_bytes, stream, nullptr, nullptr, nullptr, nullptr, saved);
 }

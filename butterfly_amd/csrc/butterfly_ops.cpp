@@ -137,6 +137,13 @@ void *current_stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(
 
 void check_rc(int rc, const char *who) { TORCH_CHECK(rc == BF_OK, who, ": ", bf_last_error()); }
 
+// Answer of one of the library's size queries: BF_SIZE_INVALID means the problem was refused.
+size_t valid_size(size_t bytes)
+{
+    TORCH_CHECK(bytes != BF_SIZE_INVALID, "torch_butterfly: ", bf_last_error());
+    return bytes;
+}
+
 // Dense copy of a (small) twiddle tensor; also materialises lazy conjugation.
 // dense and 16-byte aligned (the kernels read factor blocks with 16-byte loads): a contiguous view
 // at an odd offset into its storage is copied
@@ -233,7 +240,7 @@ Tensor multiply_fw_impl(const Tensor &twiddle, const Tensor &input, const Tensor
         p.d_input_stride[0] = s.batch > 1 ? s.nstacks * dw : 0;
         p.d_input_stride[1] = s.nstacks > 1 ? dw : 0;
         p.d_input_stride[2] = s.input_size > 1 ? 1 : 0;
-        const size_t nsaved = bf_butterfly_multiply_saved_bytes(&p);
+        const size_t nsaved = valid_size(bf_butterfly_multiply_saved_bytes(&p));
         if (nsaved > 0) {
             *keep = at::empty({(int64_t)nsaved}, x.options().dtype(at::kByte));
             check_rc(bf_butterfly_multiply_fw_saving(&p, tw.data_ptr(), x.data_ptr(), b.defined() ? b.data_ptr() : nullptr,
@@ -243,7 +250,7 @@ Tensor multiply_fw_impl(const Tensor &twiddle, const Tensor &input, const Tensor
             return output;
         }
     }
-    const size_t ws_bytes = bf_butterfly_multiply_fw_workspace_bytes(&p);
+    const size_t ws_bytes = valid_size(bf_butterfly_multiply_fw_workspace_bytes(&p));
     Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
     if (ip || oi) {
         check_rc(bf_butterfly_multiply_perm_fw(&p, tw.data_ptr(), x.data_ptr(), ip, oi,
@@ -293,7 +300,7 @@ Tensor butterfly_bias_grad(const Tensor grad)
     while (((int64_t)1 << p.log_n) < p.output_size) ++p.log_n;
     set_strides(p.output_stride, g);
     Tensor d_bias = at::empty({p.nstacks, p.output_size}, g.options());
-    const size_t ws_bytes = bf_butterfly_bias_grad_workspace_bytes(&p);
+    const size_t ws_bytes = valid_size(bf_butterfly_bias_grad_workspace_bytes(&p));
     Tensor ws = at::empty({(int64_t)ws_bytes}, g.options().dtype(at::kByte));
     check_rc(bf_butterfly_bias_grad(&p, g.data_ptr(), d_bias.data_ptr(), ws.data_ptr(), ws_bytes, current_stream()),
              "butterfly_bias_grad");
@@ -344,12 +351,21 @@ std::tuple<Tensor, Tensor, Tensor> multiply_bw_impl(const Tensor &twiddle, const
     Tensor keep_in, keep_out;
     const int32_t *ip = table_ptr(in_perm, keep_in, x, s.n, "in_perm", who);
     const int32_t *oi = table_ptr(out_index, keep_out, x, s.n, "out_index", who);
-    if (kept.defined()) {
+    // The forward decided what to keep from a plan made with its own strides; the backward plans
+    // from the strides of grad and d_input.  Where that plan reads no kept activations, or more
+    // than the forward left, the recomputing call serves the request.
+    bool use_kept = kept.defined();
+    if (use_kept) {
+        const size_t reads = valid_size(bf_butterfly_multiply_saved_bytes(&p));
+        if (reads == 0 || reads > (size_t)kept.numel()) use_kept = false;
+    }
+    if (use_kept) {
         if (ip || oi) TORCH_CHECK(s.input_size <= s.n, who, ": column tables need input_size <= n");
         if (with_bias) d_bias = at::empty({s.nstacks, output_size}, g.options());
-        const size_t ws_bytes = bf_butterfly_multiply_bw_saved_workspace_bytes(&p, with_bias ? 1 : 0);
+        const size_t ws_bytes = valid_size(bf_butterfly_multiply_bw_saved_workspace_bytes(&p, with_bias ? 1 : 0));
         Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
-        check_rc(bf_butterfly_multiply_bw_saved(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), kept.data_ptr(), ip, oi,
+        check_rc(bf_butterfly_multiply_bw_saved(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), kept.data_ptr(),
+                                                (size_t)kept.numel(), ip, oi,
                                                 d_twiddle.data_ptr(), d_input.data_ptr(),
                                                 with_bias ? d_bias.data_ptr() : nullptr, ws.data_ptr(), ws_bytes,
                                                 current_stream()),
@@ -357,8 +373,8 @@ std::tuple<Tensor, Tensor, Tensor> multiply_bw_impl(const Tensor &twiddle, const
     } else if (ip || oi) {
         TORCH_CHECK(s.input_size <= s.n, who, ": column tables need input_size <= n");
         if (with_bias) d_bias = at::empty({s.nstacks, output_size}, g.options());
-        const size_t ws_bytes = with_bias ? bf_butterfly_multiply_bias_bw_workspace_bytes(&p)
-                                          : bf_butterfly_multiply_bw_workspace_bytes(&p);
+        const size_t ws_bytes = with_bias ? valid_size(bf_butterfly_multiply_bias_bw_workspace_bytes(&p))
+                                          : valid_size(bf_butterfly_multiply_bw_workspace_bytes(&p));
         Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
         check_rc(bf_butterfly_multiply_perm_bw(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), ip, oi,
                                                d_twiddle.data_ptr(), d_input.data_ptr(),
@@ -367,14 +383,14 @@ std::tuple<Tensor, Tensor, Tensor> multiply_bw_impl(const Tensor &twiddle, const
                  who);
     } else if (with_bias) {
         d_bias = at::empty({s.nstacks, output_size}, g.options());
-        const size_t ws_bytes = bf_butterfly_multiply_bias_bw_workspace_bytes(&p);
+        const size_t ws_bytes = valid_size(bf_butterfly_multiply_bias_bw_workspace_bytes(&p));
         Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
         check_rc(bf_butterfly_multiply_bias_bw(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), d_twiddle.data_ptr(),
                                                d_input.data_ptr(), d_bias.data_ptr(), ws.data_ptr(), ws_bytes,
                                                current_stream()),
                  who);
     } else {
-        const size_t ws_bytes = bf_butterfly_multiply_bw_workspace_bytes(&p);
+        const size_t ws_bytes = valid_size(bf_butterfly_multiply_bw_workspace_bytes(&p));
         Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
         check_rc(bf_butterfly_multiply_bw(&p, tw.data_ptr(), x.data_ptr(), g.data_ptr(), d_twiddle.data_ptr(),
                                           d_input.data_ptr(), ws.data_ptr(), ws_bytes, current_stream()),
@@ -710,7 +726,7 @@ Tensor base4_fw_impl(const Tensor &twiddle4, const Tensor &twiddle2, const Tenso
         p.d_input_stride[0] = s.batch > 1 ? s.nstacks * dw : 0;
         p.d_input_stride[1] = s.nstacks > 1 ? dw : 0;
         p.d_input_stride[2] = s.input_size > 1 ? 1 : 0;
-        const size_t nsaved = bf_butterfly_multiply_base4_saved_bytes(&p);
+        const size_t nsaved = valid_size(bf_butterfly_multiply_base4_saved_bytes(&p));
         if (nsaved > 0) {
             *keep = at::empty({(int64_t)nsaved}, x.options().dtype(at::kByte));
             check_rc(bf_butterfly_multiply_base4_fw_saving(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(),
@@ -720,7 +736,7 @@ Tensor base4_fw_impl(const Tensor &twiddle4, const Tensor &twiddle2, const Tenso
             return output;
         }
     }
-    const size_t ws_bytes = bf_butterfly_multiply_base4_fw_workspace_bytes(&p);
+    const size_t ws_bytes = valid_size(bf_butterfly_multiply_base4_fw_workspace_bytes(&p));
     Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
     check_rc(bf_butterfly_multiply_base4_fw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(), output.data_ptr(),
                                             ws.data_ptr(), ws_bytes, current_stream()),
@@ -756,16 +772,23 @@ std::tuple<Tensor, Tensor, Tensor> base4_bw_impl(const Tensor &twiddle4, const T
     bf_problem p = make_problem(s, x, increasing_stride, output_size, "butterfly_multiply_base4_bw");
     set_strides(p.output_stride, g);
     set_strides(p.d_input_stride, d_input);
-    if (kept.defined()) {
-        const size_t ws_bytes = bf_butterfly_multiply_base4_bw_saved_workspace_bytes(&p);
+    // (as in the base-2 backward: the plan of this call decides whether the kept planes serve it)
+    bool use_kept = kept.defined();
+    if (use_kept) {
+        const size_t reads = valid_size(bf_butterfly_multiply_base4_saved_bytes(&p));
+        if (reads == 0 || reads > (size_t)kept.numel()) use_kept = false;
+    }
+    if (use_kept) {
+        const size_t ws_bytes = valid_size(bf_butterfly_multiply_base4_bw_saved_workspace_bytes(&p));
         Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
         check_rc(bf_butterfly_multiply_base4_bw_saved(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(), g.data_ptr(),
-                                                      kept.data_ptr(), d4.data_ptr(), d2.data_ptr(), d_input.data_ptr(),
+                                                      kept.data_ptr(), (size_t)kept.numel(), d4.data_ptr(), d2.data_ptr(),
+                                                      d_input.data_ptr(),
                                                       ws.data_ptr(), ws_bytes, current_stream()),
                  "butterfly_multiply_base4_bw");
         return std::make_tuple(d4, d2, d_input);
     }
-    const size_t ws_bytes = bf_butterfly_multiply_base4_bw_workspace_bytes(&p);
+    const size_t ws_bytes = valid_size(bf_butterfly_multiply_base4_bw_workspace_bytes(&p));
     Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
     check_rc(bf_butterfly_multiply_base4_bw(&p, tw4.data_ptr(), tw2.data_ptr(), x.data_ptr(), g.data_ptr(),
                                             d4.data_ptr(), d2.data_ptr(), d_input.data_ptr(), ws.data_ptr(),

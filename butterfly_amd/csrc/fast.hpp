@@ -441,10 +441,18 @@ __device__ __forceinline__ void load_row_to_lds(BufDesc desc, unsigned lds_addr,
                  : "memory");
 }
 
+// BF_SAFE_WAITS (a build switch, off in the shipped library): every counted wait becomes "wait for
+// all of this wavefront's memory operations".  Results must be the same with and without it; a
+// difference would mean a count is wrong.  The row pipelines then also wait for their own stores,
+// so the kernels run slower.
 template <int N>
 __device__ __forceinline__ void wait_rows_in_lds()
 {
+#ifdef BF_SAFE_WAITS
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#else
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+#endif
 }
 
 typedef __attribute__((address_space(3))) float LdsFloat;

@@ -32,6 +32,10 @@ extern "C" {
 #define BF_ERR_HIP (-3)         /* a HIP call or kernel launch failed                 */
 #define BF_ERR_WORKSPACE (-4)   /* workspace missing or too small                     */
 
+/* What every size query (*_workspace_bytes, *_saved_bytes) answers for a problem that does not
+ * pass validation (bf_last_error() says why); 0 means "valid, no such memory needed".       */
+#define BF_SIZE_INVALID ((size_t)-1)
+
 /* Problem description shared by all entry points.  Plain data, no ownership. */
 typedef struct bf_problem {
     int32_t dtype;             /* BF_F32 or BF_C64                                              */
@@ -159,12 +163,15 @@ int bf_butterfly_multiply_fw_saving(const bf_problem *p, const void *twiddle, co
                                     size_t saved_capacity, void *stream);
 size_t bf_butterfly_multiply_bw_saved_workspace_bytes(const bf_problem *p, int with_bias);
 /* d_bias (S, O) may be NULL; when given it receives the column sums of grad as in
- * bf_butterfly_multiply_bias_bw (size the workspace with with_bias != 0).                   */
+ * bf_butterfly_multiply_bias_bw (size the workspace with with_bias != 0).  saved_bytes: size of
+ * the area behind `saved`; the call plans from ITS problem (strides of grad and d_input, column
+ * tables) which planes it reads and answers BF_ERR_WORKSPACE when the area is smaller than
+ * that, BF_ERR_INVALID when that plan reads none (then use bf_butterfly_multiply_bw).        */
 int bf_butterfly_multiply_bw_saved(const bf_problem *p, const void *twiddle, const void *input,
-                                   const void *grad, const void *saved, const int32_t *in_perm,
-                                   const int32_t *out_index, void *d_twiddle, void *d_input,
-                                   void *d_bias, void *workspace, size_t workspace_bytes,
-                                   void *stream);
+                                   const void *grad, const void *saved, size_t saved_bytes,
+                                   const int32_t *in_perm, const int32_t *out_index,
+                                   void *d_twiddle, void *d_input, void *d_bias, void *workspace,
+                                   size_t workspace_bytes, void *stream);
 
 /* Diagnostic, host only (no device call): how the base-2 forward (backward != 0: backward)
  * call for this problem is cut into launches, one text line per pass in order --
@@ -235,9 +242,9 @@ int bf_butterfly_multiply_base4_fw_saving(const bf_problem *p, const void *twidd
 size_t bf_butterfly_multiply_base4_bw_saved_workspace_bytes(const bf_problem *p);
 int bf_butterfly_multiply_base4_bw_saved(const bf_problem *p, const void *twiddle4,
                                          const void *twiddle2, const void *input,
-                                         const void *grad, const void *saved, void *d_twiddle4,
-                                         void *d_twiddle2, void *d_input, void *workspace,
-                                         size_t workspace_bytes, void *stream);
+                                         const void *grad, const void *saved, size_t saved_bytes,
+                                         void *d_twiddle4, void *d_twiddle2, void *d_input,
+                                         void *workspace, size_t workspace_bytes, void *stream);
 
 /* bf_butterfly_multiply_bw for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): same operands and results,

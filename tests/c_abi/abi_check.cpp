@@ -233,6 +233,24 @@ int main()
     const int rc = bf_butterfly_multiply_fw(&bad, nullptr, nullptr, nullptr, nullptr, 0, nullptr);
     std::printf("output_size > n: rc %d (%s)\n", rc, bf_last_error());
     if (rc != BF_ERR_INVALID) ++failures;
+    // ... and its size queries say "invalid", which is not the same as "no workspace needed"
+    const size_t bad_ws = bf_butterfly_multiply_bw_workspace_bytes(&bad);
+    const bf_problem small = problem(BF_F32, 1, 4, 1, 3, 1, 8, 8);
+    const size_t small_ws = bf_butterfly_multiply_fw_workspace_bytes(&small);
+    std::printf("size queries: invalid problem %s, single-launch forward %zu bytes\n",
+                bad_ws == BF_SIZE_INVALID ? "BF_SIZE_INVALID" : "a size", small_ws);
+    if (bad_ws != BF_SIZE_INVALID || small_ws != 0) ++failures;
+    // the activation-keeping pair: the backward checks the size of the area it is handed
+    {
+        const bf_problem q = problem(BF_F32, 1, 8, 1, 12, 2, 4096, 4096);
+        const size_t keep = bf_butterfly_multiply_saved_bytes(&q);
+        const size_t ws_bytes = bf_butterfly_multiply_bw_saved_workspace_bytes(&q, 0);
+        DeviceBuffer area(keep), ws(ws_bytes), t((size_t)2 * 12 * 2048 * 4 * 4), v((size_t)8 * 4096 * 4);
+        const int short_rc = bf_butterfly_multiply_bw_saved(&q, t.p, v.p, v.p, area.p, keep / 2, nullptr, nullptr, t.p, v.p,
+                                                            nullptr, ws.p, ws_bytes, nullptr);
+        std::printf("saved area too small: rc %d (%s)\n", short_rc, bf_last_error());
+        if (keep == 0 || keep == BF_SIZE_INVALID || short_rc != BF_ERR_WORKSPACE) ++failures;
+    }
     std::printf(failures ? "%d case(s) FAILED\n" : "all cases ok\n", failures);
     return failures ? 1 : 0;
 }

@@ -1,5 +1,6 @@
 """Parity of the HIP library (through its C ABI and through the registered operators)
 against the CPU oracle.  Tolerances are max|err| / max|ref|: 1e-5 forward, 1e-4 gradients."""
+import ctypes
 import sys
 
 import numpy as np
@@ -1181,3 +1182,49 @@ def test_two_streams_with_their_own_workspaces():
             assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
             assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
             assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
+def test_backward_checks_the_size_of_the_saved_area():
+    """bf_butterfly_multiply_bw_saved is told how large the area behind `saved` is and refuses one
+    that is smaller than the planes its own plan reads."""
+    from butterfly_amd import _capi
+    rng = np.random.default_rng(7400)
+    tw, x, g = make_case(rng, np.float32, 20, 1, 12, 2)
+    with pytest.raises(_capi.ButterflyError) as info:
+        _capi.multiply_fw_bw_saving(dev(tw), dev(x), dev(g), True, saved_given=4096)
+    assert info.value.code == _capi.BF_ERR_WORKSPACE
+    torch.cuda.synchronize()
+
+
+def test_autograd_backward_with_a_gradient_whose_plan_keeps_nothing():
+    """The forward keeps activations for the backward plan it expects; a gradient that arrives as a
+    view with a huge batch stride makes the backward plan differently (rows out of reach of 32-bit
+    offsets -> the fallback kernels, which read no kept activations).  The operator then recomputes
+    instead of failing."""
+    import butterfly_amd  # noqa: F401
+    ops = torch.ops.torch_butterfly
+    rng = np.random.default_rng(7401)
+    B, L, nb = 6, 11, 1
+    n = 1 << L
+    tw, x, g = make_case(rng, np.float32, B, 1, L, nb)
+    twd, xd = dev(tw).requires_grad_(), dev(x).requires_grad_()
+    y = ops.butterfly_multiply(twd, xd, True, None)
+    # rows of the gradient 2^27 elements (512 MiB) apart: a view into a 3 GiB buffer
+    stride = 1 << 27
+    big = torch.empty(B * stride, dtype=torch.float32, device="cuda")
+    gview = torch.as_strided(big, (B, 1, n), (stride, n, 1))
+    gview.copy_(dev(g))
+    say("autograd with strided gradient", gview.stride())
+    # the premise: with these strides the backward keeps nothing, with dense ones it does
+    from butterfly_amd import _capi
+    p = _capi.make_problem(xd.detach(), L, nb, True, n)
+    p.output_stride = _capi._strides(gview)
+    p.d_input_stride = _capi._strides(xd.detach())
+    assert _capi.lib().bf_butterfly_multiply_saved_bytes(ctypes.byref(p)) == 0
+    p.output_stride = _capi._strides(dev(g))
+    assert _capi.lib().bf_butterfly_multiply_saved_bytes(ctypes.byref(p)) > 0
+    dtw, dx = torch.autograd.grad(y, (twd, xd), gview)
+    torch.cuda.synchronize()
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, True)
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL

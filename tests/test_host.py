@@ -51,7 +51,25 @@ def test_c_abi_rejects_bad_problems_on_the_host():
     # workspace query is pure host arithmetic
     p.input_stride[2] = 1
     p.batch, p.log_n, p.nblocks = 16384, 10, 2
-    assert L.bf_butterfly_multiply_bw_workspace_bytes(ctypes.byref(p)) > 0
+    assert 0 < L.bf_butterfly_multiply_bw_workspace_bytes(ctypes.byref(p)) < _capi.SIZE_INVALID
+    # ... and tells "no workspace needed" (0) from "not a valid problem" (BF_SIZE_INVALID)
+    p.input_size = p.output_size = 1024
+    for name in ("d_input_stride", "output_stride", "input_stride"):
+        getattr(p, name)[0], getattr(p, name)[1], getattr(p, name)[2] = 1024, 1024, 1
+    assert L.bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p)) == 0
+    assert L.bf_butterfly_multiply_saved_bytes(ctypes.byref(p)) == 0
+    p.output_size = 1025
+    queries = [L.bf_butterfly_multiply_fw_workspace_bytes, L.bf_butterfly_multiply_bw_workspace_bytes,
+               L.bf_butterfly_multiply_saved_bytes, L.bf_butterfly_multiply_base4_fw_workspace_bytes,
+               L.bf_butterfly_multiply_base4_bw_workspace_bytes, L.bf_butterfly_multiply_base4_saved_bytes,
+               L.bf_butterfly_multiply_bias_bw_workspace_bytes, L.bf_butterfly_bias_grad_workspace_bytes,
+               L.bf_butterfly_multiply_base4_bw_saved_workspace_bytes]
+    for q in queries:
+        assert q(ctypes.byref(p)) == _capi.SIZE_INVALID, q.__name__
+        assert b"output_size" in L.bf_last_error()
+    assert L.bf_butterfly_multiply_bw_saved_workspace_bytes(ctypes.byref(p), 0) == _capi.SIZE_INVALID
+    with pytest.raises(_capi.ButterflyError):
+        _capi._size(L.bf_butterfly_multiply_fw_workspace_bytes(ctypes.byref(p)))
 
 
 def test_operator_schemas_and_host_side_checks():

@@ -39,8 +39,21 @@ def run_pair(tw, x, g, inc):
     dx = torch.full(xd.shape, float("nan"), dtype=xd.dtype, device=xd.device)
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    # PyTorch's statistics see its own allocator only; the device's free memory also sees a
+    # hipMalloc made inside the library
+    # (one call first: the runtime loads a kernel's code on its first launch, which is not the
+    # library allocating)
     _capi.multiply_bw_noalloc(twd, xd, gd, inc, dtw, dx)
+    torch.cuda.synchronize()
+    dtw.fill_(float("nan"))
+    dx.fill_(float("nan"))
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info()[0]
+    _capi.multiply_bw_noalloc(twd, xd, gd, inc, dtw, dx)
+    torch.cuda.synchronize()
     assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     ref_dtw, ref_dx = _capi.multiply_bw(twd, xd, gd, inc)
     torch.cuda.synchronize()
     assert torch.equal(dtw, ref_dtw) and torch.equal(dx, ref_dx)
