@@ -1438,13 +1438,23 @@ __global__ __launch_bounds__(kFastThreads) void fast_bw_kernel(FastBwArgs a)
         iteration(std::integral_constant<int, 0>{}, masked, it, vF, gv, carry, actP, actQ);
         iteration(std::integral_constant<int, 1>{}, masked, it + 1, vF, gv, carry, actQ, actP);
         // iterations it, it + 1 are FULL when the furthest group they request exists in every slot
-        for (it = 1; it < nit && (R * (it + 2 + AHEAD) + R) * SLOTS <= rows_valid; it += 2) {
+        // An odd iteration left over at the end runs on its own where the kernel has the registers
+        // for a third copy of the body (whole rows of 1024); the others start one more pair, whose
+        // second half finds no rows.
+        constexpr int ODD_TAIL = SLOTS == 1 ? 1 : 0;
+        for (it = 1; it + ODD_TAIL < nit && (R * (it + 2 + AHEAD) + R) * SLOTS <= rows_valid; it += 2) {
             iteration(std::integral_constant<int, 0>{}, unmasked, it, vF, gv, carry, actP, actQ);
             iteration(std::integral_constant<int, 1>{}, unmasked, it + 1, vF, gv, carry, actQ, actP);
         }
-        for (; it < nit; it += 2) {
+        for (; it + ODD_TAIL < nit; it += 2) {
             iteration(std::integral_constant<int, 0>{}, masked, it, vF, gv, carry, actP, actQ);
             iteration(std::integral_constant<int, 1>{}, masked, it + 1, vF, gv, carry, actQ, actP);
+        }
+        if constexpr (ODD_TAIL != 0) {
+            if (it < nit) {
+                iteration(std::integral_constant<int, 0>{}, masked, it, vF, gv, carry, actP, actQ);
+                ++it;
+            }
         }
         wait_rows_in_lds<0>();  // requests past the last group (they fetch nothing)
         flush_it = it - 1;   // the last iteration that ran (it may lie past the last group)

@@ -1228,3 +1228,26 @@ def test_autograd_backward_with_a_gradient_whose_plan_keeps_nothing():
     dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, True)
     assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
     assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
+@pytest.mark.parametrize("B", [1, 7, 64, 300, 1100])
+def test_small_batches_of_the_inference_shapes(B):
+    """The batch sizes of the reference's inference benchmarks (/root/reference/butterfly/benchmark_linear.py,
+    torch_butterfly/input_padding_benchmark.py): 1024-wide rows with one and two blocks and the
+    4096-wide two-block Linear drop-in, complex 1024.  At these sizes the backward call runs on
+    fewer workgroups than compute units (fewer partial slices to write and reduce), so the row
+    loops of its workgroups get longer than the batch alone would make them."""
+    from butterfly_amd import _capi
+    rng = np.random.default_rng(7500 + B)
+    for dtype, L, nb, inc in [(np.float32, 10, 1, True), (np.float32, 10, 2, False), (np.float32, 12, 2, True),
+                              (np.complex64, 10, 1, True), (np.float32, 7, 2, True)]:
+        say("small batch", B, np.dtype(dtype).name, L, nb, inc)
+        tw, x, g = make_case(rng, dtype, B, 1, L, nb)
+        y_ref = oracle.butterfly_fw(tw, x, inc)
+        dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+        y = _capi.multiply_fw(dev(tw), dev(x), inc)
+        dtw, dx = _capi.multiply_bw(dev(tw), dev(x), dev(g), inc)
+        torch.cuda.synchronize()
+        assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
+        assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+        assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
