@@ -188,6 +188,19 @@ def test_wavelet_haar_against_the_direct_recursion():
     assert close(special.wavelet_haar(n)(x), want, 1e-4)
 
 
+def test_wavelet_haar_on_the_example_of_the_pywavelets_manual():
+    """Known answer: the PyWavelets manual gives pywt.wavedec([1..8], 'db1', level=2) =
+    [5, 13], [-2, -2], [-0.70710678] * 4 (db1 is the Haar wavelet; approximation first, then
+    details from coarse to fine, a detail being (even - odd) / sqrt(2)).  wavelet_haar decomposes
+    to full depth (reference tests/test_special.py:365-372 compares with pywt.wavedec at its
+    default, maximal level), i.e. one more level on [5, 13]: 18 / sqrt(2), -8 / sqrt(2)."""
+    from butterfly_amd import special
+    x = torch.arange(1.0, 9.0).reshape(1, 8)
+    r = math.sqrt(0.5)
+    want = torch.tensor([[18 * r, -8 * r, -2.0, -2.0, -r, -r, -r, -r]])
+    assert close(special.wavelet_haar(8)(x), want, 1e-5)
+
+
 def test_combine_constructors_as_the_reference_tests_them():
     import butterfly_amd
     from butterfly_amd import combine
