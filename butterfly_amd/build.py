@@ -33,7 +33,9 @@ def _run(cmd):
 
 # Kernels whose row pipelines wait for their LDS-direct row fetches with hand-counted
 # `s_waitcnt vmcnt(N)`: N is right only while the compiler adds no memory operation of its own
-# between request and wait, i.e. while nothing spills to scratch memory.
+# between request and wait, i.e. while nothing spills to scratch memory.  (Scalar registers that the
+# compiler parks in the lanes of a vector register -- "SGPRs Spill" with a scratch size of 0 -- move
+# no memory and are allowed: the forward variants compiled for eight wavefronts per SIMD have a few.)
 GATED_KERNELS = ("fast_fw_kernel", "fast_bw_kernel", "wide_fw_kernel", "fast4_fw_kernel", "fast4_bw_kernel",
                  "fast4g_fw_kernel", "fast4g_bw_kernel")
 RESOURCES = os.path.join(PKG, "kernel_resources.txt")
@@ -61,7 +63,7 @@ def check_kernel_resources(path=RESOURCES):
         kernels = parse_kernel_resources(f.read())
     gated = {k: v for k, v in kernels.items() if any(g in k for g in GATED_KERNELS)}
     bad = [k for k, v in gated.items()
-           if v.get("ScratchSize", 1) != 0 or v.get("VGPRs Spill", 1) != 0 or v.get("SGPRs Spill", 1) != 0]
+           if v.get("ScratchSize", 1) != 0 or v.get("VGPRs Spill", 1) != 0 or "SGPRs Spill" not in v]
     return bad, len(gated)
 
 
@@ -83,7 +85,7 @@ def build_hip():
         raise RuntimeError("no resource-usage remarks for the register-resident kernels: cannot check for spills")
     if bad:
         raise RuntimeError("kernels with hand-counted memory waits use scratch memory or spill: " + ", ".join(bad))
-    print(f"{seen} register-resident kernels: no scratch memory, no spills", flush=True)
+    print(f"{seen} register-resident kernels: no scratch memory, no vector-register spills", flush=True)
     return LIB_HIP
 
 

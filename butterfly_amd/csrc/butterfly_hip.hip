@@ -179,11 +179,12 @@ int num_cu()
 #ifndef BF_FAST_FW_ROWS
 #define BF_FAST_FW_ROWS 4
 #endif
-#ifndef BF_FAST_FW_WGS
-#define BF_FAST_FW_WGS 1
-#endif
 constexpr int kFastFwRows = BF_FAST_FW_ROWS;  // row groups in flight per forward workgroup
-constexpr int kFastFwWgPerCu = BF_FAST_FW_WGS;  // forward workgroups resident per compute unit
+// Iterations (of kFastFwRows row groups) a forward workgroup must have left before a float pass
+// over two blocks is spread over two workgroups per compute unit (see fw_wg_per_cu).
+#ifndef BF_FAST_FW_PAIR_MIN_ITERS
+#define BF_FAST_FW_PAIR_MIN_ITERS 6
+#endif
 constexpr int kFastFwRowsComplex = 2;       // complex64: half as many (LDS and registers double)
 
 // ---- register-resident multi-pass path (float and complex64, base-2, n <= 2^24) -------------------------
@@ -239,6 +240,25 @@ int64_t pass_lanes(const bf_problem *p, const Pass &q)
     if (q.wide) return 1;
     const int reach = q.span ? 10 : q.L;
     return (int64_t)1 << (p->log_n > reach ? p->log_n - reach : 0);
+}
+
+// Forward workgroups per compute unit.  The kernel fits a CU twice (64 registers, 64 KiB of LDS).
+// A float pass over two blocks is bound by its own chain of arithmetic and LDS transpositions,
+// not by memory, and two resident workgroups fill each other's gaps (33.3 against 36.2 us at
+// 16384 rows of 1024); each of them loads the whole factor set, so it takes rows to pay off
+// (2048 rows: 10.0 against 8.6 us for one block).  One-block passes run at the memory rate either way.
+// (The 64-register variant of the two-block forward kernel for 512-element rows, decreasing
+// stride first, does not fit its registers -- the build refuses kernels that spill -- so that
+// plan always runs one workgroup per CU.)
+constexpr bool fw_pairable(int L, bool inc) { return !(L == 9 && !inc); }
+
+int fw_wg_per_cu(const bf_problem *p, const Pass &q)
+{
+    if (q.wide || q.span || q.NB != 2 || p->dtype != BF_F32 || !fw_pairable(q.L, q.inc)) return 1;
+    const int64_t slots = 1024 >> q.L;
+    const int64_t iters = ((p->batch + slots - 1) / slots + kFastFwRows - 1) / kFastFwRows;
+    const int64_t pairs = std::max<int64_t>(1, 2 * (int64_t)num_cu() / (p->nstacks * pass_lanes(p, q)));
+    return iters >= pairs * BF_FAST_FW_PAIR_MIN_ITERS ? 2 : 1;
 }
 
 int stage_bit(const bf_problem *p, int t)
@@ -443,7 +463,7 @@ bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
         const Pass &q = pl.pass[k];
         const FastGrid g = q.wide ? wide_grid(p->batch, p->nstacks)
                                   : fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), backward ? 1 : fw_rows(p),
-                                              backward ? 1 : kFastFwWgPerCu, cap, backward);
+                                              backward ? 1 : fw_wg_per_cu(p, q), cap, backward);
         rows = std::max(rows, (g.groups_per_wg + kFastFwRows + 2) * g.slots);
     }
     const int64_t dense[3] = {p->nstacks * n, n, 1};
@@ -454,12 +474,19 @@ bool passes_addressable(const bf_problem *p, const PassPlan &pl, bool backward)
     return true;
 }
 
+// paired: the grid holds two workgroups per compute unit (fw_wg_per_cu)
 template <int L, int NB, bool INC>
-void launch_fast_fw_t(bool cplx, const FastFwArgs &a, dim3 grid, hipStream_t stream)
+void launch_fast_fw_t(bool cplx, bool paired, const FastFwArgs &a, dim3 grid, hipStream_t stream)
 {
     if constexpr (NB == 1) {
         if (cplx) {
             hipLaunchKernelGGL((fast_fw_kernel<float2, FastPlan<L, NB, INC>, kFastFwRowsComplex>), grid, dim3(kFastThreads), 0,
+                               stream, a);
+            return;
+        }
+    } else if constexpr (fw_pairable(L, INC)) {
+        if (paired) {
+            hipLaunchKernelGGL((fast_fw_kernel<float, FastPlan<L, NB, INC>, kFastFwRows, 8>), grid, dim3(kFastThreads), 0,
                                stream, a);
             return;
         }
@@ -615,8 +642,8 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
 #endif
             BF_HIP_CHECK(hipGetLastError());
         } else {
-            const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), fw_rows(p), kFastFwWgPerCu,
-                                         row_cap(p, false));
+            const int per_cu = fw_wg_per_cu(p, q);
+            const FastGrid g = fast_grid(p->batch, q.L, p->nstacks * pass_lanes(p, q), fw_rows(p), per_cu, row_cap(p, false));
             FastFwArgs a = {};
             a.tw = tw;
             a.tw_stack_stride = p->nblocks * p->log_n * (n / 2) * 4;
@@ -639,7 +666,7 @@ int multipass_forward(const bf_problem *p, const PassPlan &pl, const void *tw, c
                 const int rc = launch_span(p->dtype == BF_C64, q, false, false, &a, nullptr, grid, stream);
                 if (rc) return rc;
             } else {
-                BF_FAST_DISPATCH(launch_fast_fw_t, q, p->dtype == BF_C64, a, grid, stream);
+                BF_FAST_DISPATCH(launch_fast_fw_t, q, p->dtype == BF_C64, per_cu == 2, a, grid, stream);
             }
             BF_HIP_CHECK(hipGetLastError());
         }

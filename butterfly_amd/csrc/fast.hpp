@@ -667,36 +667,45 @@ constexpr int bw_operations_behind_awaited_rows()
     return -1;
 }
 
-// Forward kernel: the rows of the next iteration are requested during the previous one (request
-// r in phase r mod (TT + 1), phase p behind barrier p); behind them come that iteration's R
-// stores and the waiting iteration's requests of the phases in front of its last barrier.
+// Forward kernel: the rows of the next iteration are requested during the previous one, behind
+// its barriers (request r behind barrier 1 + r mod TT; all at the top of the iteration when there
+// is no barrier); behind the last of them come that iteration's R stores and the waiting
+// iteration's requests of the phases in front of its last barrier.
 template <int R, int TT>
 constexpr int fw_operations_behind_awaited_rows()
 {
-    int younger = R;
-    for (int phase = 0; phase < (TT == 0 ? 1 : TT); ++phase)
-        for (int r = 0; r < R; ++r) younger += r % (TT + 1) == phase ? 1 : 0;
+    int younger = R;                                       // the stores closing the previous iteration
+    if (TT == 0) return younger + R;                       // the waiting iteration's own requests, at its top
+    for (int barrier = 1; barrier < TT; ++barrier)         // the wait stands in front of barrier TT
+        for (int r = 0; r < R; ++r) younger += 1 + r % TT == barrier ? 1 : 0;
     return younger;
 }
 
-#ifndef BF_FAST_FW_WAVES
-#define BF_FAST_FW_WAVES 4
-#endif
 // P: FastPlan<L, NB, INC> (whole blocks of a row or chunk) or SpanPlan<H, MODE> (a span of high
 // bits of a long row; gridDim.z = n / 1024 tiles).
-template <typename T, typename P, int R>
-__global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel(FastFwArgs a)
+// WAVES: wavefronts per SIMD the kernel is compiled for.  8 keeps it within 64 registers, so that
+// two workgroups fit a compute unit (see TWO_SETS for the LDS side); the host asks for that where
+// two resident workgroups pay off.
+template <typename T, typename P, int R, int WAVES = 4>
+__global__ __launch_bounds__(kFastThreads, WAVES) void fast_fw_kernel(FastFwArgs a)
 {
     constexpr int L = P::LOG;
     constexpr int n = 1 << L, NS = P::NS, SLOTS = P::SLOTS;
     constexpr int EB = (int)sizeof(T);
-    // float rows are fetched straight into LDS, two iterations (2 R row groups) ahead, and the
-    // walk starts in the layout of its first stage; complex64 rows arrive in registers, layout A
+    // float rows are fetched straight into LDS, up to two iterations (2 R row groups) ahead, and
+    // the walk starts in the layout of its first stage; complex64 rows arrive in registers, layout A
     constexpr bool DIRECT = sizeof(T) == 4;
     constexpr int SF = DIRECT ? P::layout(0) : 0;
     constexpr int TT = P::fw_transposes_total(SF);  // barriers per iteration
     __shared__ __align__(16) T lds[TT > 0 ? 2 * R * kFastRowWords : 1];
-    __shared__ float lds_rows[DIRECT ? 4 * R * kFastRowWords : 1];  // four sets of R row slots
+    // Row slots in LDS.  A set is only read at the top of its iteration, so with a barrier in the
+    // iteration (TT >= 1) the requests for the iteration after next can refill it as soon as the
+    // first barrier has passed: two sets (64 KiB with the transpose buffers at R = 4, which lets two
+    // workgroups share a compute unit).  Without a barrier a set stays untouched for a whole
+    // iteration after its reads: four sets, requests at the top.
+    constexpr bool TWO_SETS = TT >= 1;
+    constexpr int SETS = TWO_SETS ? 2 : 4;
+    __shared__ float lds_rows[DIRECT ? SETS * R * kFastRowWords : 1];
     const int t = threadIdx.x;
     const int stack = blockIdx.y;
     const int chunk = blockIdx.z;
@@ -763,18 +772,19 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
             v[r] = buf_load<T>(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
         }
     };
-    // The requests of an iteration are spread over its TT + 1 phases (row r goes out at the
-    // start of phase r mod (TT + 1)): sixteen wavefronts asking for R rows each at the same
+    // The requests of an iteration are spread over the phases behind its barriers (row r goes
+    // out behind barrier 1 + r mod TT): sixteen wavefronts asking for R rows each at the same
     // moment, right behind the previous iteration's stores, queue up at the memory pipeline.
+    // PHASE 0 is the top of the iteration: only a kernel without barriers requests there.
     auto fetch_phase = [&](int grel, int set, auto PHASE, bool full) {
         static_for<0, R>([&](auto RR) {
-            if constexpr (RR % (TT + 1) == decltype(PHASE)::value) fetch_row(grel, set, RR, full);
+            if constexpr ((TWO_SETS ? 1 + RR % (TT > 0 ? TT : 1) : 0) == decltype(PHASE)::value) fetch_row(grel, set, RR, full);
         });
     };
     // requests of an iteration that go out before its last barrier (all of them when there is none)
     constexpr int EARLY = [] {
         int c = 0;
-        for (int r = 0; r < R; ++r) c += (TT == 0 || r % (TT + 1) < TT) ? 1 : 0;
+        for (int r = 0; r < R; ++r) c += (TT == 0 || 1 + r % (TT > 0 ? TT : 1) < TT) ? 1 : 0;
         return c;
     }();
     // Before the last barrier of an iteration each wavefront waits for the rows of the next
@@ -802,9 +812,14 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
     auto iteration = [&](int grel, auto FULL) {
         constexpr bool full = decltype(FULL)::value;
         T v[R];
+        // Transposes alternate between the two halves of `lds` across iteration boundaries too
+        // (an odd number per iteration flips the start): a wavefront writes a half again only
+        // behind the barrier of the transpose in between, which every wavefront reaches after
+        // its read of that half.
+        const int flip = (TT & 1) ? (grel / R) & 1 : 0;
         if constexpr (DIRECT) {
-            const int set = (grel / R) & 3;
-            fetch_phase(grel + 2 * R, (set + 2) & 3, std::integral_constant<int, 0>{}, full);
+            const int set = (grel / R) & (SETS - 1);
+            fetch_phase(grel + 2 * R, (set + 2) & (SETS - 1), std::integral_constant<int, 0>{}, full);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const float x = lds_rows[(set * R + r) * kFastRowWords + (SF ? c.fB : c.fA)];
@@ -822,21 +837,21 @@ __global__ __launch_bounds__(kFastThreads, BF_FAST_FW_WAVES) void fast_fw_kernel
             if constexpr (P::layout(s) != P::layout_before(s, SF)) {
                 constexpr int nth = P::fw_transposes_before(s, SF);  // transposes done so far
                 constexpr int to_b = P::layout(s);
-                T *buf = lds + (nth & 1) * R * kFastRowWords;
+                T *buf = lds + ((nth + flip) & 1) * R * kFastRowWords;
                 const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
                 transpose_rows<T, R, DIRECT && nth + 1 == TT, YOUNGER>(buf, wr, rd, v);
                 if constexpr (DIRECT)
-                    fetch_phase(grel + 2 * R, (((grel / R) & 3) + 2) & 3, std::integral_constant<int, nth + 1>{}, full);
+                    fetch_phase(grel + 2 * R, ((grel / R) + 2) & (SETS - 1), std::integral_constant<int, nth + 1>{}, full);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) v[r] = fw_product<K>(v[r], ta[s], tb[s], c.bperm_addr);
         });
         if constexpr (P::layout(NS - 1) != 0) {
             constexpr int nth = P::fw_transposes_before(NS, SF);
-            T *buf = lds + (nth & 1) * R * kFastRowWords;
+            T *buf = lds + ((nth + flip) & 1) * R * kFastRowWords;
             transpose_rows<T, R, DIRECT, YOUNGER>(buf, c.fB, c.fA, v);
             if constexpr (DIRECT)
-                fetch_phase(grel + 2 * R, (((grel / R) & 3) + 2) & 3, std::integral_constant<int, nth + 1>{}, full);
+                fetch_phase(grel + 2 * R, ((grel / R) + 2) & (SETS - 1), std::integral_constant<int, nth + 1>{}, full);
         }
         if constexpr (DIRECT && TT == 0) wait_rows_in_lds<YOUNGER>();
 #pragma unroll

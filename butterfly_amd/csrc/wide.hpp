@@ -166,6 +166,8 @@ __global__ __launch_bounds__(kFastThreads) void wide_fw_kernel(FastFwArgs a)
     }
     for (int row = 0; row < nr; ++row) {
         T v[Q];
+        // (the two halves of `lds` alternate across iteration boundaries too: see fast_fw_kernel)
+        const int flip = (TT & 1) ? row & 1 : 0;
         if constexpr (DIRECT) {
             fetch_row(row + 2);
 #pragma unroll
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(kFastThreads) void wide_fw_kernel(FastFwArgs a)
             if constexpr (P::layout(s) != P::layout_before(s, SF)) {
                 constexpr int nth = P::transposes_before(s, SF);
                 constexpr int to_b = P::layout(s);
-                T *buf = lds + (nth & 1) * Q * kFastRowWords;
+                T *buf = lds + ((nth + flip) & 1) * Q * kFastRowWords;
                 const int wr = to_b ? c.fA : c.fB, rd = to_b ? c.fB : c.fA;
                 transpose_rows<T, Q, DIRECT && nth + 1 == TT, 2 * Q>(buf, wr, rd, v);
             }
@@ -204,7 +206,7 @@ __global__ __launch_bounds__(kFastThreads) void wide_fw_kernel(FastFwArgs a)
         });
         if constexpr (P::layout(NS - 1) != 0) {
             constexpr int nth = P::transposes_before(NS, SF);
-            T *buf = lds + (nth & 1) * Q * kFastRowWords;
+            T *buf = lds + ((nth + flip) & 1) * Q * kFastRowWords;
             transpose_rows<T, Q, DIRECT, 2 * Q>(buf, c.fB, c.fA, v);
         }
 #pragma unroll

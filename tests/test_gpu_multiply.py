@@ -1251,3 +1251,33 @@ def test_small_batches_of_the_inference_shapes(B):
         assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL
         assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
         assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
+@pytest.mark.parametrize("B,S,L,inc,I,O", [(16384, 1, 10, True, None, None), (13001, 1, 10, False, 1000, 700),
+                                           (50000, 2, 8, False, None, None), (100003, 1, 7, True, None, None),
+                                           (30000, 1, 9, True, None, None), (30000, 1, 9, False, None, None),
+                                           (400000, 1, 4, False, None, None)],
+                         ids=lambda v: str(v))
+def test_forward_with_two_workgroups_per_compute_unit(B, S, L, inc, I, O):
+    """Float passes over two blocks put two forward workgroups on every compute unit once each of
+    them has enough rows (the 64-register variant of the kernel, two row sets in LDS): batches
+    beyond that threshold for several row lengths, both stride orders, a ragged last group, padded
+    and trimmed widths; forward and backward against the oracle.  (512-element rows with decreasing
+    stride first stay on one workgroup per unit; they are here for the same sizes.)"""
+    from butterfly_amd import _capi
+    rng = np.random.default_rng(7100 + L + int(inc))
+    tw, x, g = make_case(rng, np.float32, B, S, L, 2, I, O)
+    say("paired forward case", B, S, L, inc, I, O)
+    y_ref = oracle.butterfly_fw(tw, x, inc, O)
+    twd, xd = dev(tw), dev(x)
+    for rep in range(3):   # repeated calls: the row pipeline must not depend on timing
+        y = _capi.multiply_fw(twd, xd, inc, O)
+        torch.cuda.synchronize()
+        assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL, (B, S, L, inc, rep)
+    if B > 17000:      # (the scalar oracle's backward takes seconds per case at these sizes)
+        return
+    dtw_ref, dx_ref = oracle.butterfly_bw(tw, x, g, inc)
+    dtw, dx = _capi.multiply_bw(twd, xd, dev(g), inc)
+    torch.cuda.synchronize()
+    assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
+    assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
