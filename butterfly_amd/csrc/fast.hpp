@@ -667,17 +667,21 @@ constexpr int bw_operations_behind_awaited_rows()
     return -1;
 }
 
-// Forward kernel: the rows of the next iteration are requested during the previous one, behind
-// its barriers (request r behind barrier 1 + r mod TT; all at the top of the iteration when there
-// is no barrier); behind the last of them come that iteration's R stores and the waiting
+// Forward kernel: the rows of the next iteration are requested during the previous one (request
+// r in phase r mod (TT + 1), phase p behind barrier p; TWO_SETS: behind barrier 1 + r mod TT,
+// none at the top); behind the last of them come that iteration's R stores and the waiting
 // iteration's requests of the phases in front of its last barrier.
-template <int R, int TT>
+template <int R, int TT, bool TWO_SETS>
 constexpr int fw_operations_behind_awaited_rows()
 {
     int younger = R;                                       // the stores closing the previous iteration
-    if (TT == 0) return younger + R;                       // the waiting iteration's own requests, at its top
-    for (int barrier = 1; barrier < TT; ++barrier)         // the wait stands in front of barrier TT
-        for (int r = 0; r < R; ++r) younger += 1 + r % TT == barrier ? 1 : 0;
+    // the waiting iteration's own requests up to the wait, which stands in front of barrier TT
+    // (in front of the stores when there is no barrier)
+    for (int phase = 0; phase < (TT == 0 ? 1 : TT); ++phase)
+        for (int r = 0; r < R; ++r) {
+            const int at = TWO_SETS ? 1 + r % (TT > 0 ? TT : 1) : r % (TT + 1);
+            younger += at == phase ? 1 : 0;
+        }
     return younger;
 }
 
@@ -698,12 +702,13 @@ __global__ __launch_bounds__(kFastThreads, WAVES) void fast_fw_kernel(FastFwArgs
     constexpr int SF = DIRECT ? P::layout(0) : 0;
     constexpr int TT = P::fw_transposes_total(SF);  // barriers per iteration
     __shared__ __align__(16) T lds[TT > 0 ? 2 * R * kFastRowWords : 1];
-    // Row slots in LDS.  A set is only read at the top of its iteration, so with a barrier in the
-    // iteration (TT >= 1) the requests for the iteration after next can refill it as soon as the
-    // first barrier has passed: two sets (64 KiB with the transpose buffers at R = 4, which lets two
-    // workgroups share a compute unit).  Without a barrier a set stays untouched for a whole
-    // iteration after its reads: four sets, requests at the top.
-    constexpr bool TWO_SETS = TT >= 1;
+    // Row slots in LDS: four sets of R, an iteration's requests starting at its top, two
+    // iterations ahead.  The variant compiled for two workgroups per compute unit has room for two
+    // sets only (64 KiB with the transpose buffers at R = 4): a set is read at the top of its
+    // iteration and nowhere else, so the requests for the iteration after next refill it as soon as
+    // the first barrier has passed.  (One workgroup per unit keeps the longer lead: a memory-bound
+    // pass over one block is 6 % slower with two sets.)
+    constexpr bool TWO_SETS = TT >= 1 && WAVES >= 8;
     constexpr int SETS = TWO_SETS ? 2 : 4;
     __shared__ float lds_rows[DIRECT ? SETS * R * kFastRowWords : 1];
     const int t = threadIdx.x;
@@ -772,26 +777,27 @@ __global__ __launch_bounds__(kFastThreads, WAVES) void fast_fw_kernel(FastFwArgs
             v[r] = buf_load<T>(in_rs, ok ? in_thr : kOob, (grel + r) * SLOTS * in_row);
         }
     };
-    // The requests of an iteration are spread over the phases behind its barriers (row r goes
-    // out behind barrier 1 + r mod TT): sixteen wavefronts asking for R rows each at the same
-    // moment, right behind the previous iteration's stores, queue up at the memory pipeline.
-    // PHASE 0 is the top of the iteration: only a kernel without barriers requests there.
+    // The requests of an iteration are spread over its phases (phase 0: the top, phase p: behind
+    // barrier p; row r goes out in phase r mod (TT + 1), with TWO_SETS in phase 1 + r mod TT):
+    // sixteen wavefronts asking for R rows each at the same moment, right behind the previous
+    // iteration's stores, queue up at the memory pipeline.
+    constexpr auto phase_of = [](int r) { return TWO_SETS ? 1 + r % (TT > 0 ? TT : 1) : r % (TT + 1); };
     auto fetch_phase = [&](int grel, int set, auto PHASE, bool full) {
         static_for<0, R>([&](auto RR) {
-            if constexpr ((TWO_SETS ? 1 + RR % (TT > 0 ? TT : 1) : 0) == decltype(PHASE)::value) fetch_row(grel, set, RR, full);
+            if constexpr (phase_of(RR) == decltype(PHASE)::value) fetch_row(grel, set, RR, full);
         });
     };
     // requests of an iteration that go out before its last barrier (all of them when there is none)
-    constexpr int EARLY = [] {
+    constexpr int EARLY = [phase_of] {
         int c = 0;
-        for (int r = 0; r < R; ++r) c += (TT == 0 || 1 + r % (TT > 0 ? TT : 1) < TT) ? 1 : 0;
+        for (int r = 0; r < R; ++r) c += (TT == 0 || phase_of(r) < TT) ? 1 : 0;
         return c;
     }();
     // Before the last barrier of an iteration each wavefront waits for the rows of the next
     // iteration, requested during the previous one.  Younger than those: the previous
     // iteration's R stores and this iteration's EARLY requests.
     constexpr int YOUNGER = R + EARLY;
-    static_assert(!DIRECT || YOUNGER == fw_operations_behind_awaited_rows<R, TT>(), "wait count of the row fetch");
+    static_assert(!DIRECT || YOUNGER == fw_operations_behind_awaited_rows<R, TT, TWO_SETS>(), "wait count of the row fetch");
 
     T nxt[R];
     if constexpr (DIRECT) {
