@@ -794,6 +794,20 @@ Fast4GArgs fast4g_block_args(const bf_problem *p, const void *tw4, const void *t
     return a;
 }
 
+// Forward workgroups per compute unit of the aligned float kernels (fast4.hpp).  They fit a CU
+// twice as they are (at most 51 registers, 33 KiB of LDS), and where a block crosses between the
+// layouts (n >= 256: LDS transposes, barriers) two resident workgroups fill each other's gaps once
+// each has a few iterations: 23.0 against 25.9 us at 16384 x 4 rows of 256, 24.3 against 27.5 at
+// 16384 rows of 1024; rows of 64 stay within a wavefront and gain nothing.
+int fast4_fw_wg_per_cu(const bf_problem *p)
+{
+    if (fast4_general(p) || p->log_n < 8) return 1;
+    const int64_t slots = 1024 >> p->log_n;
+    const int64_t iters = ((p->batch + slots - 1) / slots + kFast4FwRows - 1) / kFast4FwRows;
+    const int64_t pairs = std::max<int64_t>(1, 2 * (int64_t)num_cu() / p->nstacks);
+    return iters >= pairs * BF_FAST_FW_PAIR_MIN_ITERS ? 2 : 1;
+}
+
 // forward of blocks [first, last) through the base-4 kernels; `scratch` as in multipass_forward
 int fast4_forward(const bf_problem *p, const void *tw4, const void *tw2, const void *input, void *output,
                   void *scratch, const View &in_view, const View &out_view, int first, int last, hipStream_t stream)
@@ -801,7 +815,7 @@ int fast4_forward(const bf_problem *p, const void *tw4, const void *tw2, const v
     const int64_t n = (int64_t)1 << p->log_n;
     const int L = (int)p->log_n;
     const View dense = dense_view(p->nstacks, n);
-    const FastGrid g = fast_grid(p->batch, L, p->nstacks, fast4_fw_rows(p), 1);
+    const FastGrid g = fast_grid(p->batch, L, p->nstacks, fast4_fw_rows(p), fast4_fw_wg_per_cu(p));
     if (fast4_general(p)) {
         for (int k = first; k < last; ++k) {
             Fast4GArgs a = fast4g_block_args(p, tw4, tw2, k);

@@ -1281,3 +1281,27 @@ def test_forward_with_two_workgroups_per_compute_unit(B, S, L, inc, I, O):
     torch.cuda.synchronize()
     assert rel_err(dx.cpu().numpy(), dx_ref) < BW_TOL
     assert rel_err(dtw.cpu().numpy(), dtw_ref) < BW_TOL
+
+
+@pytest.mark.parametrize("B,S,L,nb,inc,I,O", [(16384, 1, 10, 1, True, None, None), (70001, 1, 8, 2, False, 250, 200),
+                                              (13000, 1, 10, 2, False, None, None), (40000, 3, 8, 1, True, None, None)],
+                         ids=lambda v: str(v))
+def test_base4_forward_with_two_workgroups_per_compute_unit(B, S, L, nb, inc, I, O):
+    """The aligned base-4 forward kernels run two workgroups per compute unit for rows of 256 and
+    1024 once each workgroup has enough rows: batches beyond that threshold, both stride orders,
+    a ragged last group, padded and trimmed widths, against the oracle; calls repeated."""
+    from butterfly_amd import _capi
+    n = 1 << L
+    I = n if I is None else I
+    O = n if O is None else O
+    rng = np.random.default_rng(7300 + L + nb)
+    say("paired base-4 forward case", B, S, L, nb, inc, I, O)
+    tw4 = (randn(rng, (S, nb, L // 2, n // 4, 4, 4), np.float32) / 2).astype(np.float32)
+    tw2 = np.zeros((S, nb, 0, n // 2, 2, 2), np.float32)
+    x = randn(rng, (B, S, I), np.float32)
+    y_ref = oracle.butterfly_base4_fw(tw4, tw2, x, inc, O)
+    t4, t2, xd = dev(tw4), dev(tw2), dev(x)
+    for rep in range(3):
+        y = _capi.multiply_base4_fw(t4, t2, xd, inc, O)
+        torch.cuda.synchronize()
+        assert rel_err(y.cpu().numpy(), y_ref) < FW_TOL, (B, S, L, nb, inc, rep)
